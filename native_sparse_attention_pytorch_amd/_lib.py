@@ -1,0 +1,53 @@
+"""ctypes binding of libnsa_hip.so (declarations: include/nsa_hip.h).  There is no fallback:
+if the library is missing or a call fails, a RuntimeError is raised."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libnsa_hip.so")
+
+_lib = None
+
+
+class SelectDesc(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("kv_heads", C.c_int32), ("group", C.c_int32), ("seq", C.c_int32),
+        ("num_sel", C.c_int32), ("block", C.c_int32), ("dim_head", C.c_int32), ("causal", C.c_int32),
+        ("idx_is_int64", C.c_int32), ("scale", C.c_float),
+        ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3), ("o_stride", C.c_int64 * 3),
+    ]
+
+
+_ERR = {-1: "invalid argument", -2: "shape not supported by the compiled kernels", -3: "workspace too small"}
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m native_sparse_attention_pytorch_amd.build` "
+                "(hipcc, gfx950).  There is no non-HIP fallback.")
+        L = C.CDLL(LIB_PATH)
+        vp, sz = C.c_void_p, C.c_size_t
+        L.nsa_abi_version.restype = C.c_int
+        L.nsa_select_workspace_bytes.argtypes = [C.POINTER(SelectDesc), C.POINTER(sz), C.POINTER(sz), C.POINTER(sz)]
+        L.nsa_select_build_index.argtypes = [C.POINTER(SelectDesc), vp, vp, vp, sz, vp]
+        L.nsa_select_fwd.argtypes = [C.POINTER(SelectDesc), vp, vp, vp, vp, vp, vp, vp, sz, vp, vp, vp]
+        L.nsa_select_bwd.argtypes = [C.POINTER(SelectDesc)] + [vp] * 10 + [sz] + [vp] * 4
+        L.nsa_selftest_mfma.argtypes = [vp] * 6
+        L.nsa_selftest_mfma.restype = C.c_int
+        for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):
+            getattr(L, name).restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def check(rc: int, what: str):
+    if rc == 0:
+        return
+    if rc < 0:
+        raise RuntimeError(f"{what}: {_ERR.get(rc, 'error')} (code {rc})")
+    raise RuntimeError(f"{what}: HIP launch failed with hipError_t {rc}")

@@ -1,0 +1,744 @@
+// Block-selection attention for gfx950, walked KV-block by KV-block.
+//
+// The reference kernel (TRI.py:73-484) is query-centric: every 16-query tile re-gathers the
+// S selected K/V blocks of each of its queries, so a K/V block is fetched once per (query,
+// slot) pair and only the G heads of one query share a fetched key (arithmetic intensity ~G
+// flop/byte).  Here the (query, slot) pairs are first counting-sorted by block (the "inverse
+// index"); one wavefront then keeps a 64-key K/V block resident in registers as MFMA operands
+// and streams through it the queries that selected it, 32 rows (= 32/G pairs x G heads) at a
+// time.  Per pair the kernel moves G*d*2 bytes of Q in and a G*d partial result out instead of
+// 2*B*d*2 bytes of K/V.  Each pair gets its own locally normalised softmax partial; a second,
+// bandwidth-bound kernel merges a query's partials (log-sum-exp merge).  The backward uses the
+// same walk: dK/dV of a block accumulate on chip in the wave that owns the block (no atomics),
+// dQ partials are merged per query like the forward partials.
+//
+// No LDS staging is used for operands: register transposes are done with an MFMA against a
+// constant identity operand (see make_ident in nsa_common.hpp).
+#include "nsa_common.hpp"
+#include "nsa_select_plan.hpp"
+
+namespace nsa {
+
+// ------------------------------------------------------------------------------- index build
+
+constexpr int kCountChunk = 256;   // queries per counting chunk
+
+__device__ __forceinline__ int read_idx(const void* idx, int is64, size_t pos) {
+  if (is64) {
+    long long v = reinterpret_cast<const long long*>(idx)[pos];
+    return (v < 0 || v > 0x7fffffffLL) ? -1 : (int)v;
+  }
+  return reinterpret_cast<const int*>(idx)[pos];
+}
+
+// cnt[bh][chunk][j] = number of live slots of the chunk's queries that name block j
+__global__ __launch_bounds__(256) void sel_count_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, char* iws) {
+  extern __shared__ int hist[];
+  const int c = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
+  for (int j = tid; j < P.W; j += 256) hist[j] = 0;
+  __syncthreads();
+  const int i = c * kCountChunk + tid;
+  if (i < P.n) {
+    const size_t base = ((size_t)bh * P.n + i) * P.S;
+    for (int s = 0; s < P.S; ++s) {
+      if (fmask[base + s]) {
+        const int j = read_idx(idx, P.idx64, base + s);
+        if (j >= 0 && j < P.W) atomicAdd(&hist[j], 1);     // integer LDS counter: order-independent
+      }
+    }
+  }
+  __syncthreads();
+  int* cnt = reinterpret_cast<int*>(iws + P.off_cnt) + ((size_t)bh * P.nch + c) * P.W;
+  for (int j = tid; j < P.W; j += 256) cnt[j] = hist[j];
+}
+
+// exclusive scans: over chunks per block (in place in cnt), over blocks (blk_off), and the two
+// work-unit tables (a unit = up to chunk_f / chunk_kv pairs of one block's virtual list, which
+// is the block's own queries, if causal, followed by the queries that selected it)
+__global__ __launch_bounds__(256) void sel_scan_kernel(const SelPlan P, char* iws) {
+  extern __shared__ int tot[];
+  const int bh = blockIdx.x, tid = threadIdx.x;
+  int* cnt = reinterpret_cast<int*>(iws + P.off_cnt) + (size_t)bh * P.nch * P.W;
+  for (int j = tid; j < P.W; j += 256) {
+    int run = 0;
+    for (int c = 0; c < P.nch; ++c) {
+      const int t = cnt[(size_t)c * P.W + j];
+      cnt[(size_t)c * P.W + j] = run;
+      run += t;
+    }
+    tot[j] = run;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int* blk = reinterpret_cast<int*>(iws + P.off_blk) + (size_t)bh * (P.W + 1);
+    int* uf = reinterpret_cast<int*>(iws + P.off_unitf) + (size_t)bh * (P.W + 1);
+    int* uk = reinterpret_cast<int*>(iws + P.off_unitkv) + (size_t)bh * (P.W + 1);
+    int acc = 0, af = 0, ak = 0;
+    for (int j = 0; j < P.W; ++j) {
+      blk[j] = acc; uf[j] = af; uk[j] = ak;
+      const int own = P.causal ? min(P.B, P.n - j * P.B) : 0;
+      const int L = own + tot[j];
+      acc += tot[j];
+      af += (L + P.chunk_f - 1) / P.chunk_f;
+      ak += (L + P.chunk_kv - 1) / P.chunk_kv;
+    }
+    blk[P.W] = acc; uf[P.W] = af; uk[P.W] = ak;
+  }
+}
+
+// list[bh][blk_off[j] + ...] = query * SP + slot, ordered by (block, counting chunk, query, slot)
+__global__ __launch_bounds__(64) void sel_fill_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, char* iws) {
+  extern __shared__ int base[];
+  const int c = blockIdx.x, bh = blockIdx.y, lane = threadIdx.x;
+  const int* cnt = reinterpret_cast<const int*>(iws + P.off_cnt) + ((size_t)bh * P.nch + c) * P.W;
+  const int* blk = reinterpret_cast<const int*>(iws + P.off_blk) + (size_t)bh * (P.W + 1);
+  int* list = reinterpret_cast<int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
+  for (int j = lane; j < P.W; j += 64) base[j] = blk[j] + cnt[j];
+  __syncthreads();
+  const int q0 = c * kCountChunk;
+  const int nq = min(kCountChunk, P.n - q0);
+  const int total = nq * P.S;
+  for (int e0 = 0; e0 < total; e0 += 64) {
+    const int e = e0 + lane;
+    int j = -1, entry = 0;
+    if (e < total) {
+      const int qi = q0 + e / P.S, s = e % P.S;
+      const size_t pos = ((size_t)bh * P.n + qi) * P.S + s;
+      if (fmask[pos]) {
+        j = read_idx(idx, P.idx64, pos);
+        if (j >= P.W) j = -1;
+        entry = qi * P.SP + s;
+      }
+    }
+    const int key = (j >= 0) ? j : (-1 - lane);      // dead lanes never match anything
+    int rank = 0, same = 0;
+#pragma unroll
+    for (int t = 0; t < 64; ++t) {
+      const int kt = __builtin_amdgcn_readlane(key, t);
+      const int eq = (kt == key) ? 1 : 0;
+      rank += (t < lane) ? eq : 0;
+      same += eq;
+    }
+    if (j >= 0) list[base[j] + rank] = entry;
+    __syncthreads();
+    if (j >= 0 && rank == same - 1) base[j] += same;
+    __syncthreads();
+  }
+}
+
+// --------------------------------------------------------------------------- shared pieces
+
+struct UnitInfo {
+  int j, own, lst0, v0, v1;
+};
+
+// unit -> (block j, range [v0, v1) of its virtual list).  Returns false for padding units.
+__device__ __forceinline__ bool locate_unit(const SelPlan& P, const char* iws, size_t off_unit, int chunk, int bh, int u, UnitInfo& ui) {
+  const int* unit_off = reinterpret_cast<const int*>(iws + off_unit) + (size_t)bh * (P.W + 1);
+  if (u >= unit_off[P.W]) return false;
+  int lo = 0, hi = P.W - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (unit_off[mid] <= u) lo = mid; else hi = mid - 1;
+  }
+  // blocks with an empty list own no unit: unit_off[lo] == unit_off[lo+1]; the search lands on
+  // the last j with unit_off[j] <= u, which is the one whose range contains u
+  const int* blk = reinterpret_cast<const int*>(iws + P.off_blk) + (size_t)bh * (P.W + 1);
+  ui.j = lo;
+  ui.own = P.causal ? min(P.B, P.n - lo * P.B) : 0;
+  ui.lst0 = blk[lo];
+  const int L = ui.own + (blk[lo + 1] - blk[lo]);
+  ui.v0 = (u - unit_off[lo]) * chunk;
+  ui.v1 = min(L, ui.v0 + chunk);
+  return ui.v0 < ui.v1;
+}
+
+struct RowInfo {
+  int i, slot, lim, g;
+  bool valid;
+};
+
+// Row `nrow` (0..31) of the 32-row tile starting at virtual position vt.
+__device__ __forceinline__ RowInfo locate_row(const SelPlan& P, const int* list, const UnitInfo& ui, int vt, int nrow) {
+  RowInfo r;
+  const int pv = vt + (nrow >> P.lg);
+  r.valid = pv < ui.v1;
+  const int pvc = r.valid ? pv : vt;
+  r.g = nrow & (P.g - 1);
+  if (pvc < ui.own) {
+    r.i = ui.j * P.B + pvc; r.slot = P.S; r.lim = pvc;
+  } else {
+    const int e = list[ui.lst0 + pvc - ui.own];
+    r.i = e / P.SP; r.slot = e - r.i * P.SP; r.lim = P.B - 1;
+  }
+  return r;
+}
+
+// ------------------------------------------------------------------------------- forward
+
+template <int D, int KT>
+__global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+                                                     const __bf16* __restrict__ v, const char* __restrict__ iws, char* __restrict__ fws) {
+  constexpr int KS = D / 16, DT = D / 32;
+  const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
+  const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
+  UnitInfo ui;
+  if (!locate_unit(P, iws, P.off_unitf, P.chunk_f, bh, blockIdx.x, ui)) return;
+  const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
+
+  bf16x8 Kf[KT][KS];
+  bf16x8 VT[DT][KT][2];
+  {
+    bf16x8 ilo, ihi;
+    make_ident(lane, ilo, ihi);
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      const int kl = 32 * kt + n_;
+      const long key = (long)ui.j * P.B + kl;
+      const bool ok = kl < P.B && key < P.n;
+      const long keyc = ok ? key : 0;
+      const __bf16* kp = k + b * P.sk[0] + hk * P.sk[1] + keyc * P.sk[2] + 8 * h;
+      const __bf16* vp = v + b * P.sv[0] + hk * P.sv[1] + keyc * P.sv[2] + 8 * h;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) Kf[kt][ks] = ok ? load8(kp + 16 * ks) : zero_frag();
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const bf16x8 va = ok ? load8(vp + 32 * dt) : zero_frag();
+        const bf16x8 vb = ok ? load8(vp + 32 * dt + 16) : zero_frag();
+        floatx16 t = mfma32(va, ilo, zero_acc());
+        t = mfma32(vb, ihi, t);
+        VT[dt][kt][0] = pack8(t, 0);
+        VT[dt][kt][1] = pack8(t, 8);
+      }
+    }
+  }
+
+  __bf16* opart = reinterpret_cast<__bf16*>(fws + P.off_opart);
+  float* lsepart = reinterpret_cast<float*>(fws + P.off_lsepart);
+  const float sc = P.scale * kLog2e;
+  const int ppt = 32 >> P.lg;
+
+  for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
+    const RowInfo r = locate_row(P, list, ui, vt, n_);
+    const __bf16* qp = q + b * P.sq[0] + (long)(hk * P.g + r.g) * P.sq[1] + (long)r.i * P.sq[2] + 8 * h;
+    bf16x8 Qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) Qf[ks] = load8(qp + 16 * ks);
+
+    floatx16 Sa[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      Sa[kt] = zero_acc();
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) Sa[kt] = mfma32(Kf[kt][ks], Qf[ks], Sa[kt]);
+    }
+    // local softmax over the block's keys; this lane holds 16*KT keys of row n_, lane^32 the rest
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int i2 = 0; i2 < 16; ++i2) {
+        const int kl = 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
+        const float s = (kl <= r.lim) ? Sa[kt][i2] * sc : -INFINITY;
+        Sa[kt][i2] = s;
+        mx = fmaxf(mx, s);
+      }
+    mx = fmaxf(mx, xor32(mx));
+    float l = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int i2 = 0; i2 < 16; ++i2) {
+        const float p = fast_exp2(Sa[kt][i2] - mx);
+        Sa[kt][i2] = p;
+        l += p;
+      }
+    l += xor32(l);
+
+    floatx16 Oa[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) Oa[dt] = zero_acc();
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int u2 = 0; u2 < 2; ++u2) {
+        const bf16x8 Pf = pack8(Sa[kt], 8 * u2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) Oa[dt] = mfma32(VT[dt][kt][u2], Pf, Oa[dt]);
+      }
+
+    if (r.valid) {
+      const float inv = 1.0f / l;
+      const size_t row = (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g;
+      __bf16* op = opart + row * D + 4 * h;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+          store4_bf16(op + 32 * dt + 8 * a, Oa[dt][4 * a] * inv, Oa[dt][4 * a + 1] * inv, Oa[dt][4 * a + 2] * inv, Oa[dt][4 * a + 3] * inv);
+      if (h == 0) lsepart[row] = (mx + fast_log2(l)) * kLn2;
+    }
+  }
+}
+
+// live-slot bitmask of query (bh, i): bit s < S = selected slot s, bit S = own block
+__device__ __forceinline__ unsigned long long live_slots(const SelPlan& P, const void* idx, const uint8_t* fmask, int bh, int i, int lane) {
+  bool ok = false;
+  if (lane < P.S) {
+    const size_t pos = ((size_t)bh * P.n + i) * P.S + lane;
+    if (fmask[pos]) {
+      const int j = read_idx(idx, P.idx64, pos);
+      ok = j >= 0 && j < P.W;
+    }
+  } else if (lane == P.S) {
+    ok = P.causal != 0;
+  }
+  return __ballot(ok);
+}
+
+// merge the per-slot partials of one query: out = sum_s exp(lse_s - LSE) * o_s
+template <int D>
+__global__ __launch_bounds__(256) void sel_fwd_combine_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, const char* __restrict__ fws,
+                                                             __bf16* __restrict__ out, float* __restrict__ lse) {
+  const int lane = threadIdx.x & 63;
+  const long qi = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (qi >= (long)P.bh * P.n) return;
+  const int bh = (int)(qi / P.n), i = (int)(qi % P.n);
+  const int b = bh / P.hkv, hk = bh % P.hkv;
+  const unsigned long long live = live_slots(P, idx, fmask, bh, i, lane);
+  const __bf16* opart = reinterpret_cast<const __bf16*>(fws + P.off_opart);
+  const float* lsepart = reinterpret_cast<const float*>(fws + P.off_lsepart);
+  constexpr int CPR = D / 8;                    // 16-byte chunks per row
+  for (int c = lane; c < P.g * CPR; c += 64) {
+    const int g = c / CPR, dd = (c % CPR) * 8;
+    const size_t row0 = ((size_t)bh * P.n + i) * P.SP * P.g + g;
+    float mx = -INFINITY;
+    for (unsigned long long m = live; m; m &= m - 1) {
+      const int s = __builtin_ctzll(m);
+      mx = fmaxf(mx, lsepart[row0 + (size_t)s * P.g]);
+    }
+    float sum = 0.f;
+    for (unsigned long long m = live; m; m &= m - 1) {
+      const int s = __builtin_ctzll(m);
+      sum += __expf(lsepart[row0 + (size_t)s * P.g] - mx);
+    }
+    const float L = live ? mx + __logf(sum) : -INFINITY;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (unsigned long long m = live; m; m &= m - 1) {
+      const int s = __builtin_ctzll(m);
+      const size_t row = row0 + (size_t)s * P.g;
+      const float w = __expf(lsepart[row] - L);
+      const bf16x8 o = load8(opart + row * D + dd);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += w * (float)o[e];
+    }
+    const int hq = hk * P.g + g;
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (__bf16)acc[e];
+    *reinterpret_cast<bf16x8*>(out + b * P.so[0] + (long)hq * P.so[1] + (long)i * P.so[2] + dd) = r;
+    if (dd == 0) lse[((size_t)b * P.hkv * P.g + hq) * P.n + i] = L;
+  }
+}
+
+// ------------------------------------------------------------------------------ backward
+
+// delta[b,hq,i] = sum_d out * d_out   (TRI.py:696-756)
+template <int D>
+__global__ __launch_bounds__(256) void sel_delta_kernel(const SelPlan P, const __bf16* __restrict__ out, const __bf16* __restrict__ dout, float* __restrict__ delta) {
+  constexpr int LPR = D / 8;                   // lanes per row
+  constexpr int RPB = 256 / LPR;               // rows per block
+  const int tid = threadIdx.x;
+  const long row = (long)blockIdx.x * RPB + tid / LPR;
+  const long rows = (long)P.bh * P.g * P.n;
+  const int dd = (tid % LPR) * 8;
+  float s = 0.f;
+  if (row < rows) {
+    const long i = row % P.n, bhq = row / P.n;
+    const long b = bhq / (P.hkv * P.g), hq = bhq % (P.hkv * P.g);
+    const long off = b * P.so[0] + hq * P.so[1] + i * P.so[2] + dd;
+    const bf16x8 o = load8(out + off), d = load8(dout + off);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += (float)o[e] * (float)d[e];
+  }
+#pragma unroll
+  for (int m = LPR / 2; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+  if (row < rows && (tid % LPR) == 0) delta[row] = s;
+}
+
+// dQ partial of every (query, slot) pair; same walk and register layout as the forward
+template <int D, int KT>
+__global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+                                                        const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
+                                                        const float* __restrict__ lse, const float* __restrict__ delta,
+                                                        const char* __restrict__ iws, char* __restrict__ bws) {
+  constexpr int KS = D / 16, DT = D / 32;
+  const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
+  const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
+  UnitInfo ui;
+  if (!locate_unit(P, iws, P.off_unitf, P.chunk_f, bh, blockIdx.x, ui)) return;
+  const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
+
+  bf16x8 Kf[KT][KS], Vf[KT][KS];
+  bf16x8 KTf[DT][KT][2];
+  {
+    bf16x8 ilo, ihi;
+    make_ident(lane, ilo, ihi);
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      const int kl = 32 * kt + n_;
+      const long key = (long)ui.j * P.B + kl;
+      const bool ok = kl < P.B && key < P.n;
+      const long keyc = ok ? key : 0;
+      const __bf16* kp = k + b * P.sk[0] + hk * P.sk[1] + keyc * P.sk[2] + 8 * h;
+      const __bf16* vp = v + b * P.sv[0] + hk * P.sv[1] + keyc * P.sv[2] + 8 * h;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        Kf[kt][ks] = ok ? load8(kp + 16 * ks) : zero_frag();
+        Vf[kt][ks] = ok ? load8(vp + 16 * ks) : zero_frag();
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        floatx16 t = mfma32(Kf[kt][2 * dt], ilo, zero_acc());
+        t = mfma32(Kf[kt][2 * dt + 1], ihi, t);
+        KTf[dt][kt][0] = pack8(t, 0);
+        KTf[dt][kt][1] = pack8(t, 8);
+      }
+    }
+  }
+
+  __bf16* dqpart = reinterpret_cast<__bf16*>(bws + P.off_dqpart);
+  const float sc = P.scale * kLog2e;
+  const int ppt = 32 >> P.lg;
+  const int HQ = P.hkv * P.g;
+
+  for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
+    const RowInfo r = locate_row(P, list, ui, vt, n_);
+    const int hq = hk * P.g + r.g;
+    const __bf16* qp = q + b * P.sq[0] + (long)hq * P.sq[1] + (long)r.i * P.sq[2] + 8 * h;
+    const __bf16* dop = dout + b * P.so[0] + (long)hq * P.so[1] + (long)r.i * P.so[2] + 8 * h;
+    bf16x8 Qf[KS], Gf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) { Qf[ks] = load8(qp + 16 * ks); Gf[ks] = load8(dop + 16 * ks); }
+    const size_t srow = ((size_t)b * HQ + hq) * P.n + r.i;
+    const float lse_r = lse[srow] * kLog2e;
+    const float del_r = delta[srow];
+
+    floatx16 Sa[KT], Pa[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      Sa[kt] = zero_acc(); Pa[kt] = zero_acc();
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        Sa[kt] = mfma32(Kf[kt][ks], Qf[ks], Sa[kt]);
+        Pa[kt] = mfma32(Vf[kt][ks], Gf[ks], Pa[kt]);
+      }
+    }
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int i2 = 0; i2 < 16; ++i2) {
+        const int kl = 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
+        const float p = (kl <= r.lim) ? fast_exp2(Sa[kt][i2] * sc - lse_r) : 0.f;
+        Sa[kt][i2] = p * (Pa[kt][i2] - del_r);
+      }
+    floatx16 Qa[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) Qa[dt] = zero_acc();
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int u2 = 0; u2 < 2; ++u2) {
+        const bf16x8 Sf = pack8(Sa[kt], 8 * u2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) Qa[dt] = mfma32(KTf[dt][kt][u2], Sf, Qa[dt]);
+      }
+    if (r.valid) {
+      const size_t row = (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g;
+      __bf16* op = dqpart + row * D + 4 * h;
+      const float s = P.scale;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+          store4_bf16(op + 32 * dt + 8 * a, Qa[dt][4 * a] * s, Qa[dt][4 * a + 1] * s, Qa[dt][4 * a + 2] * s, Qa[dt][4 * a + 3] * s);
+    }
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, const char* __restrict__ bws,
+                                                                __bf16* __restrict__ dq) {
+  const int lane = threadIdx.x & 63;
+  const long qi = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (qi >= (long)P.bh * P.n) return;
+  const int bh = (int)(qi / P.n), i = (int)(qi % P.n);
+  const int b = bh / P.hkv, hk = bh % P.hkv;
+  const unsigned long long live = live_slots(P, idx, fmask, bh, i, lane);
+  const __bf16* dqpart = reinterpret_cast<const __bf16*>(bws + P.off_dqpart);
+  constexpr int CPR = D / 8;
+  for (int c = lane; c < P.g * CPR; c += 64) {
+    const int g = c / CPR, dd = (c % CPR) * 8;
+    const size_t row0 = ((size_t)bh * P.n + i) * P.SP * P.g + g;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (unsigned long long m = live; m; m &= m - 1) {
+      const int s = __builtin_ctzll(m);
+      const bf16x8 o = load8(dqpart + (row0 + (size_t)s * P.g) * D + dd);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += (float)o[e];
+    }
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = (__bf16)acc[e];
+    const long hq = hk * P.g + g;
+    *reinterpret_cast<bf16x8*>(dq + (((long)b * P.hkv * P.g + hq) * P.n + i) * D + dd) = r;
+  }
+}
+
+// dK/dV of one 32-key tile of one block, accumulated over a chunk of the block's virtual list.
+// S is computed as Q K^T (rows on the MFMA M side) so that P and dS come out with lane <-> key
+// and registers <-> rows, which is the B-operand layout of dV^T = dO^T P and dK^T = Q^T dS;
+// dO^T and Q^T (lane <-> feature, registers <-> rows) are made with identity-MFMA transposes.
+template <int D, int KT>
+__global__ __launch_bounds__(64) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+                                                         const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
+                                                         const float* __restrict__ lse, const float* __restrict__ delta,
+                                                         const char* __restrict__ iws, char* __restrict__ bws) {
+  constexpr int KS = D / 16, DT = D / 32;
+  __shared__ __align__(16) float lse_s[32];
+  __shared__ __align__(16) float del_s[32];
+  __shared__ __align__(16) int lim_s[32];
+  const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
+  const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
+  const int u = blockIdx.x / KT, kt = blockIdx.x % KT;
+  UnitInfo ui;
+  if (!locate_unit(P, iws, P.off_unitkv, P.chunk_kv, bh, u, ui)) return;
+  const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
+
+  bf16x8 Kf[KS], Vf[KS], ilo, ihi;
+  make_ident(lane, ilo, ihi);
+  const int kl = 32 * kt + n_;                 // this lane's key inside the block
+  {
+    const long key = (long)ui.j * P.B + kl;
+    const bool ok = kl < P.B && key < P.n;
+    const long keyc = ok ? key : 0;
+    const __bf16* kp = k + b * P.sk[0] + hk * P.sk[1] + keyc * P.sk[2] + 8 * h;
+    const __bf16* vp = v + b * P.sv[0] + hk * P.sv[1] + keyc * P.sv[2] + 8 * h;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      Kf[ks] = ok ? load8(kp + 16 * ks) : zero_frag();
+      Vf[ks] = ok ? load8(vp + 16 * ks) : zero_frag();
+    }
+  }
+  floatx16 dKa[DT], dVa[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) { dKa[dt] = zero_acc(); dVa[dt] = zero_acc(); }
+
+  const float sc = P.scale * kLog2e;
+  const int ppt = 32 >> P.lg;
+  const int HQ = P.hkv * P.g;
+
+  for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
+    const RowInfo r = locate_row(P, list, ui, vt, n_);
+    const int hq = hk * P.g + r.g;
+    const __bf16* qp = q + b * P.sq[0] + (long)hq * P.sq[1] + (long)r.i * P.sq[2] + 8 * h;
+    const __bf16* dop = dout + b * P.so[0] + (long)hq * P.so[1] + (long)r.i * P.so[2] + 8 * h;
+    bf16x8 Qf[KS], Gf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) { Qf[ks] = load8(qp + 16 * ks); Gf[ks] = load8(dop + 16 * ks); }
+    if (h == 0) {
+      const size_t srow = ((size_t)b * HQ + hq) * P.n + r.i;
+      lse_s[n_] = r.valid ? lse[srow] * kLog2e : INFINITY;   // +inf: a padding row gets p = 0
+      del_s[n_] = delta[srow];
+      lim_s[n_] = r.lim;
+    }
+    __syncthreads();
+
+    floatx16 Sa = zero_acc(), Pa = zero_acc();
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      Sa = mfma32(Qf[ks], Kf[ks], Sa);         // [row][key]: lane <-> key, registers <-> rows
+      Pa = mfma32(Gf[ks], Vf[ks], Pa);
+    }
+    floatx16 dSa;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const floatx4 l4 = *reinterpret_cast<const floatx4*>(&lse_s[8 * a + 4 * h]);
+      const floatx4 d4 = *reinterpret_cast<const floatx4*>(&del_s[8 * a + 4 * h]);
+      const int* m4 = &lim_s[8 * a + 4 * h];
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) {
+        const int i2 = 4 * a + bb;
+        const float p = (kl <= m4[bb]) ? fast_exp2(Sa[i2] * sc - l4[bb]) : 0.f;
+        Sa[i2] = p;
+        dSa[i2] = p * (Pa[i2] - d4[bb]);
+      }
+    }
+    const bf16x8 Pf0 = pack8(Sa, 0), Pf1 = pack8(Sa, 8);
+    const bf16x8 Sf0 = pack8(dSa, 0), Sf1 = pack8(dSa, 8);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      floatx16 t = mfma32(Gf[2 * dt], ilo, zero_acc());
+      t = mfma32(Gf[2 * dt + 1], ihi, t);      // t[row][feature]: lane <-> feature, registers <-> rows
+      dVa[dt] = mfma32(pack8(t, 0), Pf0, dVa[dt]);
+      dVa[dt] = mfma32(pack8(t, 8), Pf1, dVa[dt]);
+      t = mfma32(Qf[2 * dt], ilo, zero_acc());
+      t = mfma32(Qf[2 * dt + 1], ihi, t);
+      dKa[dt] = mfma32(pack8(t, 0), Sf0, dKa[dt]);
+      dKa[dt] = mfma32(pack8(t, 8), Sf1, dKa[dt]);
+    }
+    __syncthreads();
+  }
+
+  // partial [unit][2][32*KT keys][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][key kl]
+  float* part = reinterpret_cast<float*>(bws + P.off_dkvpart) + ((size_t)bh * P.ub_kv + u) * (2 * 32 * KT * D);
+  float* pk = part + (size_t)kl * D + 4 * h;
+  float* pv = pk + 32 * KT * D;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      floatx4 x, y;
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) { x[bb] = dKa[dt][4 * a + bb]; y[bb] = dVa[dt][4 * a + bb]; }
+      *reinterpret_cast<floatx4*>(pk + 32 * dt + 8 * a) = x;
+      *reinterpret_cast<floatx4*>(pv + 32 * dt + 8 * a) = y;
+    }
+}
+
+// dk/dv of block j = sum of its units' partials (fixed order -> bit-reproducible)
+template <int D, int KT>
+__global__ __launch_bounds__(256) void sel_bwd_dkv_reduce_kernel(const SelPlan P, const char* __restrict__ iws, const char* __restrict__ bws,
+                                                                __bf16* __restrict__ dk, __bf16* __restrict__ dv) {
+  const int j = blockIdx.x, bh = blockIdx.y;
+  const int* unit_off = reinterpret_cast<const int*>(iws + P.off_unitkv) + (size_t)bh * (P.W + 1);
+  const int u0 = unit_off[j], u1 = unit_off[j + 1];
+  const float* part = reinterpret_cast<const float*>(bws + P.off_dkvpart) + (size_t)bh * P.ub_kv * (2 * 32 * KT * D);
+  const int keys = min(P.B, P.n - j * P.B);
+  constexpr int CPR = D / 4;
+  for (int c = threadIdx.x; c < 2 * keys * CPR; c += 256) {
+    const int which = c / (keys * CPR), rem = c % (keys * CPR);
+    const int key = rem / CPR, dd = (rem % CPR) * 4;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int u = u0; u < u1; ++u) {
+      const floatx4 x = *reinterpret_cast<const floatx4*>(part + (size_t)u * (2 * 32 * KT * D) + (size_t)which * (32 * KT * D) + (size_t)key * D + dd);
+      acc += x;
+    }
+    const float s = which == 0 ? P.scale : 1.0f;
+    __bf16* dst = (which == 0 ? dk : dv) + (((size_t)bh * P.n) + (size_t)j * P.B + key) * D + dd;
+    store4_bf16(dst, acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s);
+  }
+}
+
+}  // namespace nsa
+
+// ----------------------------------------------------------------------------------- host
+
+using namespace nsa;
+
+#define NSA_LAUNCH_CHECK()                         \
+  do {                                             \
+    hipError_t e_ = hipGetLastError();             \
+    if (e_ != hipSuccess) return (int)e_;          \
+  } while (0)
+
+extern "C" int nsa_select_workspace_bytes(const nsa_select_desc* d, size_t* index_bytes, size_t* fwd_bytes, size_t* bwd_bytes) {
+  SelPlan P;
+  const int rc = make_plan(d, P);
+  if (rc) return rc;
+  if (index_bytes) *index_bytes = P.index_total;
+  if (fwd_bytes) *fwd_bytes = P.fwd_total;
+  if (bwd_bytes) *bwd_bytes = P.bwd_total;
+  return 0;
+}
+
+extern "C" int nsa_select_build_index(const nsa_select_desc* d, const void* idx, const uint8_t* fmask, void* index_ws, size_t index_bytes, void* stream) {
+  SelPlan P;
+  const int rc = make_plan(d, P);
+  if (rc) return rc;
+  if (index_bytes < P.index_total) return NSA_E_WORKSPACE;
+  if (!index_ws || (P.S > 0 && (!idx || !fmask))) return NSA_E_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  char* iws = (char*)index_ws;
+  const size_t lds = (size_t)P.W * sizeof(int);
+  hipLaunchKernelGGL(sel_count_kernel, dim3(P.nch, P.bh), dim3(256), lds, st, P, idx, fmask, iws);
+  NSA_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sel_scan_kernel, dim3(P.bh), dim3(256), lds, st, P, iws);
+  NSA_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sel_fill_kernel, dim3(P.nch, P.bh), dim3(64), lds, st, P, idx, fmask, iws);
+  NSA_LAUNCH_CHECK();
+  return 0;
+}
+
+template <int D, int KT>
+static int launch_fwd(const SelPlan& P, const void* q, const void* k, const void* v, const void* idx, const uint8_t* fmask,
+                      const void* iws, void* fws, void* out, float* lse, hipStream_t st) {
+  hipLaunchKernelGGL((sel_fwd_kernel<D, KT>), dim3(P.ub_f, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+                     (const char*)iws, (char*)fws);
+  NSA_LAUNCH_CHECK();
+  const long nq = (long)P.bh * P.n;
+  hipLaunchKernelGGL((sel_fwd_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)fws, (__bf16*)out, lse);
+  NSA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int nsa_select_fwd(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* idx, const uint8_t* fmask,
+                              const void* index_ws, void* fwd_ws, size_t fwd_bytes, void* out, float* lse, void* stream) {
+  SelPlan P;
+  const int rc = make_plan(d, P);
+  if (rc) return rc;
+  if (fwd_bytes < P.fwd_total) return NSA_E_WORKSPACE;
+  if (!q || !k || !v || !index_ws || !fwd_ws || !out || !lse) return NSA_E_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  const int KT = (P.B + 31) / 32;
+  if (P.D == 64 && KT == 1) return launch_fwd<64, 1>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st);
+  if (P.D == 64 && KT == 2) return launch_fwd<64, 2>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st);
+  if (P.D == 128 && KT == 1) return launch_fwd<128, 1>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st);
+  if (P.D == 128 && KT == 2) return launch_fwd<128, 2>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st);
+  return NSA_E_UNSUPPORTED;
+}
+
+template <int D, int KT>
+static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
+                      const void* idx, const uint8_t* fmask, const void* iws, void* bws, void* dq, void* dk, void* dv, hipStream_t st) {
+  float* delta = reinterpret_cast<float*>((char*)bws + P.off_delta);
+  const long rows = (long)P.bh * P.g * P.n;
+  constexpr int RPB = 256 / (D / 8);
+  hipLaunchKernelGGL((sel_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, delta);
+  NSA_LAUNCH_CHECK();
+  hipLaunchKernelGGL((sel_bwd_dq_kernel<D, KT>), dim3(P.ub_f, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+                     (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
+  NSA_LAUNCH_CHECK();
+  const long nq = (long)P.bh * P.n;
+  hipLaunchKernelGGL((sel_bwd_dq_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)bws, (__bf16*)dq);
+  NSA_LAUNCH_CHECK();
+  hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT>), dim3(P.ub_kv * KT, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+                     (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
+  NSA_LAUNCH_CHECK();
+  hipLaunchKernelGGL((sel_bwd_dkv_reduce_kernel<D, KT>), dim3(P.W, P.bh), dim3(256), 0, st, P, (const char*)iws, (const char*)bws, (__bf16*)dk, (__bf16*)dv);
+  NSA_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* out, const void* d_out,
+                              const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
+                              void* dq, void* dk, void* dv, void* stream) {
+  SelPlan P;
+  const int rc = make_plan(d, P);
+  if (rc) return rc;
+  if (bwd_bytes < P.bwd_total) return NSA_E_WORKSPACE;
+  if (!q || !k || !v || !out || !d_out || !lse || !index_ws || !bwd_ws || !dq || !dk || !dv) return NSA_E_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  const int KT = (P.B + 31) / 32;
+  if (P.D == 64 && KT == 1) return launch_bwd<64, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st);
+  if (P.D == 64 && KT == 2) return launch_bwd<64, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st);
+  if (P.D == 128 && KT == 1) return launch_bwd<128, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st);
+  if (P.D == 128 && KT == 2) return launch_bwd<128, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st);
+  return NSA_E_UNSUPPORTED;
+}
+
+extern "C" int nsa_abi_version(void) { return 1; }

@@ -1,0 +1,81 @@
+// Host-side launch plan of the block-selection kernels: validated dimensions, work-unit sizes
+// and the byte layout of the three caller-owned workspaces.  Recomputed from the descriptor on
+// every call (pure function, a few dozen integer operations), passed to kernels by value.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+#include "../../include/nsa_hip.h"
+
+namespace nsa {
+
+struct SelPlan {
+  int b, hkv, g, lg, n, S, SP, B, D, causal, W, nch, bh, idx64;
+  float scale;
+  int chunk_f, chunk_kv;     // pairs per work unit (forward / dQ walk, dK/dV walk)
+  int ub_f, ub_kv;           // upper bound of work units per (batch, kv head)
+  long list_cap;             // inverse-index entries reserved per (batch, kv head)
+  long sq[3], sk[3], sv[3], so[3];
+  // index workspace
+  size_t off_cnt, off_blk, off_unitf, off_unitkv, off_list, index_total;
+  // forward workspace
+  size_t off_opart, off_lsepart, fwd_total;
+  // backward workspace
+  size_t off_delta, off_dqpart, off_dkvpart, bwd_total;
+};
+
+static inline size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static inline int make_plan(const nsa_select_desc* d, SelPlan& P) {
+  if (!d) return NSA_E_ARG;
+  if (d->batch <= 0 || d->kv_heads <= 0 || d->group <= 0 || d->seq <= 0 || d->num_sel < 0 || d->block <= 0) return NSA_E_ARG;
+  if (d->dim_head != 64 && d->dim_head != 128) return NSA_E_UNSUPPORTED;
+  if (d->block != 16 && d->block != 32 && d->block != 64) return NSA_E_UNSUPPORTED;
+  if (d->group > 32 || (d->group & (d->group - 1))) return NSA_E_UNSUPPORTED;
+  if (d->num_sel > 62) return NSA_E_UNSUPPORTED;
+  if (!d->causal && d->num_sel == 0) return NSA_E_ARG;
+  P.b = d->batch; P.hkv = d->kv_heads; P.g = d->group; P.n = d->seq; P.S = d->num_sel; P.SP = d->num_sel + 1;
+  P.B = d->block; P.D = d->dim_head; P.causal = d->causal ? 1 : 0; P.idx64 = d->idx_is_int64 ? 1 : 0;
+  P.scale = d->scale;
+  P.lg = 0;
+  while ((1 << P.lg) < P.g) ++P.lg;
+  P.W = (P.n + P.B - 1) / P.B;
+  if (P.W > 16384) return NSA_E_UNSUPPORTED;
+  if ((long)P.n * P.SP >= 0x7fffffffL) return NSA_E_UNSUPPORTED;
+  P.nch = (P.n + 255) / 256;
+  const long bh = (long)P.b * P.hkv;
+  if (bh > 65535) return NSA_E_UNSUPPORTED;
+  P.bh = (int)bh;
+  for (int t = 0; t < 3; ++t) { P.sq[t] = d->q_stride[t]; P.sk[t] = d->k_stride[t]; P.sv[t] = d->v_stride[t]; P.so[t] = d->o_stride[t]; }
+  for (int t = 0; t < 3; ++t)
+    if ((P.sq[t] | P.sk[t] | P.sv[t] | P.so[t]) & 7) return NSA_E_ARG;      // rows must start 16-byte aligned
+  P.chunk_f = 256;
+  P.chunk_kv = 1024;
+  const long pairs = (long)P.n * (P.S + P.causal);
+  P.ub_f = (int)(P.W + (pairs + P.chunk_f - 1) / P.chunk_f);
+  P.ub_kv = (int)(P.W + (pairs + P.chunk_kv - 1) / P.chunk_kv);
+  P.list_cap = (long)P.n * (P.S > 0 ? P.S : 1);
+
+  size_t o = 0;
+  P.off_cnt = o;    o = align_up(o + (size_t)bh * P.nch * P.W * 4);
+  P.off_blk = o;    o = align_up(o + (size_t)bh * (P.W + 1) * 4);
+  P.off_unitf = o;  o = align_up(o + (size_t)bh * (P.W + 1) * 4);
+  P.off_unitkv = o; o = align_up(o + (size_t)bh * (P.W + 1) * 4);
+  P.off_list = o;   o = align_up(o + (size_t)bh * P.list_cap * 4);
+  P.index_total = o;
+
+  const size_t prow = (size_t)bh * P.n * P.SP * P.g;      // partial rows: (query, slot, head)
+  o = 0;
+  P.off_opart = o;   o = align_up(o + prow * P.D * 2);
+  P.off_lsepart = o; o = align_up(o + prow * 4);
+  P.fwd_total = o;
+
+  const int KT = (P.B + 31) / 32;
+  o = 0;
+  P.off_delta = o;   o = align_up(o + (size_t)bh * P.g * P.n * 4);
+  P.off_dqpart = o;  o = align_up(o + prow * P.D * 2);
+  P.off_dkvpart = o; o = align_up(o + (size_t)bh * P.ub_kv * 2 * 32 * KT * P.D * 4);
+  P.bwd_total = o;
+  return 0;
+}
+
+}  // namespace nsa

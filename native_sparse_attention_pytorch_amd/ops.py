@@ -1,0 +1,163 @@
+"""torch.library custom ops over the C ABI of libnsa_hip.so, and the functional entry points
+that mirror the reference's operator interface.
+
+`native_sparse_attend` keeps the signature of
+native_sparse_attention_pytorch/triton_native_sparse_attention.py:1938-1950 (argument names,
+meaning, asserts); the op runs hand-written gfx950 kernels and nothing else - CPU tensors or a
+missing library raise.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+_BF16 = torch.bfloat16
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Tensor | None) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _rows_ok(t: Tensor) -> bool:
+    return t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+
+
+def _prep(t: Tensor) -> Tensor:
+    """bf16 with unit stride on the head dimension and 16-byte aligned rows (a view when it
+    already is: the qkv projection's 'b n (h d) -> b h n d' view qualifies)."""
+    if t.dtype != _BF16:
+        raise RuntimeError(f"HIP kernels take bfloat16 tensors, got {t.dtype}")
+    if not t.is_cuda:
+        raise RuntimeError("HIP kernels need device tensors; there is no CPU fallback")
+    return t if _rows_ok(t) else t.contiguous()
+
+
+def _select_desc(q, k, v, o, num_sel, block, causal, scale, idx_is_int64) -> _lib.SelectDesc:
+    b, hq, n, d = q.shape
+    hk = k.shape[1]
+    dsc = _lib.SelectDesc()
+    dsc.batch, dsc.kv_heads, dsc.group, dsc.seq = b, hk, hq // hk, n
+    dsc.num_sel, dsc.block, dsc.dim_head, dsc.causal = num_sel, block, d, int(causal)
+    dsc.idx_is_int64 = int(idx_is_int64)
+    dsc.scale = scale
+    for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("o_stride", o)):
+        getattr(dsc, name)[:] = list(t.stride()[:3])
+    return dsc
+
+
+def _ws_sizes(dsc) -> tuple[int, int, int]:
+    a, f, w = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    _lib.check(_lib.lib().nsa_select_workspace_bytes(C.byref(dsc), C.byref(a), C.byref(f), C.byref(w)), "nsa_select_workspace_bytes")
+    return a.value, f.value, w.value
+
+
+# ------------------------------------------------------------------------------- selection
+
+@torch.library.custom_op("nsa_amd::select_fwd", mutates_args=())
+def select_fwd(q: Tensor, k: Tensor, v: Tensor, idx: Tensor, fmask: Tensor, block: int, causal: bool, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    b, hq, n, d = q.shape
+    idx = idx.contiguous()
+    fm = fmask.contiguous().view(torch.uint8) if fmask.dtype == torch.bool else fmask.contiguous().to(torch.uint8)
+    if idx.dtype not in (torch.int64, torch.int32):
+        raise RuntimeError("selected_block_indices must be int64 or int32")
+    out = torch.empty((b, hq, n, d), dtype=_BF16, device=q.device)
+    lse = torch.empty((b, hq, n), dtype=torch.float32, device=q.device)
+    dsc = _select_desc(q, k, v, out, idx.shape[-1], block, causal, scale, idx.dtype == torch.int64)
+    ib, fb, _ = _ws_sizes(dsc)
+    index_ws = torch.empty(ib, dtype=torch.uint8, device=q.device)
+    fwd_ws = torch.empty(fb, dtype=torch.uint8, device=q.device)
+    L = _lib.lib()
+    st = _stream()
+    _lib.check(L.nsa_select_build_index(C.byref(dsc), _ptr(idx), _ptr(fm), _ptr(index_ws), ib, st), "nsa_select_build_index")
+    _lib.check(L.nsa_select_fwd(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(idx), _ptr(fm), _ptr(index_ws), _ptr(fwd_ws), fb,
+                                _ptr(out), _ptr(lse), st), "nsa_select_fwd")
+    return out, lse, index_ws
+
+
+@select_fwd.register_fake
+def _(q, k, v, idx, fmask, block, causal, scale):
+    b, hq, n, d = q.shape
+    return (q.new_empty((b, hq, n, d)), q.new_empty((b, hq, n), dtype=torch.float32), q.new_empty((1,), dtype=torch.uint8))
+
+
+@torch.library.custom_op("nsa_amd::select_bwd", mutates_args=())
+def select_bwd(q: Tensor, k: Tensor, v: Tensor, out: Tensor, dout: Tensor, lse: Tensor, idx: Tensor, fmask: Tensor,
+               index_ws: Tensor, block: int, causal: bool, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    out = out.contiguous()
+    dout = dout.contiguous()
+    if dout.dtype != _BF16:
+        dout = dout.to(_BF16)
+    idx = idx.contiguous()
+    fm = fmask.contiguous().view(torch.uint8) if fmask.dtype == torch.bool else fmask.contiguous().to(torch.uint8)
+    b, hq, n, d = q.shape
+    hk = k.shape[1]
+    dq = torch.empty((b, hq, n, d), dtype=_BF16, device=q.device)
+    dk = torch.empty((b, hk, n, d), dtype=_BF16, device=q.device)
+    dv = torch.empty((b, hk, n, d), dtype=_BF16, device=q.device)
+    dsc = _select_desc(q, k, v, out, idx.shape[-1], block, causal, scale, idx.dtype == torch.int64)
+    ib, _, wb = _ws_sizes(dsc)
+    if index_ws.numel() < ib:
+        raise RuntimeError("inverse index workspace does not belong to these shapes")
+    bwd_ws = torch.empty(wb, dtype=torch.uint8, device=q.device)
+    _lib.check(_lib.lib().nsa_select_bwd(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(idx), _ptr(fm),
+                                         _ptr(index_ws), _ptr(bwd_ws), wb, _ptr(dq), _ptr(dk), _ptr(dv), _stream()), "nsa_select_bwd")
+    return dq, dk, dv
+
+
+@select_bwd.register_fake
+def _(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale):
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
+def _select_setup(ctx, inputs, output):
+    q, k, v, idx, fmask, block, causal, scale = inputs
+    out, lse, index_ws = output
+    ctx.save_for_backward(q, k, v, out, lse, idx, fmask, index_ws)
+    ctx.args = (block, causal, scale)
+
+
+def _select_backward(ctx, dout, dlse, dws):
+    q, k, v, out, lse, idx, fmask, index_ws = ctx.saved_tensors
+    block, causal, scale = ctx.args
+    dq, dk, dv = select_bwd(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale)
+    return dq, dk, dv, None, None, None, None, None
+
+
+select_fwd.register_autograd(_select_backward, setup_context=_select_setup)
+
+
+def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, selected_block_indices: Tensor, fmask: Tensor,
+                         sel_scale: Tensor | None = None, include_block_causal: bool = True, return_lse: bool = False,
+                         block_dk_dv_use_dot=None, return_sliding_window_out: bool = False):
+    """Drop-in for native_sparse_attend (TRI.py:1938-1987): fq [b,Hq,n,d], fk/fv [b,Hkv,n,d],
+    selected_block_indices / fmask [b,Hkv|Hq,n,S].  Returns out [b,Hq,n,d] in fq's dtype and,
+    on request, lse [b,Hq,n] (fp32).  Inputs are computed in bf16 (the reference computes in
+    fp16, TRI.py:1845).  `block_dk_dv_use_dot` is accepted and ignored (a Triton tuning switch)."""
+    q_heads, kv_heads, sel_heads = fq.shape[1], fk.shape[1], selected_block_indices.shape[1]
+    assert q_heads % kv_heads == 0
+    assert sel_heads in (q_heads, kv_heads)
+    assert block_size >= 16, 'fine selection block size must be 16 or greater for now'
+    if return_sliding_window_out:
+        raise NotImplementedError("the fused sliding-window output is experimental in the reference "
+                                  "(test_triton_nsa.py:144) and is served by sliding_attend here")
+    if sel_scale is not None:
+        raise NotImplementedError("sel_scale (differentiable top-k gates) is not implemented in the HIP path yet")
+    dtype = fq.dtype
+    if kv_heads != sel_heads:                         # per-query-head selection: TRI.py:1961-1962
+        g = q_heads // kv_heads
+        fk, fv = fk.repeat_interleave(g, dim=1), fv.repeat_interleave(g, dim=1)
+    scale = fq.shape[-1] ** -0.5
+    out, lse, _ = select_fwd(fq.to(_BF16), fk.to(_BF16), fv.to(_BF16), selected_block_indices, fmask,
+                             int(block_size), bool(include_block_causal), float(scale))
+    out = out.to(dtype)
+    return (out, lse) if return_lse else out

@@ -1,0 +1,173 @@
+"""Parity of the HIP block-selection attention (through the C ABI) against the CPU oracle.
+Tolerances are BASELINE.json's: forward 2e-2 abs / 1e-2 rel in bf16, gradients 5e-2 rel."""
+import ctypes as C
+
+import pytest
+import torch
+
+from oracle import nsa_oracle as O
+from tests.util import assert_close, causal_random_selection
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def _inputs(b, hq, hk, n, d, seed):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda h: (torch.randn(b, h, n, d, generator=g) * d ** -0.25).to(torch.bfloat16)
+    return mk(hq), mk(hk), mk(hk), mk(hq)
+
+
+def test_mfma_register_layout_selftest():
+    from native_sparse_attention_pytorch_amd import _lib
+    g = torch.Generator().manual_seed(0)
+    A = torch.randn(32, 16, generator=g).to(torch.bfloat16).to(DEV)
+    B = torch.randn(16, 32, generator=g).to(torch.bfloat16).to(DEV)
+    X = torch.randn(32, 32, generator=g).to(torch.bfloat16).to(DEV)
+    Cm = torch.zeros(32, 32, device=DEV)
+    T = torch.zeros(32, 32, device=DEV)
+    rc = _lib.lib().nsa_selftest_mfma(A.data_ptr(), B.data_ptr(), Cm.data_ptr(), X.data_ptr(), T.data_ptr(),
+                                      torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.allclose(Cm.cpu(), A.float().cpu() @ B.float().cpu(), atol=1e-4)
+    assert torch.equal(T.cpu(), X.float().cpu())
+
+
+CASES = [
+    # b, hq, hk, n,   d,  B,  S
+    (2, 4, 2, 200, 64, 16, 3),       # ragged n, G=2
+    (1, 8, 2, 512, 128, 64, 4),      # G=4, d=128
+    (1, 4, 4, 300, 64, 32, 5),       # G=1, ragged
+    (1, 16, 2, 1024, 64, 64, 16),    # G=8, config-2-like
+    (1, 8, 2, 1000, 128, 32, 7),     # ragged, d=128, B=32
+]
+
+
+@pytest.mark.parametrize("b,hq,hk,n,d,B,S", CASES)
+def test_select_fwd_bwd_matches_oracle(b, hq, hk, n, d, B, S):
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    print(f"case b={b} hq={hq} hk={hk} n={n} d={d} B={B} S={S}", flush=True)
+    q, k, v, do = _inputs(b, hq, hk, n, d, seed=n + S)
+    idx, msk = causal_random_selection(b, hk, n, B, S, seed=7)
+
+    qr, kr, vr = (t.float().requires_grad_() for t in (q, k, v))
+    ref, ref_lse = O.select_attend(qr, kr, vr, idx, msk, B, causal=True, return_lse=True)
+    (ref * do.float()).sum().backward()
+
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    out, lse = native_sparse_attend(qg, kg, vg, B, idx.to(DEV), msk.to(DEV), return_lse=True)
+    (out.float() * do.to(DEV).float()).sum().backward()
+    torch.cuda.synchronize()
+
+    assert_close(out, ref, 2e-2, 1e-2, "out")
+    assert_close(lse, ref_lse, 1e-2, 1e-3, "lse")
+    for name, got, want in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
+        assert_close(got, want, 2e-2 * want.abs().max().item(), 5e-2, name)
+
+
+def test_select_reference_script_contract():
+    """Shapes and input law of test_triton_nsa.py:137-153: ragged n=507, duplicate block ids,
+    random slot mask; tolerances of test_triton_nsa.py:189-197."""
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    b, hq, hk, n, d, B, S = 4, 8, 2, 507, 64, 32, 2
+    g = torch.Generator().manual_seed(11)
+    q, k, v = (torch.randn(b, h, n, d, generator=g).to(torch.bfloat16) for h in (hq, hk, hk))
+    idx = torch.randint(0, 2, (b, hk, n, S), generator=g)
+    msk = torch.randint(0, 2, (b, hk, n, S), generator=g).bool()
+    qr, kr, vr = (t.float().requires_grad_() for t in (q, k, v))
+    ref, ref_lse = O.select_attend(qr, kr, vr, idx, msk, B, causal=True, return_lse=True)
+    ref.sum().backward()
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    out, lse = native_sparse_attend(qg, kg, vg, B, idx.to(DEV), msk.to(DEV), return_lse=True)
+    out.float().sum().backward()
+    torch.cuda.synchronize()
+    assert_close(out, ref, 2e-2, 1e-2, "out")
+    assert_close(lse, ref_lse, 1e-2, 0, "lse")
+    assert_close(vg.grad, vr.grad, 2e-2 * vr.grad.abs().max().item(), 5e-2, "dv")
+    assert_close(qg.grad, qr.grad, 2e-2 * qr.grad.abs().max().item(), 5e-2, "dq")
+    assert_close(kg.grad, kr.grad, 2e-2 * kr.grad.abs().max().item(), 5e-2, "dk")
+
+
+def test_select_strided_views_and_per_head_selection():
+    """q/k/v as 'b n (h d) -> b h n d' views of one projection output (NSA.py:583-585) and
+    selection per query head (query_heads_share_selected_kv=False, TRI.py:1961-1962)."""
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    b, hq, hk, n, d, B, S = 2, 4, 2, 256, 64, 16, 4
+    g = torch.Generator().manual_seed(5)
+    proj = (torch.randn(b, n, (hq + 2 * hk) * d, generator=g) * 0.5).to(torch.bfloat16)
+    def views(t):
+        q, k, v = t.split((hq * d, hk * d, hk * d), dim=-1)
+        sh = lambda x: x.reshape(b, n, -1, d).permute(0, 2, 1, 3)
+        return sh(q), sh(k), sh(v)
+    idx, msk = causal_random_selection(b, hq, n, B, S, seed=3)
+    q, k, v = views(proj.float())
+    ref = O.select_attend(q, k, v, idx, msk, B, causal=True)
+    qg, kg, vg = views(proj.to(DEV))
+    assert not qg.is_contiguous()
+    out = native_sparse_attend(qg, kg, vg, B, idx.to(DEV), msk.to(DEV))
+    assert_close(out, ref, 2e-2, 1e-2, "out (strided, per-head selection)")
+
+
+def test_select_backward_is_bit_reproducible():
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    b, hq, hk, n, d, B, S = 1, 8, 2, 2048, 64, 64, 8
+    q, k, v, do = _inputs(b, hq, hk, n, d, seed=1)
+    idx, msk = causal_random_selection(b, hk, n, B, S, seed=2)
+    grads = []
+    for _ in range(2):
+        qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+        out = native_sparse_attend(qg, kg, vg, B, idx.to(DEV), msk.to(DEV))
+        (out.float() * do.to(DEV).float()).sum().backward()
+        torch.cuda.synchronize()
+        grads.append((out.detach().clone(), qg.grad.clone(), kg.grad.clone(), vg.grad.clone()))
+    for a, b_ in zip(*grads):
+        assert torch.equal(a, b_)
+
+
+def test_select_full_size_property():
+    """BASELINE config 2 size (n=8192, 16/4 heads, d=64, B=64, 15 selected + own block): with
+    every earlier block selected where possible the result must equal dense causal attention
+    for the first S*B+B tokens, and rows are convex combinations of V everywhere."""
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    b, hq, hk, n, d, B, S = 1, 16, 4, 8192, 64, 64, 15
+    q, k, v, _ = _inputs(b, hq, hk, n, d, seed=9)
+    idx, msk = causal_random_selection(b, hk, n, B, S, seed=4)
+    out, lse = native_sparse_attend(q.to(DEV), k.to(DEV), v.to(DEV), B, idx.to(DEV), msk.to(DEV), return_lse=True)
+    m = (S + 1) * B                       # queries below m see their whole causal prefix
+    g = hq // hk
+    dense = torch.nn.functional.scaled_dot_product_attention(
+        q[:, :, :m].float(), k[:, :, :m].float().repeat_interleave(g, 1), v[:, :, :m].float().repeat_interleave(g, 1), is_causal=True)
+    assert_close(out[:, :, :m], dense, 2e-2, 1e-2, "dense prefix")
+    vmax = v.float().abs().amax(dim=(2,), keepdim=True).repeat_interleave(g, 1)
+    assert (out.float().cpu().abs() <= vmax + 1e-2).all()
+    assert torch.isfinite(lse).all()
+    # brute-force rows for a slice of late queries
+    sl = slice(n - 128, n)
+    sel_ref = _oracle_rows(q.float(), k.float(), v.float(), idx, msk, B, sl)
+    assert_close(out[:, :, sl], sel_ref, 2e-2, 1e-2, "late queries")
+
+
+def _oracle_rows(q, k, v, idx, msk, B, sl):
+    """brute-force (python loops) selection attention for the queries of a slice"""
+    import math
+    n = q.shape[2]
+    out = torch.zeros(q.shape[0], q.shape[1], sl.stop - sl.start, q.shape[3])
+    import torch.nn.functional as F
+    b, hq, _, d = q.shape
+    hk = k.shape[1]
+    g = hq // hk
+    W = math.ceil(n / B)
+    kp = F.pad(k, (0, 0, 0, W * B - n)).reshape(b, hk, W, B, d)
+    vp = F.pad(v, (0, 0, 0, W * B - n)).reshape(b, hk, W, B, d)
+    for t, i in enumerate(range(sl.start, sl.stop)):
+        for bi in range(b):
+            for h in range(hk):
+                blocks = [int(j) for j, m in zip(idx[bi, h, i], msk[bi, h, i]) if m]
+                keys = torch.cat([kp[bi, h, j] for j in blocks] + [k[bi, h, (i // B) * B:i + 1]])
+                vals = torch.cat([vp[bi, h, j] for j in blocks] + [v[bi, h, (i // B) * B:i + 1]])
+                for gg in range(g):
+                    p = torch.softmax((keys @ q[bi, h * g + gg, i]) * d ** -0.5, dim=0)
+                    out[bi, h * g + gg, t] = p @ vals
+    return out

@@ -1,0 +1,38 @@
+"""Shared helpers for the parity tests."""
+import math
+
+import torch
+
+
+def causal_random_selection(b, h, n, B, S, seed, own_reserved=0):
+    """For query i in block w = i // B: min(w, S) distinct blocks drawn uniformly from [0, w)
+    (random-score top-k), remaining slots dead.  Vectorised; CPU int64/bool tensors."""
+    g = torch.Generator().manual_seed(seed)
+    W = math.ceil(n / B)
+    scores = torch.rand(b, h, n, W, generator=g)
+    blk = (torch.arange(n) // B)[None, None, :, None]
+    scores = scores.masked_fill(torch.arange(W)[None, None, None, :] >= blk, -1.0)
+    k = min(S, W)
+    vals, idx = scores.topk(k, dim=-1)
+    mask = vals >= 0
+    if k < S:
+        idx = torch.nn.functional.pad(idx, (0, S - k))
+        mask = torch.nn.functional.pad(mask, (0, S - k))
+    idx = idx.masked_fill(~mask, 0)
+    return idx, mask
+
+
+def rel_err(a, b):
+    return ((a.float() - b.float()).abs().max() / b.float().abs().max().clamp_min(1e-12)).item()
+
+
+def assert_close(got, want, atol, rtol, what=""):
+    got, want = got.float().cpu(), want.float().cpu()
+    err = (got - want).abs()
+    tol = atol + rtol * want.abs()
+    bad = err > tol
+    if bad.any():
+        i = torch.nonzero(bad)[0].tolist()
+        raise AssertionError(f"{what}: {int(bad.sum())}/{bad.numel()} elements out of tolerance; "
+                             f"max err {err.max().item():.4g} (ref max {want.abs().max().item():.4g}); first at {i}: "
+                             f"got {got[tuple(i)].item():.6g} want {want[tuple(i)].item():.6g}")
