@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""Headline benchmark: block-selection attention forward+backward at sequence 32k in bf16
+(BASELINE.json configs[3]: batch 1, 32 query heads, 8 kv heads, dim_head 128,
+selection_block_size 64, 16 blocks per query = 15 selected + the query's own block).
+
+One "step" = inverse-index build + forward + backward through the C ABI of libnsa_hip.so with
+all inputs resident in HBM.  Prints ONE JSON line (see the keys below).  `value` is the
+algorithmic TFLOP/s of the whole step: 14*d*P FLOP, P = attended (query, key) pairs summed over
+query heads, causal-discounted own block.  Kernel durations come from HIP events recorded on the
+launch stream between the kernels (nsa_select_*_timed).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_PEAK_TFLOPS = 2500.0      # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+
+CFG = dict(batch=1, seq=32768, heads=32, kv_heads=8, dim_head=128, block=64, num_sel=15)
+
+
+def selection(b, h, n, B, S, seed, device):
+    """15 distinct causal blocks per query, uniform over the blocks before the query's own
+    block (random-score top-k), fixed seed; dead slots for early queries."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    W = math.ceil(n / B)
+    scores = torch.rand(b, h, n, W, generator=g, device=device)
+    blk = (torch.arange(n, device=device) // B)[None, None, :, None]
+    scores = scores.masked_fill(torch.arange(W, device=device)[None, None, None, :] >= blk, -1.0)
+    vals, idx = scores.topk(min(S, W), dim=-1)
+    mask = vals >= 0
+    return idx.masked_fill(~mask, 0).contiguous(), mask.contiguous()
+
+
+def attended_pairs(b, hq, n, B, s_total):
+    W = math.ceil(n / B)
+    return b * hq * sum(B * (min(w, s_total - 1) * B + (B + 1) / 2) for w in range(W))
+
+
+class HipEvents:
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+
+    def make(self, n):
+        arr = (C.c_void_p * n)()
+        for i in range(n):
+            e = C.c_void_p()
+            assert self.hip.hipEventCreate(C.byref(e)) == 0
+            arr[i] = e
+        return arr
+
+    def record(self, ev, stream):
+        assert self.hip.hipEventRecord(ev, stream) == 0
+
+    def ms(self, a, b):
+        out = C.c_float()
+        rc = self.hip.hipEventElapsedTime(C.byref(out), a, b)
+        assert rc == 0, rc
+        return out.value
+
+
+def cpu_baseline(cfg, q, k, v, do, idx, msk, nq=512):
+    """The CPU oracle (fp32 restatement of the reference's pure-torch path) on a bounded sample:
+    the last `nq` queries of the same workload against the full-length K/V, forward+backward."""
+    from oracle import nsa_oracle as O
+    n = cfg["seq"]
+    sl = slice(n - nq, n)
+    qc = q[:, :, sl].float().cpu().requires_grad_()
+    kc, vc = k.float().cpu().requires_grad_(), v.float().cpu().requires_grad_()
+    doc = do[:, :, sl].float().cpu()
+    ic, mc = idx[:, :, sl].cpu(), msk[:, :, sl].cpu()
+    t0 = time.perf_counter()
+    out = O.select_attend(qc, kc, vc, ic, mc, cfg["block"], causal=True, q_offset=n - nq, chunk=128)
+    (out * doc).sum().backward()
+    dt = time.perf_counter() - t0
+    return dict(value=nq * cfg["batch"] / dt, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"last {nq} of {n} queries (each attends 16 blocks), full-length K/V, fp32 fwd+bwd, {dt:.1f} s; "
+                       f"host has {os.cpu_count()} logical CPUs"), out.detach()
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X (no CPU fallback for the product path)", file=sys.stderr)
+        sys.exit(2)
+
+    from native_sparse_attention_pytorch_amd import _lib, ops
+    L = _lib.lib()
+    dev = "cuda"
+    cfg = CFG
+    b, n, hq, hk, d, B, S = cfg["batch"], cfg["seq"], cfg["heads"], cfg["kv_heads"], cfg["dim_head"], cfg["block"], cfg["num_sel"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda h: (torch.randn(b, h, n, d, generator=g, device=dev) * d ** -0.5).to(torch.bfloat16)
+    q, k, v, do = mk(hq), mk(hk), mk(hk), mk(hq)
+    idx, msk = selection(b, hk, n, B, S, 0, dev)
+    fm = msk.view(torch.uint8)
+
+    out = torch.empty_like(q)
+    lse = torch.empty(b, hq, n, dtype=torch.float32, device=dev)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dsc = ops._select_desc(q, k, v, out, S, B, True, d ** -0.5, True)
+    ib, fb, wb = ops._ws_sizes(dsc)
+    iws = torch.empty(ib, dtype=torch.uint8, device=dev)
+    # forward and backward workspaces are never live together: share one allocation
+    ws = torch.empty(max(fb, wb), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    hev = HipEvents()
+    P = lambda t: t.data_ptr()
+
+    def step(ev):
+        if ev is not None:
+            hev.record(ev[0], stream)
+        _lib.check(L.nsa_select_build_index(C.byref(dsc), P(idx), P(fm), P(iws), ib, stream), "build_index")
+        fe = C.cast(C.byref(ev, 1 * C.sizeof(C.c_void_p)), C.c_void_p) if ev is not None else None
+        be = C.cast(C.byref(ev, 4 * C.sizeof(C.c_void_p)), C.c_void_p) if ev is not None else None
+        _lib.check(L.nsa_select_fwd_timed(C.byref(dsc), P(q), P(k), P(v), P(idx), P(fm), P(iws), P(ws), fb, P(out), P(lse), stream,
+                                          fe, 3 if ev is not None else 0), "fwd")
+        _lib.check(L.nsa_select_bwd_timed(C.byref(dsc), P(q), P(k), P(v), P(out), P(do), P(lse), P(idx), P(fm), P(iws), P(ws), wb,
+                                          P(dq), P(dk), P(dv), stream, be, 6 if ev is not None else 0), "bwd")
+
+    for _ in range(args.warmup):
+        step(None)
+    torch.cuda.synchronize()
+    evs = [hev.make(10) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for e in evs:
+        step(e)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_step = dt / args.steps * 1e3
+
+    names = ["index_build", "fwd_block_walk", "fwd_merge", None, "bwd_delta", "bwd_dq_walk", "bwd_dq_merge", "bwd_dkv_walk", "bwd_dkv_reduce"]
+    kern = {}
+    for i, nm in enumerate(names):
+        if nm is not None:
+            kern[nm] = sum(hev.ms(e[i], e[i + 1]) for e in evs) / len(evs)
+
+    pairs = attended_pairs(b, hq, n, B, S + 1)
+    flop_unit = 2.0 * d * pairs                        # one d-deep contraction over all attended pairs
+    total_flop = 7 * flop_unit                         # fwd 4dP + bwd 10dP
+    value = total_flop / (ms_step * 1e-3) / 1e12
+    # algorithmic work of each MFMA kernel (recomputation counted once, in the dK/dV walk)
+    kflop = {"fwd_block_walk": 2 * flop_unit, "bwd_dkv_walk": 4 * flop_unit, "bwd_dq_walk": 1 * flop_unit}
+    dom = max(kflop, key=lambda nm: kern[nm])
+    achieved = kflop[dom] / (kern[dom] * 1e-3) / 1e12
+    roofline = dict(bound="mfma", kernel=dom, achieved=round(achieved, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                    frac=round(achieved / MFMA_PEAK_TFLOPS, 4), traffic=None,
+                    step_frac=round(value / MFMA_PEAK_TFLOPS, 4))
+
+    res = dict(metric="NSA selection-attention fwd+bwd TFLOP/s at seq 32k (bf16)", value=round(value, 2), unit="TFLOP/s",
+               n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_step, 4), higher_is_better=True,
+               scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic",
+               config=dict(workload="BASELINE configs[3]: selection attention fwd+bwd, b1 n32768 Hq32 Hkv8 d128 B64, 15 selected + own block",
+                           tokens_per_s=round(b * n / (ms_step * 1e-3), 1), attended_pairs=int(pairs), flop_per_step=total_flop),
+               kernels_ms={k_: round(v_, 4) for k_, v_ in kern.items()},
+               roofline=roofline)
+
+    if not args.no_cpu:
+        torch.set_num_threads(min(16, os.cpu_count() or 1))
+        base, ref = cpu_baseline(cfg, q, k, v, do, idx, msk)
+        res["cpu_baseline"] = base
+        err = (out[:, :, n - ref.shape[2]:].float().cpu() - ref).abs().max().item()
+        res["config"]["max_abs_err_vs_oracle_sample"] = round(err, 5)
+        res["config"]["gpu_over_cpu"] = round(res["config"]["tokens_per_s"] / base["value"], 1)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

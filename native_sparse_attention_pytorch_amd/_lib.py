@@ -39,6 +39,9 @@ def lib():
         L.nsa_select_bwd.argtypes = [C.POINTER(SelectDesc)] + [vp] * 10 + [sz] + [vp] * 4
         L.nsa_selftest_mfma.argtypes = [vp] * 6
         L.nsa_selftest_mfma.restype = C.c_int
+        L.nsa_select_fwd_timed.argtypes = L.nsa_select_fwd.argtypes + [vp, C.c_int]
+        L.nsa_select_bwd_timed.argtypes = L.nsa_select_bwd.argtypes + [vp, C.c_int]
+        L.nsa_select_fwd_timed.restype = L.nsa_select_bwd_timed.restype = C.c_int
         for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):
             getattr(L, name).restype = C.c_int
         _lib = L

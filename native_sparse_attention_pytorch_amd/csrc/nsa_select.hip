@@ -646,6 +646,11 @@ using namespace nsa;
     if (e_ != hipSuccess) return (int)e_;          \
   } while (0)
 
+// optional phase timing: record caller-created events between the kernels of one call
+static inline void mark(void* const* ev, int n, int i, hipStream_t st) {
+  if (ev && i < n && ev[i]) (void)hipEventRecord((hipEvent_t)ev[i], st);
+}
+
 extern "C" int nsa_select_workspace_bytes(const nsa_select_desc* d, size_t* index_bytes, size_t* fwd_bytes, size_t* bwd_bytes) {
   SelPlan P;
   const int rc = make_plan(d, P);
@@ -676,18 +681,22 @@ extern "C" int nsa_select_build_index(const nsa_select_desc* d, const void* idx,
 
 template <int D, int KT>
 static int launch_fwd(const SelPlan& P, const void* q, const void* k, const void* v, const void* idx, const uint8_t* fmask,
-                      const void* iws, void* fws, void* out, float* lse, hipStream_t st) {
+                      const void* iws, void* fws, void* out, float* lse, hipStream_t st, void* const* ev, int nev) {
+  mark(ev, nev, 0, st);
   hipLaunchKernelGGL((sel_fwd_kernel<D, KT>), dim3(P.ub_f, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                      (const char*)iws, (char*)fws);
   NSA_LAUNCH_CHECK();
+  mark(ev, nev, 1, st);
   const long nq = (long)P.bh * P.n;
   hipLaunchKernelGGL((sel_fwd_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)fws, (__bf16*)out, lse);
   NSA_LAUNCH_CHECK();
+  mark(ev, nev, 2, st);
   return 0;
 }
 
-extern "C" int nsa_select_fwd(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* idx, const uint8_t* fmask,
-                              const void* index_ws, void* fwd_ws, size_t fwd_bytes, void* out, float* lse, void* stream) {
+extern "C" int nsa_select_fwd_timed(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* idx, const uint8_t* fmask,
+                                    const void* index_ws, void* fwd_ws, size_t fwd_bytes, void* out, float* lse, void* stream,
+                                    void* const* ev, int nev) {
   SelPlan P;
   const int rc = make_plan(d, P);
   if (rc) return rc;
@@ -695,38 +704,49 @@ extern "C" int nsa_select_fwd(const nsa_select_desc* d, const void* q, const voi
   if (!q || !k || !v || !index_ws || !fwd_ws || !out || !lse) return NSA_E_ARG;
   hipStream_t st = (hipStream_t)stream;
   const int KT = (P.B + 31) / 32;
-  if (P.D == 64 && KT == 1) return launch_fwd<64, 1>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st);
-  if (P.D == 64 && KT == 2) return launch_fwd<64, 2>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st);
-  if (P.D == 128 && KT == 1) return launch_fwd<128, 1>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st);
-  if (P.D == 128 && KT == 2) return launch_fwd<128, 2>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st);
+  if (P.D == 64 && KT == 1) return launch_fwd<64, 1>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st, ev, nev);
+  if (P.D == 64 && KT == 2) return launch_fwd<64, 2>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st, ev, nev);
+  if (P.D == 128 && KT == 1) return launch_fwd<128, 1>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st, ev, nev);
+  if (P.D == 128 && KT == 2) return launch_fwd<128, 2>(P, q, k, v, idx, fmask, index_ws, fwd_ws, out, lse, st, ev, nev);
   return NSA_E_UNSUPPORTED;
+}
+
+extern "C" int nsa_select_fwd(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* idx, const uint8_t* fmask,
+                              const void* index_ws, void* fwd_ws, size_t fwd_bytes, void* out, float* lse, void* stream) {
+  return nsa_select_fwd_timed(d, q, k, v, idx, fmask, index_ws, fwd_ws, fwd_bytes, out, lse, stream, nullptr, 0);
 }
 
 template <int D, int KT>
 static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
-                      const void* idx, const uint8_t* fmask, const void* iws, void* bws, void* dq, void* dk, void* dv, hipStream_t st) {
+                      const void* idx, const uint8_t* fmask, const void* iws, void* bws, void* dq, void* dk, void* dv, hipStream_t st, void* const* ev, int nev) {
+  mark(ev, nev, 0, st);
   float* delta = reinterpret_cast<float*>((char*)bws + P.off_delta);
   const long rows = (long)P.bh * P.g * P.n;
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((sel_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, delta);
   NSA_LAUNCH_CHECK();
+  mark(ev, nev, 1, st);
   hipLaunchKernelGGL((sel_bwd_dq_kernel<D, KT>), dim3(P.ub_f, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                      (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
   NSA_LAUNCH_CHECK();
+  mark(ev, nev, 2, st);
   const long nq = (long)P.bh * P.n;
   hipLaunchKernelGGL((sel_bwd_dq_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)bws, (__bf16*)dq);
   NSA_LAUNCH_CHECK();
+  mark(ev, nev, 3, st);
   hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT>), dim3(P.ub_kv * KT, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                      (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
   NSA_LAUNCH_CHECK();
+  mark(ev, nev, 4, st);
   hipLaunchKernelGGL((sel_bwd_dkv_reduce_kernel<D, KT>), dim3(P.W, P.bh), dim3(256), 0, st, P, (const char*)iws, (const char*)bws, (__bf16*)dk, (__bf16*)dv);
   NSA_LAUNCH_CHECK();
+  mark(ev, nev, 5, st);
   return 0;
 }
 
-extern "C" int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* out, const void* d_out,
-                              const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
-                              void* dq, void* dk, void* dv, void* stream) {
+extern "C" int nsa_select_bwd_timed(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* out, const void* d_out,
+                                    const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
+                                    void* dq, void* dk, void* dv, void* stream, void* const* ev, int nev) {
   SelPlan P;
   const int rc = make_plan(d, P);
   if (rc) return rc;
@@ -734,11 +754,17 @@ extern "C" int nsa_select_bwd(const nsa_select_desc* d, const void* q, const voi
   if (!q || !k || !v || !out || !d_out || !lse || !index_ws || !bwd_ws || !dq || !dk || !dv) return NSA_E_ARG;
   hipStream_t st = (hipStream_t)stream;
   const int KT = (P.B + 31) / 32;
-  if (P.D == 64 && KT == 1) return launch_bwd<64, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st);
-  if (P.D == 64 && KT == 2) return launch_bwd<64, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st);
-  if (P.D == 128 && KT == 1) return launch_bwd<128, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st);
-  if (P.D == 128 && KT == 2) return launch_bwd<128, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st);
+  if (P.D == 64 && KT == 1) return launch_bwd<64, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st, ev, nev);
+  if (P.D == 64 && KT == 2) return launch_bwd<64, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st, ev, nev);
+  if (P.D == 128 && KT == 1) return launch_bwd<128, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st, ev, nev);
+  if (P.D == 128 && KT == 2) return launch_bwd<128, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st, ev, nev);
   return NSA_E_UNSUPPORTED;
+}
+
+extern "C" int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* out, const void* d_out,
+                              const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
+                              void* dq, void* dk, void* dv, void* stream) {
+  return nsa_select_bwd_timed(d, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, bwd_bytes, dq, dk, dv, stream, nullptr, 0);
 }
 
 extern "C" int nsa_abi_version(void) { return 1; }

@@ -196,7 +196,7 @@ def topk_lower_index_first(scores: torch.Tensor, k: int):
 
 # --------------------------------------------------------- selection (fine) attention
 
-def select_attend(q, k, v, idx, fmask, block, causal=True, gates=None, return_lse=False, chunk=256):
+def select_attend(q, k, v, idx, fmask, block, causal=True, gates=None, return_lse=False, chunk=256, q_offset=0):
     """Block-selection attention in gather form.  NSA.py:741-819, test_triton_nsa.py:32-133.
 
     q [b,Hq,n,d]; k,v [b,Hkv,n,d]; idx,fmask [b,Hsel,n,S] with Hsel in (Hkv, Hq).
@@ -205,8 +205,11 @@ def select_attend(q, k, v, idx, fmask, block, causal=True, gates=None, return_ls
     duplicates counted once per slot - plus, when `causal`, its own block under a
     lower-triangular mask.  `gates` [b,Hsel,n,S] multiplies the selected keys (NSA.py:793-797).
     Chunked over queries; mathematically identical to the reference's one-shot gather.
+    `q_offset`: q/idx/fmask hold only the queries at positions q_offset .. q_offset+len-1 of
+    the sequence k/v span (used to time or check a slice of a long sequence).
     """
-    b, hq, n, d = q.shape
+    b, hq, nq, d = q.shape
+    n = k.shape[2]
     hk = k.shape[1]
     hs = idx.shape[1]
     S = idx.shape[-1]
@@ -221,14 +224,14 @@ def select_attend(q, k, v, idx, fmask, block, causal=True, gates=None, return_ls
     kp = F.pad(k, (0, 0, 0, pad)).reshape(b, hk, W, block, d)
     vp = F.pad(v, (0, 0, 0, pad)).reshape(b, hk, W, block, d)
     out = torch.empty_like(q)
-    lse = torch.empty(b, hq, n, dtype=torch.float32)
+    lse = torch.empty(b, hq, nq, dtype=torch.float32)
     tril = torch.ones(block, block, dtype=torch.bool).tril()
     bi = torch.arange(b)[:, None, None, None]
     hi = torch.arange(hk)[None, :, None, None]
-    for s0 in range(0, n, chunk):
-        s1 = min(n, s0 + chunk)
+    for s0 in range(0, nq, chunk):
+        s1 = min(nq, s0 + chunk)
         c = s1 - s0
-        pos = torch.arange(s0, s1)
+        pos = torch.arange(s0, s1) + q_offset
         ci = idx[:, :, s0:s1].long()                                    # [b,hk,c,S]
         cm = fmask[:, :, s0:s1]
         cg = gates[:, :, s0:s1] if gates is not None else None

@@ -173,6 +173,18 @@ def test_select_attend_equals_dense_mask(n, B, S, hq, hk, causal):
     assert torch.allclose(lse, want_lse, atol=1e-5)
 
 
+def test_select_attend_query_slice():
+    gen = torch.Generator().manual_seed(6)
+    b, hq, hk, n, d, B, S = 1, 4, 2, 40, 8, 8, 2
+    q = torch.randn(b, hq, n, d, generator=gen)
+    k = torch.randn(b, hk, n, d, generator=gen)
+    v = torch.randn(b, hk, n, d, generator=gen)
+    idx, msk = random_selection(b, hk, n, B, S, gen)
+    full = O.select_attend(q, k, v, idx, msk, B)
+    part = O.select_attend(q[:, :, 19:33], k, v, idx[:, :, 19:33], msk[:, :, 19:33], B, q_offset=19, chunk=5)
+    assert torch.allclose(part, full[:, :, 19:33], atol=1e-6)
+
+
 def test_select_attend_special_cases():
     gen = torch.Generator().manual_seed(2)
     b, hq, hk, n, d, B = 1, 4, 2, 48, 8, 8
