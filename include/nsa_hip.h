@@ -79,6 +79,62 @@ int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const
                    const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
                    void* dq, void* dk, void* dv, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Interval-masked GQA flash attention: one kernel family for
+ *   mode 0 "band"   - the sliding-window branch.  Replaces LocalAttention(window_size, causal,
+ *                     exact_windowsize, autopad) as called at NSA.py:250-257, 841-850: query i
+ *                     sees keys j with 0 <= i-j <= window (causal) or |i-j| <= window, which is
+ *                     the mask of NSA.py:48-56; k/v have `seq` rows, num_mem = 0;
+ *   mode 1 "stride" - the compressed branch.  Replaces attend(q, ck, cv, cmask, return_sim=True)
+ *                     (NSA.py:153-184, 632-639): k/v hold num_mem memory rows (always visible)
+ *                     followed by num_keys compressed keys; compressed key c is visible to query i
+ *                     iff (c+1)*stride - 1 < i when causal, always otherwise.  With `pool` set the
+ *                     forward also writes the block-importance logits of NSA.py:652-691 to
+ *                     `pooled` (fp32 [batch, kv_heads or heads, seq, nb], nb = num_keys /
+ *                     (sel_block/stride)): mean of the scaled logits over the compressed keys of
+ *                     fine block j and, if `share`, over the group's heads; -inf where the
+ *                     reference's fill values (-finfo.max/10 for an invisible key, -finfo.max for
+ *                     the query's own block when stride != sel_block) make the softmax term zero.
+ * out/lse as for nsa_select_fwd; dq contiguous [batch, heads, seq, d]; dk, dv contiguous
+ * [batch, kv_heads, num_mem + num_keys, d].  bf16 in, fp32 accumulate, bf16 out.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct nsa_dense_desc {
+  int32_t batch, kv_heads, group, seq, num_keys, num_mem, dim_head;
+  int32_t mode, causal, window, stride;
+  int32_t pool, sel_block, share;
+  float scale;
+  int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3], do_stride[3];
+} nsa_dense_desc;
+
+int nsa_dense_workspace_bytes(const nsa_dense_desc* d, size_t* bwd_bytes);
+int nsa_dense_fwd(const nsa_dense_desc* d, const void* q, const void* k, const void* v,
+                  void* out, float* lse, float* pooled, void* stream);
+int nsa_dense_bwd(const nsa_dense_desc* d, const void* q, const void* k, const void* v,
+                  const void* out, const void* d_out, const float* lse, void* bwd_ws, size_t bwd_bytes,
+                  void* dq, void* dk, void* dv, void* stream);
+
+/* Block-importance softmax + per-query top-k.  Replaces NSA.py:693-695 (pad -1e3, softmax, drop
+ * pad), :713 (topk) and :721 (fmask = value > 1e-10).  scores: fp32 [rows, nb]; with
+ * apply_softmax != 0 they are importance logits (-inf = not selectable), otherwise ready
+ * probabilities.  Outputs [rows, k]: idx int32 (descending value, ties to the lower block index -
+ * torch.topk leaves tie order unspecified), vals fp32, fmask uint8.  nb <= 2048, k <= nb. */
+int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k, int32_t apply_softmax,
+             int32_t* idx, float* vals, uint8_t* fmask, void* stream);
+
+/* Fused strategy-gate combine.  Replaces Sigmoid + Rearrange('b n (h s) -> b h n s') + the
+ * stack/einsum + merge_heads of NSA.py:323-327, 854-860.  logits: bf16 contiguous [batch, seq,
+ * 3*heads] (pre-sigmoid output of the gate projection, column 3*h+s, s = compressed, selected,
+ * sliding); c, f, s: bf16 [batch, heads, seq, d] with element strides {batch, head, token};
+ * out / d_out: bf16 contiguous [batch, seq, heads*d]; d_logits like logits; dc, df, ds contiguous
+ * [batch, heads, seq, d]. */
+int nsa_gate_fwd(int32_t batch, int32_t heads, int32_t seq, int32_t dim_head, const void* logits,
+                 const void* c, const int64_t* c_stride, const void* f, const int64_t* f_stride,
+                 const void* s, const int64_t* s_stride, void* out, void* stream);
+int nsa_gate_bwd(int32_t batch, int32_t heads, int32_t seq, int32_t dim_head, const void* logits,
+                 const void* c, const int64_t* c_stride, const void* f, const int64_t* f_stride,
+                 const void* s, const int64_t* s_stride, const void* d_out,
+                 void* d_logits, void* dc, void* df, void* ds, void* stream);
+
 /* Same as nsa_select_fwd / nsa_select_bwd, additionally recording the caller's hipEvent_t
  * handles (created with timing enabled) between the kernels of the call, so that a benchmark
  * can time each kernel on the launch stream.  Events: fwd {start, after block walk, after

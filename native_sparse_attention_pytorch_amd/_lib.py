@@ -20,6 +20,17 @@ class SelectDesc(C.Structure):
     ]
 
 
+class DenseDesc(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("kv_heads", C.c_int32), ("group", C.c_int32), ("seq", C.c_int32),
+        ("num_keys", C.c_int32), ("num_mem", C.c_int32), ("dim_head", C.c_int32),
+        ("mode", C.c_int32), ("causal", C.c_int32), ("window", C.c_int32), ("stride", C.c_int32),
+        ("pool", C.c_int32), ("sel_block", C.c_int32), ("share", C.c_int32), ("scale", C.c_float),
+        ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
+        ("o_stride", C.c_int64 * 3), ("do_stride", C.c_int64 * 3),
+    ]
+
+
 _ERR = {-1: "invalid argument", -2: "shape not supported by the compiled kernels", -3: "workspace too small"}
 
 
@@ -42,6 +53,15 @@ def lib():
         L.nsa_select_fwd_timed.argtypes = L.nsa_select_fwd.argtypes + [vp, C.c_int]
         L.nsa_select_bwd_timed.argtypes = L.nsa_select_bwd.argtypes + [vp, C.c_int]
         L.nsa_select_fwd_timed.restype = L.nsa_select_bwd_timed.restype = C.c_int
+        L.nsa_dense_workspace_bytes.argtypes = [C.POINTER(DenseDesc), C.POINTER(sz)]
+        L.nsa_dense_fwd.argtypes = [C.POINTER(DenseDesc)] + [vp] * 7
+        L.nsa_dense_bwd.argtypes = [C.POINTER(DenseDesc)] + [vp] * 7 + [sz] + [vp] * 4
+        L.nsa_topk.argtypes = [vp, C.c_int64, C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp]
+        i3 = C.POINTER(C.c_int64)
+        L.nsa_gate_fwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp]
+        L.nsa_gate_bwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp, vp, vp, vp, vp]
+        for name in ("nsa_dense_workspace_bytes", "nsa_dense_fwd", "nsa_dense_bwd", "nsa_topk", "nsa_gate_fwd", "nsa_gate_bwd"):
+            getattr(L, name).restype = C.c_int
         for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):
             getattr(L, name).restype = C.c_int
         _lib = L

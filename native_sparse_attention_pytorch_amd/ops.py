@@ -161,3 +161,201 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
                              int(block_size), bool(include_block_causal), float(scale))
     out = out.to(dtype)
     return (out, lse) if return_lse else out
+
+
+# ----------------------------------------------------- sliding / compressed (interval masks)
+
+def _dense_desc(q, k, v, o, do, mode, causal, window, stride, num_mem, pool, sel_block, share, scale) -> _lib.DenseDesc:
+    b, hq, n, d = q.shape
+    hk = k.shape[1]
+    dsc = _lib.DenseDesc()
+    dsc.batch, dsc.kv_heads, dsc.group, dsc.seq = b, hk, hq // hk, n
+    dsc.num_keys, dsc.num_mem, dsc.dim_head = k.shape[2] - num_mem, num_mem, d
+    dsc.mode, dsc.causal, dsc.window, dsc.stride = mode, int(causal), window, stride
+    dsc.pool, dsc.sel_block, dsc.share, dsc.scale = int(pool), sel_block, int(share), scale
+    for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("o_stride", o), ("do_stride", do)):
+        getattr(dsc, name)[:] = list(t.stride()[:3])
+    return dsc
+
+
+@torch.library.custom_op("nsa_amd::dense_fwd", mutates_args=())
+def dense_fwd(q: Tensor, k: Tensor, v: Tensor, mode: int, causal: bool, window: int, stride: int, num_mem: int,
+              pool: bool, sel_block: int, share: bool, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    b, hq, n, d = q.shape
+    hk = k.shape[1]
+    out = torch.empty((b, hq, n, d), dtype=_BF16, device=q.device)
+    lse = torch.empty((b, hq, n), dtype=torch.float32, device=q.device)
+    nb = 0
+    if pool:
+        npf = sel_block // stride
+        nb = (k.shape[2] - num_mem) // npf
+    pool = bool(pool and nb > 0)
+    pooled = torch.empty((b, hk if share else hq, n, nb), dtype=torch.float32, device=q.device)
+    dsc = _dense_desc(q, k, v, out, out, mode, causal, window, stride, num_mem, pool, sel_block, share, scale)
+    _lib.check(_lib.lib().nsa_dense_fwd(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(pooled) if pool else 0, _stream()),
+               "nsa_dense_fwd")
+    return out, lse, pooled
+
+
+@dense_fwd.register_fake
+def _(q, k, v, mode, causal, window, stride, num_mem, pool, sel_block, share, scale):
+    b, hq, n, d = q.shape
+    nb = ((k.shape[2] - num_mem) // (sel_block // stride)) if pool else 0
+    return (q.new_empty((b, hq, n, d)), q.new_empty((b, hq, n), dtype=torch.float32),
+            q.new_empty((b, k.shape[1] if share else hq, n, nb), dtype=torch.float32))
+
+
+@torch.library.custom_op("nsa_amd::dense_bwd", mutates_args=())
+def dense_bwd(q: Tensor, k: Tensor, v: Tensor, out: Tensor, dout: Tensor, lse: Tensor, mode: int, causal: bool, window: int,
+              stride: int, num_mem: int, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+    q, k, v, out = _prep(q), _prep(k), _prep(v), _prep(out)
+    dout = _prep(dout if dout.dtype == _BF16 else dout.to(_BF16))
+    b, hq, n, d = q.shape
+    hk, nk = k.shape[1], k.shape[2]
+    dq = torch.empty((b, hq, n, d), dtype=_BF16, device=q.device)
+    dk = torch.empty((b, hk, nk, d), dtype=_BF16, device=q.device)
+    dv = torch.empty((b, hk, nk, d), dtype=_BF16, device=q.device)
+    dsc = _dense_desc(q, k, v, out, dout, mode, causal, window, stride, num_mem, False, 1, True, scale)
+    wb = C.c_size_t()
+    L = _lib.lib()
+    _lib.check(L.nsa_dense_workspace_bytes(C.byref(dsc), C.byref(wb)), "nsa_dense_workspace_bytes")
+    ws = torch.empty(wb.value, dtype=torch.uint8, device=q.device)
+    _lib.check(L.nsa_dense_bwd(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(ws), wb.value,
+                               _ptr(dq), _ptr(dk), _ptr(dv), _stream()), "nsa_dense_bwd")
+    return dq, dk, dv
+
+
+@dense_bwd.register_fake
+def _(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale):
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
+def _dense_setup(ctx, inputs, output):
+    q, k, v, mode, causal, window, stride, num_mem, pool, sel_block, share, scale = inputs
+    out, lse, _ = output
+    ctx.save_for_backward(q, k, v, out, lse)
+    ctx.args = (mode, causal, window, stride, num_mem, scale)
+
+
+def _dense_backward(ctx, dout, dlse, dpooled):
+    q, k, v, out, lse = ctx.saved_tensors
+    mode, causal, window, stride, num_mem, scale = ctx.args
+    dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale)
+    return (dq, dk, dv) + (None,) * 9
+
+
+dense_fwd.register_autograd(_dense_backward, setup_context=_dense_setup)
+
+
+def sliding_attend(q: Tensor, k: Tensor, v: Tensor, window_size: int, causal: bool = True) -> Tensor:
+    """Sliding-window branch: what `self.sliding_window(sq, sk, sv)` computes at NSA.py:841-850
+    (LocalAttention with exact window, autopad) without materialising the repeated k/v:
+    q [b,Hq,n,d], k/v [b,Hkv,n,d]; query i sees 0 <= i-j <= window_size (causal) or |i-j| <= it."""
+    out, _, _ = dense_fwd(q, k, v, 0, bool(causal), int(window_size), 1, 0, False, 1, True, float(q.shape[-1] ** -0.5))
+    return out
+
+
+def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int, causal: bool,
+                    sel_block: int | None = None, share: bool = True):
+    """Compressed branch: attend(q, [mem; ck], [mem; cv], cmask, return_sim=True) of NSA.py:621-639.
+    Returns (out, importance_logits) where importance_logits [b, Hkv|Hq, n, nb] are the block
+    importance logits of NSA.py:652-691 before the softmax (None if sel_block is None or no full
+    fine block exists): the logits matrix itself is never written to memory."""
+    pool = sel_block is not None
+    out, _, pooled = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), pool, int(sel_block or stride), bool(share),
+                               float(q.shape[-1] ** -0.5))
+    return out, (pooled if pool and pooled.shape[-1] > 0 else None)
+
+
+# ------------------------------------------------------------------------------------ top-k
+
+@torch.library.custom_op("nsa_amd::topk", mutates_args=())
+def topk_op(scores: Tensor, k: int, apply_softmax: bool) -> tuple[Tensor, Tensor, Tensor]:
+    if scores.dtype != torch.float32 or not scores.is_cuda:
+        raise RuntimeError("importance scores must be fp32 device tensors")
+    scores = scores.contiguous()
+    nb = scores.shape[-1]
+    rows = scores.numel() // nb
+    shp = (*scores.shape[:-1], k)
+    idx = torch.empty(shp, dtype=torch.int32, device=scores.device)
+    vals = torch.empty(shp, dtype=torch.float32, device=scores.device)
+    fm = torch.empty(shp, dtype=torch.uint8, device=scores.device)
+    _lib.check(_lib.lib().nsa_topk(_ptr(scores), rows, nb, k, int(apply_softmax), _ptr(idx), _ptr(vals), _ptr(fm), _stream()), "nsa_topk")
+    return idx, vals, fm
+
+
+@topk_op.register_fake
+def _(scores, k, apply_softmax):
+    shp = (*scores.shape[:-1], k)
+    return (scores.new_empty(shp, dtype=torch.int32), scores.new_empty(shp), scores.new_empty(shp, dtype=torch.uint8))
+
+
+def importance_topk(importance_logits: Tensor, num_selected: int):
+    """softmax with the -1e3 pad column (NSA.py:693-695) + topk (NSA.py:713) + `> 1e-10` mask
+    (NSA.py:721).  Returns (values fp32, indices int32, fmask bool), each [..., num_selected]."""
+    idx, vals, fm = topk_op(importance_logits, int(num_selected), True)
+    return vals, idx, fm.view(torch.bool)
+
+
+# --------------------------------------------------------------------------------- gate
+
+def _s3(t: Tensor):
+    return (C.c_int64 * 3)(*t.stride()[:3])
+
+
+@torch.library.custom_op("nsa_amd::gate_fwd", mutates_args=())
+def gate_fwd(logits: Tensor, c: Tensor, f: Tensor, s: Tensor) -> Tensor:
+    c, f, s = _prep(c), _prep(f), _prep(s)
+    logits = logits.contiguous()
+    if logits.dtype != _BF16:
+        raise RuntimeError("gate logits must be bfloat16")
+    b, h, n, d = c.shape
+    out = torch.empty((b, n, h * d), dtype=_BF16, device=c.device)
+    _lib.check(_lib.lib().nsa_gate_fwd(b, h, n, d, _ptr(logits), _ptr(c), _s3(c), _ptr(f), _s3(f), _ptr(s), _s3(s), _ptr(out), _stream()),
+               "nsa_gate_fwd")
+    return out
+
+
+@gate_fwd.register_fake
+def _(logits, c, f, s):
+    b, h, n, d = c.shape
+    return c.new_empty((b, n, h * d))
+
+
+@torch.library.custom_op("nsa_amd::gate_bwd", mutates_args=())
+def gate_bwd(logits: Tensor, c: Tensor, f: Tensor, s: Tensor, dout: Tensor) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    c, f, s = _prep(c), _prep(f), _prep(s)
+    logits = logits.contiguous()
+    dout = dout.contiguous()
+    if dout.dtype != _BF16:
+        dout = dout.to(_BF16)
+    b, h, n, d = c.shape
+    dl = torch.empty_like(logits)
+    dc, df, ds = (torch.empty((b, h, n, d), dtype=_BF16, device=c.device) for _ in range(3))
+    _lib.check(_lib.lib().nsa_gate_bwd(b, h, n, d, _ptr(logits), _ptr(c), _s3(c), _ptr(f), _s3(f), _ptr(s), _s3(s), _ptr(dout),
+                                       _ptr(dl), _ptr(dc), _ptr(df), _ptr(ds), _stream()), "nsa_gate_bwd")
+    return dl, dc, df, ds
+
+
+@gate_bwd.register_fake
+def _(logits, c, f, s, dout):
+    return torch.empty_like(logits), torch.empty_like(c), torch.empty_like(f), torch.empty_like(s)
+
+
+def _gate_setup(ctx, inputs, output):
+    ctx.save_for_backward(*inputs)
+
+
+def _gate_backward(ctx, dout):
+    logits, c, f, s = ctx.saved_tensors
+    return gate_bwd(logits, c, f, s, dout)
+
+
+gate_fwd.register_autograd(_gate_backward, setup_context=_gate_setup)
+
+
+def gate_combine(logits: Tensor, compressed: Tensor, selected: Tensor, sliding: Tensor) -> Tensor:
+    """sigmoid(logits) 'b n (h s) -> b h n s' weighted sum of the three branches, merged to
+    'b n (h d)' (NSA.py:323-327, 854-860).  logits are the pre-sigmoid gate projection."""
+    return gate_fwd(logits.to(_BF16), compressed, selected, sliding)

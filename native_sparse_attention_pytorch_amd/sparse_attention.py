@@ -1,0 +1,219 @@
+"""`SparseAttention` with the reference's constructor, parameter names and forward signature
+(native_sparse_attention_pytorch/native_sparse_attention.py:188-336, 549-557), whose
+training / prefill forward runs the four NSA subsystems as gfx950 HIP kernels:
+
+  compressed attention + block-importance logits   ops.compress_attend     (NSA.py:621-691)
+  importance softmax + top-k + slot mask            ops.importance_topk     (NSA.py:693-721)
+  block-selection attention                         ops.native_sparse_attend(NSA.py:717-819)
+  sliding-window attention                          ops.sliding_attend      (NSA.py:841-850)
+  sigmoid strategy gate + head merge                ops.gate_combine        (NSA.py:854-860)
+
+The dense projections (qkv, compression MLP, gate logits, output) stay `nn.Linear` GEMMs.  There
+is no non-HIP path: CPU tensors, a missing library or an unsupported shape raise.
+"""
+from __future__ import annotations
+
+from copy import deepcopy
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import ops
+
+
+class RotaryEmbedding(nn.Module):
+    """Rotary position embedding with the defaults of the package the reference imports
+    (NSA.py:14, 238): theta 10000, feature pairs (2k, 2k+1), angles in fp32."""
+
+    def __init__(self, dim: int, theta: float = 10000.0):
+        super().__init__()
+        self.freqs = nn.Parameter(1.0 / (theta ** (torch.arange(0, dim, 2).float() / dim)), requires_grad=False)
+
+    def rotate(self, t: torch.Tensor, offset: int = 0) -> torch.Tensor:
+        n = t.shape[-2]
+        pos = torch.arange(offset, offset + n, device=t.device, dtype=torch.float32)
+        ang = torch.outer(pos, self.freqs.float())
+        cos, sin = ang.cos().repeat_interleave(2, dim=-1), ang.sin().repeat_interleave(2, dim=-1)
+        tf = t.float()
+        rot = torch.stack((-tf[..., 1::2], tf[..., 0::2]), dim=-1).flatten(-2)
+        return (tf * cos + rot * sin).to(t.dtype)
+
+    def rotate_queries_with_cached_keys(self, q, k):
+        return self.rotate(q, offset=k.shape[-2] - q.shape[-2]), self.rotate(k)
+
+
+class _FlattenWindow(nn.Module):
+    def forward(self, x):                                   # 'b h w n d -> b h w (n d)'
+        return x.flatten(-2)
+
+
+class _GateLayout(nn.Module):
+    def __init__(self, heads):
+        super().__init__()
+        self.heads = heads
+
+    def forward(self, x):                                   # 'b n (h s) -> b h n s'
+        b, n, _ = x.shape
+        return x.reshape(b, n, self.heads, 3).permute(0, 2, 1, 3)
+
+
+class SparseAttention(nn.Module):
+    def __init__(
+        self,
+        dim,
+        dim_head,
+        heads,
+        sliding_window_size,
+        compress_block_size,
+        compress_block_sliding_stride,
+        selection_block_size,
+        num_selected_blocks,
+        kv_heads=None,
+        num_compressed_mem_kv=1,
+        causal=False,
+        norm=True,
+        use_diff_topk=False,
+        use_triton_kernel=False,
+        query_heads_share_selected_kv=True,
+        compress_mlp: nn.Module | None = None,
+        compress_mlp_expand_factor=1.0,
+        strategy_combine_mlp: nn.Module | None = None,
+    ):
+        super().__init__()
+        kv_heads = heads if kv_heads is None else kv_heads
+        assert kv_heads <= heads and heads % kv_heads == 0
+        self.heads, self.dim_head, self.kv_heads = heads, dim_head, kv_heads
+        self.num_grouped_queries = heads // kv_heads
+        self.scale = dim_head ** -0.5
+        dim_inner, dim_kv_inner = dim_head * heads, dim_head * kv_heads
+        self.norm = nn.RMSNorm(dim) if norm else nn.Identity()
+        self.causal = causal
+        self.rotary_emb = RotaryEmbedding(dim_head)
+        self.qkv_split = (dim_inner, dim_kv_inner, dim_kv_inner)
+        self.to_qkv = nn.Linear(dim, sum(self.qkv_split), bias=False)
+        self.sliding_window_size = sliding_window_size
+
+        self.compress_block_size = compress_block_size
+        self.compress_block_sliding_stride = compress_block_sliding_stride
+        assert compress_block_size >= compress_block_sliding_stride, 'compress_block_size must be >= compress_block_sliding_stride'
+        assert compress_block_sliding_stride > 0, 'compress_block_sliding_stride must be greater than 0'
+        assert selection_block_size % compress_block_sliding_stride == 0, \
+            f'selection_block_size {selection_block_size} must be divisible by compress_block_sliding_stride {compress_block_sliding_stride}'
+
+        assert num_compressed_mem_kv > 0
+        self.num_mem_compress_kv = num_compressed_mem_kv
+        self.compress_mem_kv = nn.Parameter(torch.zeros(2, kv_heads, num_compressed_mem_kv, dim_head))
+        self.k_intrablock_positions = nn.Parameter(torch.zeros(kv_heads, compress_block_size, dim_head))
+        self.v_intrablock_positions = nn.Parameter(torch.zeros(kv_heads, compress_block_size, dim_head))
+
+        if compress_mlp is None:
+            compress_dim = compress_block_size * dim_head
+            hidden = int(compress_mlp_expand_factor * compress_dim)
+            compress_mlp = nn.Sequential(_FlattenWindow(), nn.Linear(compress_dim, hidden), nn.ReLU(), nn.Linear(hidden, dim_head))
+        self.k_compress = deepcopy(compress_mlp)
+        self.v_compress = deepcopy(compress_mlp)
+
+        self.use_diff_topk = use_diff_topk
+        self.query_heads_share_selected_kv = query_heads_share_selected_kv
+        self.selection_block_size = selection_block_size
+        assert num_selected_blocks >= 0
+        if num_selected_blocks == 0:
+            print('`num_selected_blocks` should be set greater than 0, unless if you are ablating it for experimental purposes')
+        self.num_selected_blocks = num_selected_blocks
+        self.use_triton_kernel = use_triton_kernel      # kept for call-site compatibility; the HIP kernels always run
+
+        if strategy_combine_mlp is None:
+            strategy_combine_mlp = nn.Linear(dim, 3 * heads)
+            nn.init.zeros_(strategy_combine_mlp.weight)
+            strategy_combine_mlp.bias.data.copy_(torch.tensor([-2., -2., 2.] * heads))
+        self.to_strategy_combine = nn.Sequential(strategy_combine_mlp, nn.Sigmoid(), _GateLayout(heads))
+        self.combine_heads = nn.Linear(dim_inner, dim, bias=False)
+
+    # ------------------------------------------------------------------------------ pieces
+
+    def _split_heads(self, t):
+        b, n, hd = t.shape
+        return t.view(b, n, hd // self.dim_head, self.dim_head).permute(0, 2, 1, 3)
+
+    def _compress_windows(self, t):
+        """'b h n d' (n divisible by the stride) -> 'b h w cbs d'; window w = tokens
+        [(w+1)*stride - cbs, (w+1)*stride), zeros left of token 0 (NSA.py:270-275)."""
+        cbs, st = self.compress_block_size, self.compress_block_sliding_stride
+        b, h, L, d = t.shape
+        if L == 0:
+            return t.reshape(b, h, 0, cbs, d)
+        return F.pad(t, (0, 0, cbs - st, 0)).unfold(2, cbs, st).permute(0, 1, 2, 4, 3)
+
+    def forward_inference(self, inp, cache, return_cache=True):
+        raise NotImplementedError("single-token decode with caches (NSA.py:338-547) is outside the accelerated hot path")
+
+    def forward(self, inp, cache=None, disable_triton_kernel=False, sliding_window_flex_mask=None,
+                fine_selection_flex_mask=None, return_cache=False):
+        if cache is not None:
+            assert inp.shape[1] == 1, 'input must be single tokens if inferencing with cache key values'
+            return self.forward_inference(inp, cache, return_cache=return_cache)
+        assert not (not self.causal and return_cache)
+        if sliding_window_flex_mask is not None or fine_selection_flex_mask is not None:
+            raise NotImplementedError("flex-attention masks are a different backend; the HIP kernels implement the same masks directly")
+        if self.use_diff_topk:
+            raise NotImplementedError("use_diff_topk (gradient through the selection gates) is not implemented in the HIP path")
+        if not inp.is_cuda:
+            raise RuntimeError("SparseAttention runs on the GPU only (HIP kernels, no CPU fallback)")
+
+        b, n, _ = inp.shape
+        st, cbs, B = self.compress_block_sliding_stride, self.compress_block_size, self.selection_block_size
+        M, G = self.num_mem_compress_kv, self.num_grouped_queries
+        bf16 = torch.bfloat16
+
+        x = self.norm(inp)
+        q, k, v = self.to_qkv(x).split(self.qkv_split, dim=-1)
+        q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
+
+        # compressed keys / values from the un-rotated k, v
+        L = (n // st) * st
+        kw, vw = self._compress_windows(k[..., :L, :]), self._compress_windows(v[..., :L, :])
+        if kw.numel() > 0:
+            kw = kw + self.k_intrablock_positions[None, :, None]
+            vw = vw + self.v_intrablock_positions[None, :, None]
+        ck0, cv0 = self.k_compress(kw), self.v_compress(vw)
+        mem_k, mem_v = self.compress_mem_kv[0].to(ck0.dtype), self.compress_mem_kv[1].to(cv0.dtype)
+        ck = torch.cat((mem_k[None].expand(b, -1, -1, -1), ck0), dim=-2)
+        cv = torch.cat((mem_v[None].expand(b, -1, -1, -1), cv0), dim=-2)
+        nc = ck0.shape[-2]
+
+        want_sel = self.num_selected_blocks > 0 and nc > 0
+        share = self.query_heads_share_selected_kv
+        c_out, imp = ops.compress_attend(q.to(bf16), ck.to(bf16), cv.to(bf16), M, st, self.causal,
+                                         sel_block=B if want_sel else None, share=share)
+
+        rq, rk = self.rotary_emb.rotate_queries_with_cached_keys(q, k)
+        rq16, rk16, v16 = rq.to(bf16), rk.to(bf16), v.to(bf16)
+
+        num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
+        if num_sel > 0:
+            _, idx, fmask = ops.importance_topk(imp, num_sel)
+            f_out = ops.native_sparse_attend(rq16, rk16, v16, B, idx, fmask, include_block_causal=self.causal)
+        elif self.causal:
+            # nothing selectable: block-diagonal causal attention (NSA.py:821-837)
+            idx = torch.zeros((b, self.kv_heads, n, 0), dtype=torch.int32, device=inp.device)
+            f_out = ops.native_sparse_attend(rq16, rk16, v16, B, idx, idx.bool(), include_block_causal=True)
+        else:
+            # non-causal: every query attends its whole own block
+            own = (torch.arange(n, device=inp.device, dtype=torch.int32) // B)[None, None, :, None].expand(b, self.kv_heads, n, 1)
+            f_out = ops.native_sparse_attend(rq16, rk16, v16, B, own.contiguous(), torch.ones_like(own, dtype=torch.bool),
+                                             include_block_causal=False)
+
+        s_out = ops.sliding_attend(rq16, rk16, v16, self.sliding_window_size, causal=self.causal)
+
+        logits = self.to_strategy_combine[0](x)
+        merged = ops.gate_combine(logits, c_out, f_out, s_out)
+        out = self.combine_heads(merged.to(x.dtype))
+
+        if not return_cache:
+            return out
+        co = cbs - st
+        run_k, run_v = k, v
+        if co > 0:
+            run_k, run_v = F.pad(run_k, (0, 0, co, 0)), F.pad(run_v, (0, 0, co, 0))
+        return out, ((rk, v), ((ck0, cv0), (run_k[..., L:, :], run_v[..., L:, :])))

@@ -166,9 +166,10 @@ class _FlattenWindow(nn.Module):
 
 # ------------------------------------------------------------ importance scores + top-k
 
-def importance_from_csim(csim, num_mem, g, share, stride, block, causal_fill_dtype=None):
-    """NSA.py:652-695.  csim [b,Hq,n,num_mem+Nc] = scaled, masked compressed logits.
-    Returns softmaxed importance [b,H_sel,n,nb] (nb may be 0)."""
+def importance_logits(csim, num_mem, g, share, stride, block):
+    """NSA.py:652-691: block-importance logits before the padded softmax.  csim [b,Hq,n,num_mem+Nc]
+    = scaled, masked compressed logits.  Returns [b,H_sel,n,nb] (nb may be 0); invisible keys carry
+    the reference's fill (-finfo.max/10, averaged), the query's own block -finfo.max."""
     imp = csim[..., num_mem:]
     b, hq, n, nc = imp.shape
     if share:
@@ -182,9 +183,17 @@ def importance_from_csim(csim, num_mem, g, share, stride, block, causal_fill_dty
             nb = imp.shape[-1]
             own = (torch.arange(n)[:, None] // block) == torch.arange(nb)[None, :]
             imp = imp.masked_fill(own, _neg_max(csim))
-    imp = F.pad(imp, (1, 0), value=-1e3)
-    imp = imp.softmax(dim=-1)
-    return imp[..., 1:]
+    return imp
+
+
+def importance_softmax(logits):
+    """NSA.py:693-695: left-pad one column of -1e3, softmax, drop the column."""
+    imp = F.pad(logits, (1, 0), value=-1e3)
+    return imp.softmax(dim=-1)[..., 1:]
+
+
+def importance_from_csim(csim, num_mem, g, share, stride, block):
+    return importance_softmax(importance_logits(csim, num_mem, g, share, stride, block))
 
 
 def topk_lower_index_first(scores: torch.Tensor, k: int):
@@ -394,7 +403,9 @@ class SparseAttentionOracle(nn.Module):
             return None
         return topk_lower_index_first(imp, num_sel)
 
-    def forward(self, inp, return_parts=False):
+    def forward(self, inp, return_parts=False, selection_override=None):
+        """selection_override = (idx, fmask) replaces the module's own top-k result (used to
+        compare implementations under an identical discrete selection)."""
         b, n, _ = inp.shape
         st, B = self.compress_block_sliding_stride, self.selection_block_size
         x, q, k, v = self.project(inp)
@@ -404,7 +415,11 @@ class SparseAttentionOracle(nn.Module):
         c_out, csim = attend(q, ck, cv, mask=cmask, return_sim=True)
         rq, rk = self.rotary_emb.rotate_queries_with_cached_keys(q, k)
         sel = self.select(csim)
-        if sel is not None:
+        if selection_override is not None:
+            idx, live = selection_override
+            vals = None
+            f_out = select_attend(rq, rk, v, idx, live, B, causal=self.causal)
+        elif sel is not None:
             vals, idx = sel
             gates = (vals + (1.0 - vals).detach()) if self.use_diff_topk else None
             f_out = select_attend(rq, rk, v, idx, vals > 1e-10, B, causal=self.causal, gates=gates)
