@@ -6,7 +6,7 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libnsa_hip.so")
+LIB_PATH = os.environ.get("NSA_HIP_LIB") or os.path.join(HERE, "libnsa_hip.so")    # NSA_HIP_LIB: load another build of the same ABI
 
 _lib = None
 

@@ -66,6 +66,32 @@ __device__ __forceinline__ void make_ident(int lane, bf16x8& lo, bf16x8& hi) {
   }
 }
 
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short shortx4;
+
+// Transposed MFMA operand from a row-major bf16 tile X in LDS (row stride RS elements, RS*2
+// bytes = 32 mod 128 keeps the reads conflict-free): returns, for lane (m = lane % 32,
+// h = lane / 32), the 8 values X[row0 + 8*(e/4) + 4h + e%4][col0 + m], e = 0..7 - i.e. an
+// A/B operand whose lane index runs over 32 columns of X and whose k index runs over 16 rows
+// of X in the same order in which a 32x32 MFMA result holds its rows (registers 8u .. 8u+7).
+// Uses the gfx950 LDS transpose load: in every group of 16 lanes, lane ll receives element
+// ll % 4 of the four 8-byte rows addressed by lanes 4e + ll / 4 (e = 0..3) of its group.
+__device__ __forceinline__ bf16x8 lds_transposed_operand(const __bf16* X, int RS, int row0, int col0, int lane) {
+  const int ll = lane & 15, e = ll >> 2, qq = ll & 3, mh = (lane >> 4) & 1, h = lane >> 5;
+  const __bf16* p0 = X + (row0 + 4 * h + e) * RS + col0 + 16 * mh + 4 * qq;
+  typedef shortx4 __attribute__((address_space(3))) * lds_ptr;
+  const shortx4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
+  const shortx4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + 8 * RS));
+  typedef __attribute__((__vector_size__(8 * sizeof(short)))) short shortx8;
+  shortx8 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { r[i] = a[i]; r[4 + i] = b[i]; }
+  return __builtin_bit_cast(bf16x8, r);
+}
+
+// s_waitcnt vmcnt(0) (expcnt / lgkmcnt left at their maxima): all outstanding global loads
+// and stores of this wave have completed.
+__device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

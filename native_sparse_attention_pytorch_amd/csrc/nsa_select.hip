@@ -52,9 +52,8 @@ __global__ __launch_bounds__(256) void sel_count_kernel(const SelPlan P, const v
   for (int j = tid; j < P.W; j += 256) cnt[j] = hist[j];
 }
 
-// exclusive scans: over chunks per block (in place in cnt), over blocks (blk_off), and the two
-// work-unit tables (a unit = up to chunk_f / chunk_kv pairs of one block's virtual list, which
-// is the block's own queries, if causal, followed by the queries that selected it)
+// exclusive scan over the counting chunks of every block (in place in cnt) and over blocks
+// (blk_off)
 __global__ __launch_bounds__(256) void sel_scan_kernel(const SelPlan P, char* iws) {
   extern __shared__ int tot[];
   const int bh = blockIdx.x, tid = threadIdx.x;
@@ -71,18 +70,57 @@ __global__ __launch_bounds__(256) void sel_scan_kernel(const SelPlan P, char* iw
   __syncthreads();
   if (tid == 0) {
     int* blk = reinterpret_cast<int*>(iws + P.off_blk) + (size_t)bh * (P.W + 1);
-    int* uf = reinterpret_cast<int*>(iws + P.off_unitf) + (size_t)bh * (P.W + 1);
-    int* uk = reinterpret_cast<int*>(iws + P.off_unitkv) + (size_t)bh * (P.W + 1);
-    int acc = 0, af = 0, ak = 0;
-    for (int j = 0; j < P.W; ++j) {
-      blk[j] = acc; uf[j] = af; uk[j] = ak;
-      const int own = P.causal ? min(P.B, P.n - j * P.B) : 0;
-      const int L = own + tot[j];
-      acc += tot[j];
-      af += (L + P.chunk_f - 1) / P.chunk_f;
-      ak += (L + P.chunk_kv - 1) / P.chunk_kv;
-    }
-    blk[P.W] = acc; uf[P.W] = af; uk[P.W] = ak;
+    int acc = 0;
+    for (int j = 0; j < P.W; ++j) { blk[j] = acc; acc += tot[j]; }
+    blk[P.W] = acc;
+  }
+}
+
+// pairs of cell (phase p, block j) of table t: own queries (if the block lies in the phase and
+// the call is causal) followed by the block's list entries whose query is in the phase
+struct CellInfo { int own, first, count; };
+
+__device__ __forceinline__ CellInfo cell_info(const SelPlan& P, const char* iws, int bh, int t, int p, int j) {
+  const int* cnt = reinterpret_cast<const int*>(iws + P.off_cnt) + (size_t)bh * P.nch * P.W;
+  const int* blk = reinterpret_cast<const int*>(iws + P.off_blk) + (size_t)bh * (P.W + 1);
+  const int totj = blk[j + 1] - blk[j];
+  const int cpp = P.phase[t] / kCountChunk;                 // counting chunks per phase
+  const int c0 = p * cpp, c1 = c0 + cpp;
+  const int s0 = c0 < P.nch ? cnt[(size_t)c0 * P.W + j] : totj;
+  const int s1 = c1 < P.nch ? cnt[(size_t)c1 * P.W + j] : totj;
+  CellInfo ci;
+  ci.first = blk[j] + s0;
+  ci.count = s1 - s0;
+  ci.own = (P.causal && (j * P.B) / P.phase[t] == p) ? min(P.B, P.n - j * P.B) : 0;
+  return ci;
+}
+
+// unit_off[t][bh][cell] = exclusive prefix sum of ceil(pairs(cell) / chunk[t]), cells phase-major
+__global__ __launch_bounds__(256) void sel_units_kernel(const SelPlan P, char* iws) {
+  __shared__ int part[256];
+  const int bh = blockIdx.x, t = blockIdx.y, tid = threadIdx.x;
+  const int cells = P.np[t] * P.W;
+  int* uo = reinterpret_cast<int*>(iws + P.off_unit[t]) + (size_t)bh * (cells + 1);
+  const int per = (cells + 255) / 256;
+  const int lo = min(cells, tid * per), hi = min(cells, lo + per);
+  int sum = 0;
+  for (int c = lo; c < hi; ++c) {
+    const CellInfo ci = cell_info(P, iws, bh, t, c / P.W, c % P.W);
+    sum += (ci.own + ci.count + P.chunk[t] - 1) / P.chunk[t];
+  }
+  part[tid] = sum;
+  __syncthreads();
+  if (tid == 0) {
+    int acc = 0;
+    for (int k = 0; k < 256; ++k) { const int v = part[k]; part[k] = acc; acc += v; }
+    uo[cells] = acc;
+  }
+  __syncthreads();
+  int acc = part[tid];
+  for (int c = lo; c < hi; ++c) {
+    const CellInfo ci = cell_info(P, iws, bh, t, c / P.W, c % P.W);
+    uo[c] = acc;
+    acc += (ci.own + ci.count + P.chunk[t] - 1) / P.chunk[t];
   }
 }
 
@@ -132,25 +170,48 @@ struct UnitInfo {
   int j, own, lst0, v0, v1;
 };
 
-// unit -> (block j, range [v0, v1) of its virtual list).  Returns false for padding units.
-__device__ __forceinline__ bool locate_unit(const SelPlan& P, const char* iws, size_t off_unit, int chunk, int bh, int u, UnitInfo& ui) {
-  const int* unit_off = reinterpret_cast<const int*>(iws + off_unit) + (size_t)bh * (P.W + 1);
-  if (u >= unit_off[P.W]) return false;
-  int lo = 0, hi = P.W - 1;
-  while (lo < hi) {
+// unit u of table t -> (block j, range [v0, v1) of the cell's virtual list: `own` own-block
+// positions first, then list[lst0 ...]).  Returns false for padding units.
+__device__ __forceinline__ bool locate_unit(const SelPlan& P, const char* iws, int t, int bh, int u, UnitInfo& ui) {
+  const int cells = P.np[t] * P.W;
+  const int* unit_off = reinterpret_cast<const int*>(iws + P.off_unit[t]) + (size_t)bh * (cells + 1);
+  if (u >= unit_off[cells]) return false;
+  int lo = 0, hi = cells - 1;
+  while (lo < hi) {                       // last cell with unit_off[cell] <= u (empty cells own no unit)
     const int mid = (lo + hi + 1) >> 1;
     if (unit_off[mid] <= u) lo = mid; else hi = mid - 1;
   }
-  // blocks with an empty list own no unit: unit_off[lo] == unit_off[lo+1]; the search lands on
-  // the last j with unit_off[j] <= u, which is the one whose range contains u
-  const int* blk = reinterpret_cast<const int*>(iws + P.off_blk) + (size_t)bh * (P.W + 1);
-  ui.j = lo;
-  ui.own = P.causal ? min(P.B, P.n - lo * P.B) : 0;
-  ui.lst0 = blk[lo];
-  const int L = ui.own + (blk[lo + 1] - blk[lo]);
-  ui.v0 = (u - unit_off[lo]) * chunk;
-  ui.v1 = min(L, ui.v0 + chunk);
+  const int p = lo / P.W, j = lo % P.W;
+  const CellInfo ci = cell_info(P, iws, bh, t, p, j);
+  ui.j = j;
+  ui.own = ci.own;
+  ui.lst0 = ci.first;                     // index into the per-(batch, head) list
+  const int L = ci.own + ci.count;
+  ui.v0 = (u - unit_off[lo]) * P.chunk[t];
+  ui.v1 = min(L, ui.v0 + P.chunk[t]);
   return ui.v0 < ui.v1;
+}
+
+// Work-group id -> (batch*kv head, unit) such that all units of one head run, in table order,
+// on as few XCDs as possible (consecutive work-group ids go round-robin over the 8 XCDs), so
+// that the Q rows of a query phase are fetched into one L2 only.
+__device__ __forceinline__ bool xcd_map(const SelPlan& P, int t, int& bh, int& u) {
+  const int w = blockIdx.x, x = w & 7, tt = w >> 3;
+  if (P.bh >= 8) {
+    bh = x + 8 * (tt / P.ub[t]);
+    u = tt % P.ub[t];
+    return bh < P.bh;
+  }
+  bh = x % P.bh;
+  const int sub = x / P.bh, nsub = (8 - bh + P.bh - 1) / P.bh;
+  u = tt * nsub + sub;
+  return u < P.ub[t];
+}
+
+static inline unsigned xcd_grid(const SelPlan& P, int t) {
+  if (P.bh >= 8) return 8u * (unsigned)P.ub[t] * (unsigned)((P.bh + 7) / 8);
+  const int nsub_min = 8 / P.bh;
+  return 8u * (unsigned)((P.ub[t] + nsub_min - 1) / nsub_min);
 }
 
 struct RowInfo {
@@ -158,20 +219,102 @@ struct RowInfo {
   bool valid;
 };
 
-// Row `nrow` (0..31) of the 32-row tile starting at virtual position vt.
-__device__ __forceinline__ RowInfo locate_row(const SelPlan& P, const int* list, const UnitInfo& ui, int vt, int nrow) {
-  RowInfo r;
+// Row `nrow` (0..31) of the 32-row tile starting at virtual position vt, in two stages so that
+// the list entry (a dependent global load) is fetched tiles ahead of its use.  The fetch is
+// branch-free (it always loads, from a clamped index) so that no wait is forced at a join.
+struct RawEntry {
+  int raw, pvc;
+  bool valid;
+};
+
+__device__ __forceinline__ RawEntry fetch_entry(const SelPlan& P, const int* list, const UnitInfo& ui, int vt, int nrow) {
+  RawEntry e;
   const int pv = vt + (nrow >> P.lg);
-  r.valid = pv < ui.v1;
-  const int pvc = r.valid ? pv : vt;
+  e.valid = pv < ui.v1;
+  e.pvc = min(pv, ui.v1 - 1);
+  long li = (long)ui.lst0 + max(e.pvc - ui.own, 0);
+  li = li < P.list_cap ? li : P.list_cap - 1;
+  e.raw = list[li];
+  return e;
+}
+
+__device__ __forceinline__ RowInfo decode_entry(const SelPlan& P, const UnitInfo& ui, const RawEntry& e, int nrow) {
+  RowInfo r;
+  r.valid = e.valid;
   r.g = nrow & (P.g - 1);
-  if (pvc < ui.own) {
-    r.i = ui.j * P.B + pvc; r.slot = P.S; r.lim = pvc;
-  } else {
-    const int e = list[ui.lst0 + pvc - ui.own];
-    r.i = e / P.SP; r.slot = e - r.i * P.SP; r.lim = P.B - 1;
-  }
+  const bool own = e.pvc < ui.own;
+  const int qi = e.raw / P.SP;
+  r.i = own ? ui.j * P.B + e.pvc : qi;
+  r.slot = own ? P.S : e.raw - qi * P.SP;
+  r.lim = own ? e.pvc : P.B - 1;
   return r;
+}
+
+// Coalesced gather of a 32-row tile: row rr = (pair rr >> lg of the tile, head rr & (G-1)).
+// Each load instruction covers 64 / (D/8) whole rows (16 bytes per lane, consecutive lanes
+// consecutive addresses), which the texture path handles several times faster than 32 rows x
+// 32 bytes.  `my_i` is the query index of row (lane % 32); `base` points at the first head of
+// the kv group.  The data goes to registers first (so that it can be in flight during the
+// previous tile's compute) and is committed to a row-major LDS tile later.
+template <int D>
+__device__ __forceinline__ void issue_tile_loads(bf16x8 (&raw)[D / 16], const __bf16* __restrict__ base, long s_head, long s_tok, int my_i,
+                                                 int gmask, int lane) {
+  constexpr int CPR = D / 8, RPI = 64 / CPR, NT = 32 / RPI;
+  static_assert(NT == D / 16, "tile load count");
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int rr = t * RPI + lane / CPR, c = lane % CPR;
+    const int i = __shfl(my_i, rr, 64);
+    raw[t] = load8(base + (long)(rr & gmask) * s_head + (long)i * s_tok + 8 * c);
+  }
+}
+
+template <int D>
+__device__ __forceinline__ void commit_tile(const bf16x8 (&raw)[D / 16], __bf16* tile_s, int RS, int lane) {
+  constexpr int CPR = D / 8, RPI = 64 / CPR, NT = 32 / RPI;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int rr = t * RPI + lane / CPR, c = lane % CPR;
+    *reinterpret_cast<bf16x8*>(tile_s + rr * RS + 8 * c) = raw[t];
+  }
+}
+
+// MFMA operand (lane <-> row n_, k <-> 8 consecutive features) of k-step ks from a row-major tile
+__device__ __forceinline__ bf16x8 lds_row_operand(const __bf16* tile_s, int RS, int ks, int lane) {
+  return *reinterpret_cast<const bf16x8*>(tile_s + (lane & 31) * RS + 16 * ks + 8 * (lane >> 5));
+}
+
+// Write a wave's 32-row x D accumulator tile (transposed MFMA layout: lane <-> row n_,
+// register (dt, a, b) <-> feature 32dt + 8a + 4h + b) as bf16 rows through LDS, so that every
+// global store instruction covers whole 2*D-byte rows (16 bytes per lane, consecutive lanes
+// consecutive addresses) instead of 8-byte pieces of 32 different rows.  `row` is this lane's
+// destination row index into dst (rows of D elements); `scale` multiplies the values.
+// One wave per work-group: LDS operations of a wave execute in order, the barriers only keep the
+// compiler from reordering.
+template <int D>
+__device__ __forceinline__ void store_tile_rows(const floatx16 (&acc)[D / 32], float scale, size_t row, __bf16* __restrict__ dst,
+                                                __bf16* tile_s, size_t* row_s, int lane) {
+  constexpr int DT = D / 32, RS = D + 8;          // padded LDS row stride in elements
+  constexpr int CPR = D / 8, RPI = 64 / CPR;      // 16-byte chunks per row, rows per store instruction
+  const int n_ = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      bf16x4 r;
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) r[bb] = (__bf16)(acc[dt][4 * a + bb] * scale);
+      *reinterpret_cast<bf16x4*>(tile_s + n_ * RS + 32 * dt + 8 * a + 4 * h) = r;
+    }
+  if (h == 0) row_s[n_] = row;
+  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < 32 / RPI; ++t) {
+    const int rr = t * RPI + lane / CPR, c = lane % CPR;
+    const bf16x8 v = *reinterpret_cast<const bf16x8*>(tile_s + rr * RS + 8 * c);
+    *reinterpret_cast<bf16x8*>(dst + row_s[rr] * D + 8 * c) = v;
+  }
+  __syncthreads();
 }
 
 // ------------------------------------------------------------------------------- forward
@@ -179,11 +322,15 @@ __device__ __forceinline__ RowInfo locate_row(const SelPlan& P, const int* list,
 template <int D, int KT>
 __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                      const __bf16* __restrict__ v, const char* __restrict__ iws, char* __restrict__ fws) {
-  constexpr int KS = D / 16, DT = D / 32;
+  constexpr int KS = D / 16, DT = D / 32, TBL = 0;
+  __shared__ __align__(16) __bf16 tile_s[32 * (D + 8)];
+  __shared__ size_t row_s[32];
   const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
-  const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
+  int bh, u;
+  if (!xcd_map(P, TBL, bh, u)) return;
+  const int b = bh / P.hkv, hk = bh % P.hkv;
   UnitInfo ui;
-  if (!locate_unit(P, iws, P.off_unitf, P.chunk_f, bh, blockIdx.x, ui)) return;
+  if (!locate_unit(P, iws, TBL, bh, u, ui)) return;
   const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
 
   bf16x8 Kf[KT][KS];
@@ -218,12 +365,32 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
   const float sc = P.scale * kLog2e;
   const int ppt = 32 >> P.lg;
 
-  for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
-    const RowInfo r = locate_row(P, list, ui, vt, n_);
+  // software pipeline: list entries two tiles ahead, Q operands one tile ahead
+  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + ppt, n_);
+  RowInfo r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0, n_), n_);
+  bf16x8 Qf[KS];
+  {
     const __bf16* qp = q + b * P.sq[0] + (long)(hk * P.g + r.g) * P.sq[1] + (long)r.i * P.sq[2] + 8 * h;
-    bf16x8 Qf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) Qf[ks] = load8(qp + 16 * ks);
+  }
+
+  wait_all_loads();        // enter the loop with nothing pending, so the loop itself only waits for what it needs
+  for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
+    // issue the next tile's operand loads and the entry fetch of the tile after it first
+    const RowInfo rn = decode_entry(P, ui, e_n, n_);
+    bf16x8 Qn[KS];
+    {
+#ifdef NSA_EXP_NOGATHER
+      const __bf16* qp = q + b * P.sq[0] + (long)(hk * P.g + rn.g) * P.sq[1] + (long)(rn.i & 63) * P.sq[2] + 8 * h;
+#else
+      const __bf16* qp = q + b * P.sq[0] + (long)(hk * P.g + rn.g) * P.sq[1] + (long)rn.i * P.sq[2] + 8 * h;
+#endif
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) Qn[ks] = load8(qp + 16 * ks);
+    }
+    const RawEntry e_nn = fetch_entry(P, list, ui, vt + 2 * ppt, n_);
+    __builtin_amdgcn_sched_barrier(0);
 
     floatx16 Sa[KT];
 #pragma unroll
@@ -267,17 +434,17 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
         for (int dt = 0; dt < DT; ++dt) Oa[dt] = mfma32(VT[dt][kt][u2], Pf, Oa[dt]);
       }
 
-    if (r.valid) {
+    {
+      // padding rows write to a spare row at the end of the buffers: the stores stay
+      // unconditional, so the wait for the next tile's loads never has to cover them
       const float inv = 1.0f / l;
-      const size_t row = (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g;
-      __bf16* op = opart + row * D + 4 * h;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-          store4_bf16(op + 32 * dt + 8 * a, Oa[dt][4 * a] * inv, Oa[dt][4 * a + 1] * inv, Oa[dt][4 * a + 2] * inv, Oa[dt][4 * a + 3] * inv);
+      const size_t row = r.valid ? (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g : P.prow;
+      store_tile_rows<D>(Oa, inv, row, opart, tile_s, row_s, lane);
       if (h == 0) lsepart[row] = (mx + fast_log2(l)) * kLn2;
     }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) Qf[ks] = Qn[ks];
+    r = rn; e_n = e_nn;
   }
 }
 
@@ -374,11 +541,15 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
                                                         const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
                                                         const float* __restrict__ lse, const float* __restrict__ delta,
                                                         const char* __restrict__ iws, char* __restrict__ bws) {
-  constexpr int KS = D / 16, DT = D / 32;
+  constexpr int KS = D / 16, DT = D / 32, TBL = 1;
+  __shared__ __align__(16) __bf16 tile_s[32 * (D + 8)];
+  __shared__ size_t row_s[32];
   const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
-  const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
+  int bh, u;
+  if (!xcd_map(P, TBL, bh, u)) return;
+  const int b = bh / P.hkv, hk = bh % P.hkv;
   UnitInfo ui;
-  if (!locate_unit(P, iws, P.off_unitf, P.chunk_f, bh, blockIdx.x, ui)) return;
+  if (!locate_unit(P, iws, TBL, bh, u, ui)) return;
   const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
 
   bf16x8 Kf[KT][KS], Vf[KT][KS];
@@ -414,17 +585,38 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
   const int ppt = 32 >> P.lg;
   const int HQ = P.hkv * P.g;
 
-  for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
-    const RowInfo r = locate_row(P, list, ui, vt, n_);
+  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + ppt, n_);
+  RowInfo r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0, n_), n_);
+  bf16x8 Qf[KS], Gf[KS];
+  float lse_r, del_r;
+  {
     const int hq = hk * P.g + r.g;
     const __bf16* qp = q + b * P.sq[0] + (long)hq * P.sq[1] + (long)r.i * P.sq[2] + 8 * h;
     const __bf16* dop = dout + b * P.so[0] + (long)hq * P.so[1] + (long)r.i * P.so[2] + 8 * h;
-    bf16x8 Qf[KS], Gf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) { Qf[ks] = load8(qp + 16 * ks); Gf[ks] = load8(dop + 16 * ks); }
     const size_t srow = ((size_t)b * HQ + hq) * P.n + r.i;
-    const float lse_r = lse[srow] * kLog2e;
-    const float del_r = delta[srow];
+    lse_r = lse[srow] * kLog2e;
+    del_r = delta[srow];
+  }
+
+  wait_all_loads();        // enter the loop with nothing pending, so the loop itself only waits for what it needs
+  for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
+    const RowInfo rn = decode_entry(P, ui, e_n, n_);
+    bf16x8 Qn[KS], Gn[KS];
+    float lse_n, del_n;
+    {
+      const int hqn = hk * P.g + rn.g;
+      const __bf16* qp = q + b * P.sq[0] + (long)hqn * P.sq[1] + (long)rn.i * P.sq[2] + 8 * h;
+      const __bf16* dop = dout + b * P.so[0] + (long)hqn * P.so[1] + (long)rn.i * P.so[2] + 8 * h;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) { Qn[ks] = load8(qp + 16 * ks); Gn[ks] = load8(dop + 16 * ks); }
+      const size_t srown = ((size_t)b * HQ + hqn) * P.n + rn.i;
+      lse_n = lse[srown] * kLog2e;
+      del_n = delta[srown];
+    }
+    const RawEntry e_nn = fetch_entry(P, list, ui, vt + 2 * ppt, n_);
+    __builtin_amdgcn_sched_barrier(0);
 
     floatx16 Sa[KT], Pa[KT];
 #pragma unroll
@@ -455,16 +647,14 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) Qa[dt] = mfma32(KTf[dt][kt][u2], Sf, Qa[dt]);
       }
-    if (r.valid) {
-      const size_t row = (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g;
-      __bf16* op = dqpart + row * D + 4 * h;
-      const float s = P.scale;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-          store4_bf16(op + 32 * dt + 8 * a, Qa[dt][4 * a] * s, Qa[dt][4 * a + 1] * s, Qa[dt][4 * a + 2] * s, Qa[dt][4 * a + 3] * s);
+    {
+      const size_t row = r.valid ? (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g : P.prow;
+      store_tile_rows<D>(Qa, P.scale, row, dqpart, tile_s, row_s, lane);
     }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) { Qf[ks] = Qn[ks]; Gf[ks] = Gn[ks]; }
+    lse_r = lse_n; del_r = del_n;
+    r = rn; e_n = e_nn;
   }
 }
 
@@ -499,28 +689,34 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
   }
 }
 
-// dK/dV of one 32-key tile of one block, accumulated over a chunk of the block's virtual list.
-// S is computed as Q K^T (rows on the MFMA M side) so that P and dS come out with lane <-> key
-// and registers <-> rows, which is the B-operand layout of dV^T = dO^T P and dK^T = Q^T dS;
-// dO^T and Q^T (lane <-> feature, registers <-> rows) are made with identity-MFMA transposes.
+// dK/dV of one block, accumulated over a chunk of the block's virtual list; wave kt of the
+// work-group owns keys 32kt .. 32kt+31.  The tile's Q and dO rows are gathered once per
+// work-group with coalesced loads (wave 0: Q, wave 1: dO when there are two waves) into row-major
+// LDS tiles.  S = Q K^T is computed with rows on the MFMA M side so that P and dS come out with
+// lane <-> key and registers <-> rows, which is the B-operand layout of dV^T = dO^T P and
+// dK^T = Q^T dS; dO^T and Q^T (lane <-> feature, k <-> rows) are read from the LDS tiles with
+// the hardware transpose load.
 template <int D, int KT>
-__global__ __launch_bounds__(64) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
-                                                         const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
-                                                         const float* __restrict__ lse, const float* __restrict__ delta,
-                                                         const char* __restrict__ iws, char* __restrict__ bws) {
-  constexpr int KS = D / 16, DT = D / 32;
+__global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+                                                              const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
+                                                              const float* __restrict__ lse, const float* __restrict__ delta,
+                                                              const char* __restrict__ iws, char* __restrict__ bws) {
+  constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
   __shared__ __align__(16) float lse_s[32];
   __shared__ __align__(16) float del_s[32];
   __shared__ __align__(16) int lim_s[32];
-  const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
+  __shared__ __align__(16) __bf16 xq_s[32 * RS];
+  __shared__ __align__(16) __bf16 xg_s[32 * RS];
+  const int kt = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
-  const int u = blockIdx.x / KT, kt = blockIdx.x % KT;
+  const int u = blockIdx.x;
   UnitInfo ui;
-  if (!locate_unit(P, iws, P.off_unitkv, P.chunk_kv, bh, u, ui)) return;
+  if (!locate_unit(P, iws, 2, bh, u, ui)) return;
   const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
+  const bool load_q = KT == 1 || kt == 0, load_g = KT == 1 || kt == 1;
 
-  bf16x8 Kf[KS], Vf[KS], ilo, ihi;
-  make_ident(lane, ilo, ihi);
+  bf16x8 Kf[KS], Vf[KS];
   const int kl = 32 * kt + n_;                 // this lane's key inside the block
   {
     const long key = (long)ui.j * P.B + kl;
@@ -541,28 +737,51 @@ __global__ __launch_bounds__(64) void sel_bwd_dkv_kernel(const SelPlan P, const 
   const float sc = P.scale * kLog2e;
   const int ppt = 32 >> P.lg;
   const int HQ = P.hkv * P.g;
+  const __bf16* qbase = q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1];
+  const __bf16* gbase = dout + b * P.so[0] + (long)(hk * P.g) * P.so[1];
 
+  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + ppt, n_);
+  RowInfo r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0, n_), n_);
+  bf16x8 rawq[KS], rawg[KS];
+  float lse_r, del_r;
+  {
+    if (load_q) issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], r.i, P.g - 1, lane);
+    if (load_g) issue_tile_loads<D>(rawg, gbase, P.so[1], P.so[2], r.i, P.g - 1, lane);
+    const size_t srow = ((size_t)b * HQ + hk * P.g + r.g) * P.n + r.i;
+    lse_r = lse[srow] * kLog2e;
+    del_r = delta[srow];
+  }
+
+  wait_all_loads();        // enter the loop with nothing pending, so the loop itself only waits for what it needs
   for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
-    const RowInfo r = locate_row(P, list, ui, vt, n_);
-    const int hq = hk * P.g + r.g;
-    const __bf16* qp = q + b * P.sq[0] + (long)hq * P.sq[1] + (long)r.i * P.sq[2] + 8 * h;
-    const __bf16* dop = dout + b * P.so[0] + (long)hq * P.so[1] + (long)r.i * P.so[2] + 8 * h;
-    bf16x8 Qf[KS], Gf[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) { Qf[ks] = load8(qp + 16 * ks); Gf[ks] = load8(dop + 16 * ks); }
-    if (h == 0) {
-      const size_t srow = ((size_t)b * HQ + hq) * P.n + r.i;
-      lse_s[n_] = r.valid ? lse[srow] * kLog2e : INFINITY;   // +inf: a padding row gets p = 0
-      del_s[n_] = delta[srow];
+    // commit the current tile (loaded during the previous iteration) to LDS
+    if (load_q) commit_tile<D>(rawq, xq_s, RS, lane);
+    if (load_g) commit_tile<D>(rawg, xg_s, RS, lane);
+    if (kt == 0 && h == 0) {
+      lse_s[n_] = r.valid ? lse_r : INFINITY;              // +inf: a padding row gets p = 0
+      del_s[n_] = del_r;
       lim_s[n_] = r.lim;
     }
     __syncthreads();
 
+    // issue the next tile's loads and the entry fetch of the tile after it
+    const RowInfo rn = decode_entry(P, ui, e_n, n_);
+    if (load_q) issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], rn.i, P.g - 1, lane);
+    if (load_g) issue_tile_loads<D>(rawg, gbase, P.so[1], P.so[2], rn.i, P.g - 1, lane);
+    float lse_n, del_n;
+    {
+      const size_t srown = ((size_t)b * HQ + hk * P.g + rn.g) * P.n + rn.i;
+      lse_n = lse[srown] * kLog2e;
+      del_n = delta[srown];
+    }
+    const RawEntry e_nn = fetch_entry(P, list, ui, vt + 2 * ppt, n_);
+    __builtin_amdgcn_sched_barrier(0);
+
     floatx16 Sa = zero_acc(), Pa = zero_acc();
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      Sa = mfma32(Qf[ks], Kf[ks], Sa);         // [row][key]: lane <-> key, registers <-> rows
-      Pa = mfma32(Gf[ks], Vf[ks], Pa);
+      Sa = mfma32(lds_row_operand(xq_s, RS, ks, lane), Kf[ks], Sa);   // [row][key]: lane <-> key, registers <-> rows
+      Pa = mfma32(lds_row_operand(xg_s, RS, ks, lane), Vf[ks], Pa);
     }
     floatx16 dSa;
 #pragma unroll
@@ -582,16 +801,14 @@ __global__ __launch_bounds__(64) void sel_bwd_dkv_kernel(const SelPlan P, const 
     const bf16x8 Sf0 = pack8(dSa, 0), Sf1 = pack8(dSa, 8);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      floatx16 t = mfma32(Gf[2 * dt], ilo, zero_acc());
-      t = mfma32(Gf[2 * dt + 1], ihi, t);      // t[row][feature]: lane <-> feature, registers <-> rows
-      dVa[dt] = mfma32(pack8(t, 0), Pf0, dVa[dt]);
-      dVa[dt] = mfma32(pack8(t, 8), Pf1, dVa[dt]);
-      t = mfma32(Qf[2 * dt], ilo, zero_acc());
-      t = mfma32(Qf[2 * dt + 1], ihi, t);
-      dKa[dt] = mfma32(pack8(t, 0), Sf0, dKa[dt]);
-      dKa[dt] = mfma32(pack8(t, 8), Sf1, dKa[dt]);
+      dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 0, 32 * dt, lane), Pf0, dVa[dt]);
+      dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 16, 32 * dt, lane), Pf1, dVa[dt]);
+      dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 0, 32 * dt, lane), Sf0, dKa[dt]);
+      dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 16, 32 * dt, lane), Sf1, dKa[dt]);
     }
     __syncthreads();
+    lse_r = lse_n; del_r = del_n;
+    r = rn; e_n = e_nn;
   }
 
   // partial [unit][2][32*KT keys][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][key kl]
@@ -615,7 +832,7 @@ template <int D, int KT>
 __global__ __launch_bounds__(256) void sel_bwd_dkv_reduce_kernel(const SelPlan P, const char* __restrict__ iws, const char* __restrict__ bws,
                                                                 __bf16* __restrict__ dk, __bf16* __restrict__ dv) {
   const int j = blockIdx.x, bh = blockIdx.y;
-  const int* unit_off = reinterpret_cast<const int*>(iws + P.off_unitkv) + (size_t)bh * (P.W + 1);
+  const int* unit_off = reinterpret_cast<const int*>(iws + P.off_unit[2]) + (size_t)bh * (P.W + 1);
   const int u0 = unit_off[j], u1 = unit_off[j + 1];
   const float* part = reinterpret_cast<const float*>(bws + P.off_dkvpart) + (size_t)bh * P.ub_kv * (2 * 32 * KT * D);
   const int keys = min(P.B, P.n - j * P.B);
@@ -674,6 +891,8 @@ extern "C" int nsa_select_build_index(const nsa_select_desc* d, const void* idx,
   NSA_LAUNCH_CHECK();
   hipLaunchKernelGGL(sel_scan_kernel, dim3(P.bh), dim3(256), lds, st, P, iws);
   NSA_LAUNCH_CHECK();
+  hipLaunchKernelGGL(sel_units_kernel, dim3(P.bh, 3), dim3(256), 0, st, P, iws);
+  NSA_LAUNCH_CHECK();
   hipLaunchKernelGGL(sel_fill_kernel, dim3(P.nch, P.bh), dim3(64), lds, st, P, idx, fmask, iws);
   NSA_LAUNCH_CHECK();
   return 0;
@@ -683,7 +902,7 @@ template <int D, int KT>
 static int launch_fwd(const SelPlan& P, const void* q, const void* k, const void* v, const void* idx, const uint8_t* fmask,
                       const void* iws, void* fws, void* out, float* lse, hipStream_t st, void* const* ev, int nev) {
   mark(ev, nev, 0, st);
-  hipLaunchKernelGGL((sel_fwd_kernel<D, KT>), dim3(P.ub_f, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+  hipLaunchKernelGGL((sel_fwd_kernel<D, KT>), dim3(xcd_grid(P, 0)), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                      (const char*)iws, (char*)fws);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 1, st);
@@ -726,7 +945,7 @@ static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void
   hipLaunchKernelGGL((sel_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, delta);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 1, st);
-  hipLaunchKernelGGL((sel_bwd_dq_kernel<D, KT>), dim3(P.ub_f, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+  hipLaunchKernelGGL((sel_bwd_dq_kernel<D, KT>), dim3(xcd_grid(P, 1)), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                      (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 2, st);
@@ -734,7 +953,7 @@ static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void
   hipLaunchKernelGGL((sel_bwd_dq_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)bws, (__bf16*)dq);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 3, st);
-  hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT>), dim3(P.ub_kv * KT, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+  hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT>), dim3(P.ub_kv, P.bh), dim3(64 * KT), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                      (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 4, st);

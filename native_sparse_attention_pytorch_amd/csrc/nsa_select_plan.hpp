@@ -11,12 +11,19 @@ namespace nsa {
 struct SelPlan {
   int b, hkv, g, lg, n, S, SP, B, D, causal, W, nch, bh, idx64;
   float scale;
-  int chunk_f, chunk_kv;     // pairs per work unit (forward / dQ walk, dK/dV walk)
-  int ub_f, ub_kv;           // upper bound of work units per (batch, kv head)
+  // Work-unit tables.  A unit = up to `chunk` consecutive pairs of one (query phase, block)
+  // cell; cells are ordered phase-major so that units running at the same time gather Q rows of
+  // the same query range (L2 reuse).  Table t: 0 = forward walk, 1 = dQ walk, 2 = dK/dV walk
+  // (a single phase: the whole sequence, so a wave keeps its dK/dV accumulators as long as
+  // possible).
+  int chunk[3], phase[3], np[3], ub[3];
+  size_t off_unit[3];
+  int ub_kv;                 // = ub[2]
   long list_cap;             // inverse-index entries reserved per (batch, kv head)
+  size_t prow;               // number of partial rows; row `prow` is a spare that padding rows write to
   long sq[3], sk[3], sv[3], so[3];
   // index workspace
-  size_t off_cnt, off_blk, off_unitf, off_unitkv, off_list, index_total;
+  size_t off_cnt, off_blk, off_list, index_total;
   // forward workspace
   size_t off_opart, off_lsepart, fwd_total;
   // backward workspace
@@ -48,31 +55,43 @@ static inline int make_plan(const nsa_select_desc* d, SelPlan& P) {
   for (int t = 0; t < 3; ++t) { P.sq[t] = d->q_stride[t]; P.sk[t] = d->k_stride[t]; P.sv[t] = d->v_stride[t]; P.so[t] = d->o_stride[t]; }
   for (int t = 0; t < 3; ++t)
     if ((P.sq[t] | P.sk[t] | P.sv[t] | P.so[t]) & 7) return NSA_E_ARG;      // rows must start 16-byte aligned
-  P.chunk_f = 256;
-  P.chunk_kv = 1024;
   const long pairs = (long)P.n * (P.S + P.causal);
-  P.ub_f = (int)(P.W + (pairs + P.chunk_f - 1) / P.chunk_f);
-  P.ub_kv = (int)(P.W + (pairs + P.chunk_kv - 1) / P.chunk_kv);
+  // phase length: the Q rows (forward) / Q and dO rows (dQ walk) of one phase should sit
+  // comfortably in one XCD's 4 MB L2: ~1 MB of rows per phase
+  const long row_bytes = (long)P.g * P.D * 2;
+  long ph = 256;
+  while (ph * 2 * row_bytes <= (1L << 21) && ph < (1L << 20)) ph *= 2;
+  P.chunk[0] = 256;  P.phase[0] = (int)ph;
+  P.chunk[1] = 256;  P.phase[1] = (int)(ph > 256 ? ph / 2 : ph);
+  P.chunk[2] = 1024; P.phase[2] = ((P.n + 255) / 256) * 256;
+  for (int t = 0; t < 3; ++t) {
+    P.np[t] = (P.n + P.phase[t] - 1) / P.phase[t];
+    const long cells = (long)P.np[t] * P.W;
+    const long ub = cells + (pairs + P.chunk[t] - 1) / P.chunk[t];
+    if (ub > 0x3fffffffL) return NSA_E_UNSUPPORTED;
+    P.ub[t] = (int)ub;
+  }
+  P.ub_kv = P.ub[2];
   P.list_cap = (long)P.n * (P.S > 0 ? P.S : 1);
 
   size_t o = 0;
   P.off_cnt = o;    o = align_up(o + (size_t)bh * P.nch * P.W * 4);
   P.off_blk = o;    o = align_up(o + (size_t)bh * (P.W + 1) * 4);
-  P.off_unitf = o;  o = align_up(o + (size_t)bh * (P.W + 1) * 4);
-  P.off_unitkv = o; o = align_up(o + (size_t)bh * (P.W + 1) * 4);
+  for (int t = 0; t < 3; ++t) { P.off_unit[t] = o; o = align_up(o + (size_t)bh * ((size_t)P.np[t] * P.W + 1) * 4); }
   P.off_list = o;   o = align_up(o + (size_t)bh * P.list_cap * 4);
   P.index_total = o;
 
   const size_t prow = (size_t)bh * P.n * P.SP * P.g;      // partial rows: (query, slot, head)
+  P.prow = prow;
   o = 0;
-  P.off_opart = o;   o = align_up(o + prow * P.D * 2);
-  P.off_lsepart = o; o = align_up(o + prow * 4);
+  P.off_opart = o;   o = align_up(o + (prow + 1) * P.D * 2);
+  P.off_lsepart = o; o = align_up(o + (prow + 1) * 4);
   P.fwd_total = o;
 
   const int KT = (P.B + 31) / 32;
   o = 0;
   P.off_delta = o;   o = align_up(o + (size_t)bh * P.g * P.n * 4);
-  P.off_dqpart = o;  o = align_up(o + prow * P.D * 2);
+  P.off_dqpart = o;  o = align_up(o + (prow + 1) * P.D * 2);
   P.off_dkvpart = o; o = align_up(o + (size_t)bh * P.ub_kv * 2 * 32 * KT * P.D * 4);
   P.bwd_total = o;
   return 0;
