@@ -323,7 +323,9 @@ template <int D, int KT>
 __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                      const __bf16* __restrict__ v, const char* __restrict__ iws, char* __restrict__ fws) {
   constexpr int KS = D / 16, DT = D / 32, TBL = 0;
-  __shared__ __align__(16) __bf16 tile_s[32 * (D + 8)];
+  constexpr int RS = D + 8;
+  __shared__ __align__(16) __bf16 tile_s[32 * RS];    // output staging
+  __shared__ __align__(16) __bf16 xq_s[32 * RS];      // the tile's Q rows
   __shared__ size_t row_s[32];
   const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
   int bh, u;
@@ -365,33 +367,26 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
   const float sc = P.scale * kLog2e;
   const int ppt = 32 >> P.lg;
 
-  // software pipeline: list entries two tiles ahead, Q operands one tile ahead
+  // software pipeline: list entries two tiles ahead, Q rows (coalesced gather) one tile ahead
+  const __bf16* qbase = q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1];
   RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + ppt, n_);
   RowInfo r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0, n_), n_);
-  bf16x8 Qf[KS];
-  {
-    const __bf16* qp = q + b * P.sq[0] + (long)(hk * P.g + r.g) * P.sq[1] + (long)r.i * P.sq[2] + 8 * h;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) Qf[ks] = load8(qp + 16 * ks);
-  }
+  bf16x8 rawq[KS];
+  issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], r.i, P.g - 1, lane);
 
   wait_all_loads();        // enter the loop with nothing pending, so the loop itself only waits for what it needs
   for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
-    // issue the next tile's operand loads and the entry fetch of the tile after it first
+    commit_tile<D>(rawq, xq_s, RS, lane);
+    __syncthreads();
+    // issue the next tile's loads and the entry fetch of the tile after it
     const RowInfo rn = decode_entry(P, ui, e_n, n_);
-    bf16x8 Qn[KS];
-    {
-#ifdef NSA_EXP_NOGATHER
-      const __bf16* qp = q + b * P.sq[0] + (long)(hk * P.g + rn.g) * P.sq[1] + (long)(rn.i & 63) * P.sq[2] + 8 * h;
-#else
-      const __bf16* qp = q + b * P.sq[0] + (long)(hk * P.g + rn.g) * P.sq[1] + (long)rn.i * P.sq[2] + 8 * h;
-#endif
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) Qn[ks] = load8(qp + 16 * ks);
-    }
+    issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], rn.i, P.g - 1, lane);
     const RawEntry e_nn = fetch_entry(P, list, ui, vt + 2 * ppt, n_);
     __builtin_amdgcn_sched_barrier(0);
 
+    bf16x8 Qf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) Qf[ks] = lds_row_operand(xq_s, RS, ks, lane);
     floatx16 Sa[KT];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
@@ -442,8 +437,6 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
       store_tile_rows<D>(Oa, inv, row, opart, tile_s, row_s, lane);
       if (h == 0) lsepart[row] = (mx + fast_log2(l)) * kLn2;
     }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) Qf[ks] = Qn[ks];
     r = rn; e_n = e_nn;
   }
 }
@@ -479,28 +472,27 @@ __global__ __launch_bounds__(256) void sel_fwd_combine_kernel(const SelPlan P, c
   for (int c = lane; c < P.g * CPR; c += 64) {
     const int g = c / CPR, dd = (c % CPR) * 8;
     const size_t row0 = ((size_t)bh * P.n + i) * P.SP * P.g + g;
-    float mx = -INFINITY;
-    for (unsigned long long m = live; m; m &= m - 1) {
-      const int s = __builtin_ctzll(m);
-      mx = fmaxf(mx, lsepart[row0 + (size_t)s * P.g]);
-    }
-    float sum = 0.f;
-    for (unsigned long long m = live; m; m &= m - 1) {
-      const int s = __builtin_ctzll(m);
-      sum += __expf(lsepart[row0 + (size_t)s * P.g] - mx);
-    }
-    const float L = live ? mx + __logf(sum) : -INFINITY;
+    // one pass, streaming log-sum-exp merge: acc = sum_s exp(lse_s - m) * o_s, rescaled as m grows
+    float mx = -INFINITY, sum = 0.f;
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
     for (unsigned long long m = live; m; m &= m - 1) {
       const int s = __builtin_ctzll(m);
       const size_t row = row0 + (size_t)s * P.g;
-      const float w = __expf(lsepart[row] - L);
+      const float ls = lsepart[row];
       const bf16x8 o = load8(opart + row * D + dd);
+      const float mn = fmaxf(mx, ls);
+      const float a = __expf(mx - mn), w = __expf(ls - mn);      // first slot: mx = -inf -> a = 0
+      sum = sum * a + w;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += w * (float)o[e];
+      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * a + w * (float)o[e];
+      mx = mn;
     }
+    const float L = live ? mx + __logf(sum) : -INFINITY;
+    const float inv = live ? 1.0f / sum : 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= inv;
     const int hq = hk * P.g + g;
     bf16x8 r;
 #pragma unroll
@@ -542,7 +534,10 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
                                                         const float* __restrict__ lse, const float* __restrict__ delta,
                                                         const char* __restrict__ iws, char* __restrict__ bws) {
   constexpr int KS = D / 16, DT = D / 32, TBL = 1;
-  __shared__ __align__(16) __bf16 tile_s[32 * (D + 8)];
+  constexpr int RS = D + 8;
+  __shared__ __align__(16) __bf16 tile_s[32 * RS];    // output staging
+  __shared__ __align__(16) __bf16 xq_s[32 * RS];      // the tile's Q rows
+  __shared__ __align__(16) __bf16 xg_s[32 * RS];      // the tile's dO rows
   __shared__ size_t row_s[32];
   const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
   int bh, u;
@@ -585,39 +580,40 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
   const int ppt = 32 >> P.lg;
   const int HQ = P.hkv * P.g;
 
+  const __bf16* qbase = q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1];
+  const __bf16* gbase = dout + b * P.so[0] + (long)(hk * P.g) * P.so[1];
   RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + ppt, n_);
   RowInfo r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0, n_), n_);
-  bf16x8 Qf[KS], Gf[KS];
+  bf16x8 rawq[KS], rawg[KS];
   float lse_r, del_r;
   {
-    const int hq = hk * P.g + r.g;
-    const __bf16* qp = q + b * P.sq[0] + (long)hq * P.sq[1] + (long)r.i * P.sq[2] + 8 * h;
-    const __bf16* dop = dout + b * P.so[0] + (long)hq * P.so[1] + (long)r.i * P.so[2] + 8 * h;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) { Qf[ks] = load8(qp + 16 * ks); Gf[ks] = load8(dop + 16 * ks); }
-    const size_t srow = ((size_t)b * HQ + hq) * P.n + r.i;
+    issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], r.i, P.g - 1, lane);
+    issue_tile_loads<D>(rawg, gbase, P.so[1], P.so[2], r.i, P.g - 1, lane);
+    const size_t srow = ((size_t)b * HQ + hk * P.g + r.g) * P.n + r.i;
     lse_r = lse[srow] * kLog2e;
     del_r = delta[srow];
   }
 
   wait_all_loads();        // enter the loop with nothing pending, so the loop itself only waits for what it needs
   for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
+    commit_tile<D>(rawq, xq_s, RS, lane);
+    commit_tile<D>(rawg, xg_s, RS, lane);
+    __syncthreads();
     const RowInfo rn = decode_entry(P, ui, e_n, n_);
-    bf16x8 Qn[KS], Gn[KS];
+    issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], rn.i, P.g - 1, lane);
+    issue_tile_loads<D>(rawg, gbase, P.so[1], P.so[2], rn.i, P.g - 1, lane);
     float lse_n, del_n;
     {
-      const int hqn = hk * P.g + rn.g;
-      const __bf16* qp = q + b * P.sq[0] + (long)hqn * P.sq[1] + (long)rn.i * P.sq[2] + 8 * h;
-      const __bf16* dop = dout + b * P.so[0] + (long)hqn * P.so[1] + (long)rn.i * P.so[2] + 8 * h;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) { Qn[ks] = load8(qp + 16 * ks); Gn[ks] = load8(dop + 16 * ks); }
-      const size_t srown = ((size_t)b * HQ + hqn) * P.n + rn.i;
+      const size_t srown = ((size_t)b * HQ + hk * P.g + rn.g) * P.n + rn.i;
       lse_n = lse[srown] * kLog2e;
       del_n = delta[srown];
     }
     const RawEntry e_nn = fetch_entry(P, list, ui, vt + 2 * ppt, n_);
     __builtin_amdgcn_sched_barrier(0);
 
+    bf16x8 Qf[KS], Gf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) { Qf[ks] = lds_row_operand(xq_s, RS, ks, lane); Gf[ks] = lds_row_operand(xg_s, RS, ks, lane); }
     floatx16 Sa[KT], Pa[KT];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
@@ -651,8 +647,6 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
       const size_t row = r.valid ? (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g : P.prow;
       store_tile_rows<D>(Qa, P.scale, row, dqpart, tile_s, row_s, lane);
     }
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) { Qf[ks] = Qn[ks]; Gf[ks] = Gn[ks]; }
     lse_r = lse_n; del_r = del_n;
     r = rn; e_n = e_nn;
   }

@@ -56,11 +56,12 @@ static inline int make_plan(const nsa_select_desc* d, SelPlan& P) {
   for (int t = 0; t < 3; ++t)
     if ((P.sq[t] | P.sk[t] | P.sv[t] | P.so[t]) & 7) return NSA_E_ARG;      // rows must start 16-byte aligned
   const long pairs = (long)P.n * (P.S + P.causal);
-  // phase length: the Q rows (forward) / Q and dO rows (dQ walk) of one phase should sit
-  // comfortably in one XCD's 4 MB L2: ~1 MB of rows per phase
+  // phase length: the Q rows (forward) / Q and dO rows (dQ walk) of one phase are about the size
+  // of one XCD's 4 MB L2 (measured best on MI355X among 0.5 .. 64 MB; shorter phases make the
+  // work units too small, longer ones lose the L2 reuse of the gathered rows)
   const long row_bytes = (long)P.g * P.D * 2;
   long ph = 256;
-  while (ph * 2 * row_bytes <= (1L << 21) && ph < (1L << 20)) ph *= 2;
+  while (ph * 2 * row_bytes <= (1L << 22) && ph < (1L << 20)) ph *= 2;
   P.chunk[0] = 256;  P.phase[0] = (int)ph;
   P.chunk[1] = 256;  P.phase[1] = (int)(ph > 256 ? ph / 2 : ph);
   P.chunk[2] = 1024; P.phase[2] = ((P.n + 255) / 256) * 256;
