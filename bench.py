@@ -73,7 +73,7 @@ class HipEvents:
         return out.value
 
 
-def cpu_baseline(cfg, q, k, v, do, idx, msk, nq=512):
+def cpu_baseline(cfg, q, k, v, do, idx, msk, nq=8192):
     """The CPU oracle (fp32 restatement of the reference's pure-torch path) on a bounded sample:
     the last `nq` queries of the same workload against the full-length K/V, forward+backward."""
     from oracle import nsa_oracle as O
@@ -177,6 +177,33 @@ def main():
                            tokens_per_s=round(b * n / (ms_step * 1e-3), 1), attended_pairs=int(pairs), flop_per_step=total_flop),
                kernels_ms={k_: round(v_, 4) for k_, v_ in kern.items()},
                roofline=roofline)
+
+    # the other half of BASELINE configs[3]: compressed attention with fused importance logits +
+    # top-k over 2048 compressed keys (+1 memory slot), forward and backward, reported beside the headline
+    try:
+        g2 = torch.Generator(device=dev).manual_seed(1)
+        nc = n // 16
+        ck = (torch.randn(b, hk, nc + 1, d, generator=g2, device=dev) * d ** -0.5).to(torch.bfloat16).requires_grad_()
+        cv = (torch.randn(b, hk, nc + 1, d, generator=g2, device=dev) * d ** -0.5).to(torch.bfloat16).requires_grad_()
+        qc = q.clone().requires_grad_()
+        tms = []
+        for it in range(3):
+            e0, e1, e2, e3 = (torch.cuda.Event(enable_timing=True) for _ in range(4))
+            e0.record()
+            c_out, imp = ops.compress_attend(qc, ck, cv, 1, 16, True, sel_block=B, share=True)
+            e1.record()
+            vals_, idx_, fm_ = ops.importance_topk(imp, S + 1)
+            e2.record()
+            c_out.backward(do)
+            e3.record()
+            torch.cuda.synchronize()
+            tms.append((e0.elapsed_time(e1), e1.elapsed_time(e2), e2.elapsed_time(e3)))
+        p_cmp = b * hq * sum(i // 16 + 1 for i in range(n))
+        best = min(tms[1:], key=sum)
+        res["compressed_branch"] = dict(fwd_with_importance_ms=round(best[0], 4), topk_ms=round(best[1], 4), bwd_ms=round(best[2], 4),
+                                        attended_pairs=p_cmp, fwd_bwd_tflops=round(14 * d * p_cmp / (sum(best) * 1e-3) / 1e12, 2))
+    except Exception as ex:  # the headline must still be printed
+        res["compressed_branch"] = dict(error=repr(ex))
 
     if not args.no_cpu:
         torch.set_num_threads(min(16, os.cpu_count() or 1))

@@ -1,0 +1,58 @@
+"""Decoder-only transformer around `SparseAttention`: the training-forward harness of the
+reference (native_sparse_attention_pytorch/transformer.py:130-138 FeedForward, :142-211
+construction, :254-330 forward) with the same constructor arguments and parameter names.
+Sampling / cached decoding (transformer.py:213-252) is outside the accelerated hot path."""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from .sparse_attention import SparseAttention
+
+
+def FeedForward(dim, expansion_factor=4.):
+    hidden = int(dim * expansion_factor)
+    return nn.Sequential(nn.RMSNorm(dim), nn.Linear(dim, hidden), nn.GELU(), nn.Linear(hidden, dim))
+
+
+class Transformer(nn.Module):
+    def __init__(self, num_tokens, dim, depth, dim_head=64, heads=8, kv_heads=None, ff_expansion_factor=4.,
+                 use_sparse_attn=True, causal=True, use_flex_sliding_window=False, use_flex_fine_selection=False,
+                 use_triton_fine_selection=False, sparse_attn_kwargs: dict | None = None):
+        super().__init__()
+        if not use_sparse_attn:
+            raise NotImplementedError("only the sparse-attention model is provided (the dense baseline is not part of the hot path)")
+        if use_flex_sliding_window or use_flex_fine_selection:
+            raise NotImplementedError("flex-attention backends are not provided; the HIP kernels implement the same masks")
+        sparse_attn_kwargs = dict(sparse_attn_kwargs or dict(sliding_window_size=32, compress_block_size=4,
+                                                             compress_block_sliding_stride=4, selection_block_size=4,
+                                                             num_selected_blocks=4))
+        self.token_emb = nn.Embedding(num_tokens, dim)
+        self.causal = causal
+        layers = []
+        for _ in range(depth):
+            attn = SparseAttention(dim=dim, dim_head=dim_head, heads=heads, kv_heads=kv_heads, causal=causal,
+                                   use_triton_kernel=use_triton_fine_selection, **sparse_attn_kwargs)
+            layers.append(nn.ModuleList([attn, FeedForward(dim=dim, expansion_factor=ff_expansion_factor)]))
+        self.layers = nn.ModuleList(layers)
+        self.norm = nn.RMSNorm(dim)
+        self.to_logits = nn.Linear(dim, num_tokens, bias=False)
+
+    def forward(self, ids, return_loss=False, disable_flex=False, disable_triton_kernel=False, cache=None, return_cache=False):
+        if cache is not None:
+            raise NotImplementedError("cached decoding is outside the accelerated hot path")
+        if return_loss:
+            ids, labels = ids[:, :-1], ids[:, 1:]
+        tokens = self.token_emb(ids)
+        caches = []
+        for attn, ff in self.layers:
+            # the reference always asks the attention layer for its cache (transformer.py:308-313)
+            attn_out, layer_cache = attn(tokens, return_cache=True) if return_cache else (attn(tokens), None)
+            caches.append(layer_cache)
+            tokens = attn_out + tokens
+            tokens = ff(tokens) + tokens
+        logits = self.to_logits(self.norm(tokens))
+        if not return_loss:
+            return (logits, caches) if return_cache else logits
+        return F.cross_entropy(logits.transpose(1, 2).float(), labels)

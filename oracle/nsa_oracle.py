@@ -443,3 +443,40 @@ def gate_combine(logits, c_out, f_out, s_out):
     h = c_out.shape[1]
     g = torch.sigmoid(logits).reshape(b, n, h, 3).permute(0, 2, 1, 3)
     return merge_heads(g[..., 0:1] * c_out + g[..., 1:2] * f_out + g[..., 2:3] * s_out)
+
+
+# --------------------------------------------------------------- training-step harness
+
+def _feed_forward(dim, expansion_factor=4.0):
+    hidden = int(dim * expansion_factor)
+    return nn.Sequential(nn.RMSNorm(dim), nn.Linear(dim, hidden), nn.GELU(), nn.Linear(hidden, dim))
+
+
+class TransformerOracle(nn.Module):
+    """Restatement of the reference's training forward, transformer.py:142-211 (construction
+    order: token_emb, per layer [attention, feed-forward], norm, to_logits) and :254-330
+    (ids[:, :-1] -> logits, cross entropy against ids[:, 1:])."""
+
+    def __init__(self, num_tokens, dim, depth, dim_head=64, heads=8, kv_heads=None, ff_expansion_factor=4.0,
+                 causal=True, sparse_attn_kwargs=None):
+        super().__init__()
+        self.token_emb = nn.Embedding(num_tokens, dim)
+        layers = []
+        for _ in range(depth):
+            attn = SparseAttentionOracle(dim=dim, dim_head=dim_head, heads=heads, kv_heads=kv_heads, causal=causal, **sparse_attn_kwargs)
+            layers.append(nn.ModuleList([attn, _feed_forward(dim, ff_expansion_factor)]))
+        self.layers = nn.ModuleList(layers)
+        self.norm = nn.RMSNorm(dim)
+        self.to_logits = nn.Linear(dim, num_tokens, bias=False)
+
+    def forward(self, ids, return_loss=False):
+        if return_loss:
+            ids, labels = ids[:, :-1], ids[:, 1:]
+        tokens = self.token_emb(ids)
+        for attn, ff in self.layers:
+            tokens = attn(tokens) + tokens
+            tokens = ff(tokens) + tokens
+        logits = self.to_logits(self.norm(tokens))
+        if not return_loss:
+            return logits
+        return F.cross_entropy(logits.transpose(1, 2), labels)
