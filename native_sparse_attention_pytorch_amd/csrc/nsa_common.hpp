@@ -88,6 +88,11 @@ __device__ __forceinline__ bf16x8 lds_transposed_operand(const __bf16* X, int RS
   return __builtin_bit_cast(bf16x8, r);
 }
 
+// MFMA operand (lane <-> row n_, k <-> 8 consecutive features) of k-step ks from a row-major tile
+__device__ __forceinline__ bf16x8 lds_row_operand(const __bf16* tile_s, int RS, int ks, int lane) {
+  return *reinterpret_cast<const bf16x8*>(tile_s + (lane & 31) * RS + 16 * ks + 8 * (lane >> 5));
+}
+
 // s_waitcnt vmcnt(0) (expcnt / lgkmcnt left at their maxima): all outstanding global loads
 // and stores of this wave have completed.
 __device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }

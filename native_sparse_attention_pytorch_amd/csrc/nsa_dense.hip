@@ -9,9 +9,13 @@
 // the npf = B/st compressed keys of a fine block; -inf where the reference's fill values make
 // the softmax term vanish), which feed the top-k kernel.
 //
-// All operands live in registers (no LDS staging); V^T / K^T / Q^T / dO^T operands are made
-// with identity-MFMA transposes (nsa_common.hpp).  One wave = one 32-row tile (32/G queries x G
-// heads) in the query-stationary kernels, one 32-key tile in the key-stationary dK/dV kernel.
+// Forward and dQ are query-stationary: a work-group of 4 waves owns 128 rows (128/G consecutive
+// queries x the G heads of one kv group, so the group shares every K/V tile), each wave 32 rows.
+// 64-key K/V tiles are gathered with coalesced 16-byte loads into registers one tile ahead,
+// committed to row-major LDS tiles and read back as MFMA operands: row operands with 16-byte LDS
+// reads, transposed operands (V^T, K^T) with the gfx950 LDS transpose load.  dK/dV is
+// key-stationary: two waves own a 64-key tile (32 keys each) and stream the query rows that can
+// see it, like the dK/dV walk of the block-selection kernels.
 #include "nsa_common.hpp"
 #include "nsa_dense_plan.hpp"
 
@@ -31,31 +35,71 @@ __device__ __forceinline__ Interval visible_range(const DensePlan& P, int i) {
   return r;
 }
 
+constexpr int kBK = 64;          // keys per K/V tile
+
+// One thread's share of a cooperative, coalesced load of `nrows` rows of D bf16 (row index ->
+// memory row through `first_row`, rows >= limit read as zero) by a work-group of NT threads.
+template <int D, int NT>
+struct TileRegs {
+  static constexpr int CPR = D / 8, RPI = NT / CPR, N = kBK / RPI;
+  bf16x8 r[N];
+  __device__ __forceinline__ void load(const __bf16* __restrict__ base, long s_row, long first_row, long limit, int tid) {
+#pragma unroll
+    for (int t = 0; t < N; ++t) {
+      const long row = first_row + t * RPI + tid / CPR;
+      r[t] = (row < limit) ? load8(base + row * s_row + 8 * (tid % CPR)) : zero_frag();
+    }
+  }
+  __device__ __forceinline__ void commit(__bf16* tile_s, int RS, int tid) const {
+#pragma unroll
+    for (int t = 0; t < N; ++t) *reinterpret_cast<bf16x8*>(tile_s + (t * RPI + tid / CPR) * RS + 8 * (tid % CPR)) = r[t];
+  }
+};
+
+// Key tiles walked by a query tile: t = -1 is the memory tile (stride mode), then 64-key tiles
+// t_lo .. t_hi of the interval union.
+struct TileWalk {
+  int t_first, t_lo, t_hi;
+  __device__ __forceinline__ int next(int t) const { return t < 0 ? t_lo : t + 1; }
+};
+
+__device__ __forceinline__ TileWalk make_walk(const DensePlan& P, int i_first, int i_last) {
+  TileWalk w;
+  const int lo = visible_range(P, i_first).lo, hi = visible_range(P, i_last).hi;
+  w.t_lo = lo / kBK;
+  w.t_hi = hi >= 0 ? hi / kBK : -1;
+  w.t_first = P.mem > 0 ? -1 : w.t_lo;
+  return w;
+}
+
 // ------------------------------------------------------------------------------- forward
 template <int D>
-__global__ __launch_bounds__(64) void dense_fwd_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
-                                                       const __bf16* __restrict__ v, __bf16* __restrict__ out, float* __restrict__ lse,
-                                                       float* __restrict__ pooled) {
-  constexpr int KS = D / 16, DT = D / 32;
-  const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
+__global__ __launch_bounds__(256) void dense_fwd_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+                                                        const __bf16* __restrict__ v, __bf16* __restrict__ out, float* __restrict__ lse,
+                                                        float* __restrict__ pooled) {
+  constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
+  __shared__ __align__(16) __bf16 k_s[kBK * RS];
+  __shared__ __align__(16) __bf16 v_s[kBK * RS];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
-  const int ppt = 32 >> P.lg;
-  const int i0 = blockIdx.x * ppt;
+  const int ppt = 32 >> P.lg;                       // queries per wave tile
+  const int q0 = blockIdx.x * 4 * ppt;              // first query of the work-group
+  const int i0 = q0 + wave * ppt;
   const int pq = n_ >> P.lg, g = n_ & (P.g - 1);
   const bool valid = i0 + pq < P.n;
-  const int i = valid ? i0 + pq : P.n - 1;
-  const int ilast = min(P.n - 1, i0 + ppt - 1);
+  const int i = min(i0 + pq, P.n - 1);
   const int hq = hk * P.g + g;
 
-  bf16x8 Qf[KS], ilo, ihi;
-  make_ident(lane, ilo, ihi);
+  bf16x8 Qf[KS];
   {
     const __bf16* qp = q + b * P.sq[0] + (long)hq * P.sq[1] + (long)i * P.sq[2] + 8 * h;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) Qf[ks] = load8(qp + 16 * ks);
   }
   const Interval me = visible_range(P, i);
-  const int tile_lo = visible_range(P, i0).lo, tile_hi = visible_range(P, ilast).hi;
+  const TileWalk walk = make_walk(P, q0, min(P.n - 1, q0 + 4 * ppt - 1));
+  // this wave's own reach (its tiles are a subset of the work-group's)
+  const int my_hi = visible_range(P, min(P.n - 1, i0 + ppt - 1)).hi, my_lo = visible_range(P, min(i0, P.n - 1)).lo;
   const float sc = P.scale * kLog2e;
 
   float m = -INFINITY, l = 0.f;
@@ -63,112 +107,133 @@ __global__ __launch_bounds__(64) void dense_fwd_kernel(const DensePlan P, const 
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) Oa[dt] = zero_acc();
 
-  const __bf16* kbase = k + b * P.sk[0] + hk * P.sk[1] + 8 * h;
-  const __bf16* vbase = v + b * P.sv[0] + hk * P.sv[1] + 8 * h;
-  const int t_first = (P.mem > 0) ? -1 : (tile_lo >> 5);
-  const int t_last = tile_hi >> 5;                       // tile_hi may be -1 -> t_last = -1
+  const __bf16* kbase = k + b * P.sk[0] + hk * P.sk[1];
+  const __bf16* vbase = v + b * P.sv[0] + hk * P.sv[1];
+  TileRegs<D, 256> kr, vr;
+  auto load_tile = [&](int t) {
+    const long first = t < 0 ? 0 : (long)P.mem + (long)t * kBK;
+    const long limit = t < 0 ? P.mem : (long)P.mem + P.nkeys;
+    kr.load(kbase, P.sk[2], first, limit, tid);
+    vr.load(vbase, P.sv[2], first, limit, tid);
+  };
+  int t = walk.t_first;
+  if (t <= walk.t_hi || t < 0) load_tile(t);
 
-  for (int t = t_first; t <= t_last; ++t) {
-    if (t == 0 && t_first == -1) t = tile_lo >> 5;       // after the memory tile jump to the first visible tile
+  for (; t <= walk.t_hi; t = walk.next(t)) {
+    kr.commit(k_s, RS, tid);
+    vr.commit(v_s, RS, tid);
+    __syncthreads();
+    const int tn = walk.next(t);
+    if (tn <= walk.t_hi) load_tile(tn);
     const bool memtile = t < 0;
-    // keys of this tile: memory rows 0..mem-1, or compressed / token keys 32t .. 32t+31
-    const int kk = memtile ? n_ : 32 * t + n_;
-    const bool kok = memtile ? (n_ < P.mem) : (kk < P.nkeys);
-    const long krow = kok ? (memtile ? kk : kk + P.mem) : 0;
-    bf16x8 Kf[KS], Vv[KS];
+    const int kb0 = memtile ? 0 : t * kBK;
+    // skip tiles outside this wave's reach (the barriers below are still executed)
+    const bool active = memtile || (kb0 <= my_hi && kb0 + kBK - 1 >= my_lo);
+    if (active) {
+      floatx16 Sa[2];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      Kf[ks] = kok ? load8(kbase + krow * P.sk[2] + 16 * ks) : zero_frag();
-      Vv[ks] = kok ? load8(vbase + krow * P.sv[2] + 16 * ks) : zero_frag();
-    }
-    floatx16 Sa = zero_acc();
+      for (int kt = 0; kt < 2; ++kt) {
+        Sa[kt] = zero_acc();
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) Sa = mfma32(Kf[ks], Qf[ks], Sa);
-
-    // visibility of the 16 keys this lane holds for its row
-    const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
-    const int kb0 = memtile ? 0 : 32 * t;
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int i2 = 0; i2 < 16; ++i2) {
-      const int key = kb0 + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
-      const float s = (key >= klo && key <= khi) ? Sa[i2] * sc : -INFINITY;
-      Sa[i2] = s;
-      tmax = fmaxf(tmax, s);
-    }
-
-    if (P.pool && !memtile) {
-      // block-importance logits: groups of npf consecutive keys, then the G heads of the group
-      const float to_nat = kLn2;                         // scores are in log2 units here
-      const int npf = P.npf;
-      float grp[4];                                      // one value per register quartet (a)
-#pragma unroll
-      for (int a = 0; a < 4; ++a) grp[a] = 0.f;
-      if (npf >= 4) {
-#pragma unroll
-        for (int a = 0; a < 4; ++a) grp[a] = (Sa[4 * a] + Sa[4 * a + 1]) + (Sa[4 * a + 2] + Sa[4 * a + 3]);
-        if (npf >= 8) {
-#pragma unroll
-          for (int a = 0; a < 4; ++a) grp[a] += xor32(grp[a]);
-        }
-        if (npf == 16) { grp[0] += grp[1]; grp[2] += grp[3]; }
-        if (npf == 32) { grp[0] = (grp[0] + grp[1]) + (grp[2] + grp[3]); }
+        for (int ks = 0; ks < KS; ++ks) Sa[kt] = mfma32(lds_row_operand(k_s + 32 * kt * RS, RS, ks, lane), Qf[ks], Sa[kt]);
       }
-      // number of values this lane holds and their first key offsets inside the tile
+      const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
+      float tmax = -INFINITY;
 #pragma unroll
-      for (int i2 = 0; i2 < 16; ++i2) {
-        float val; int koff; bool mine;
-        if (npf == 1) { val = Sa[i2]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 3); mine = true; }
-        else if (npf == 2) { val = Sa[i2 & ~1] + Sa[i2 | 1]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 2); mine = (i2 & 1) == 0; }
-        else if (npf == 4) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2) + 4 * h; mine = (i2 & 3) == 0; }
-        else if (npf == 8) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2); mine = (i2 & 3) == 0 && h == 0; }
-        else if (npf == 16) { val = grp[(i2 >> 3) * 2]; koff = 16 * (i2 >> 3); mine = (i2 & 7) == 0 && h == 0; }
-        else { val = grp[0]; koff = 0; mine = i2 == 0 && h == 0; }
-        if (P.share) {
-          for (int mk = 1; mk < P.g; mk <<= 1) val += __shfl_xor(val, mk, 64);
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i2 = 0; i2 < 16; ++i2) {
+          const int key = kb0 + 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
+          const float s = (key >= klo && key <= khi) ? Sa[kt][i2] * sc : -INFINITY;
+          Sa[kt][i2] = s;
+          tmax = fmaxf(tmax, s);
         }
-        const int jblk = (kb0 + koff) / npf;
-        const bool writer = mine && valid && jblk < P.nb && (!P.share || g == 0);
-        if (writer) {
-          float Lv = val * to_nat / (float)(npf * (P.share ? P.g : 1));
-          if (P.mask_own && jblk == i / P.B) Lv = -INFINITY;
-          const long prow = P.share ? ((long)bh * P.n + i) : (((long)b * P.hkv * P.g + hq) * P.n + i);
-          pooled[prow * P.nb + jblk] = Lv;
+
+      if (P.pool && !memtile) {
+        // block-importance logits: groups of npf consecutive keys, then the G heads of the group
+        const int npf = P.npf;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+          float grp[4];
+#pragma unroll
+          for (int a = 0; a < 4; ++a) grp[a] = 0.f;
+          if (npf >= 4) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) grp[a] = (Sa[kt][4 * a] + Sa[kt][4 * a + 1]) + (Sa[kt][4 * a + 2] + Sa[kt][4 * a + 3]);
+            if (npf >= 8) {
+#pragma unroll
+              for (int a = 0; a < 4; ++a) grp[a] += xor32(grp[a]);
+            }
+            if (npf == 16) { grp[0] += grp[1]; grp[2] += grp[3]; }
+            if (npf == 32) { grp[0] = (grp[0] + grp[1]) + (grp[2] + grp[3]); }
+          }
+#pragma unroll
+          for (int i2 = 0; i2 < 16; ++i2) {
+            float val; int koff; bool mine;
+            if (npf == 1) { val = Sa[kt][i2]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 3); mine = true; }
+            else if (npf == 2) { val = Sa[kt][i2 & ~1] + Sa[kt][i2 | 1]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 2); mine = (i2 & 1) == 0; }
+            else if (npf == 4) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2) + 4 * h; mine = (i2 & 3) == 0; }
+            else if (npf == 8) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2); mine = (i2 & 3) == 0 && h == 0; }
+            else if (npf == 16) { val = grp[(i2 >> 3) * 2]; koff = 16 * (i2 >> 3); mine = (i2 & 7) == 0 && h == 0; }
+            else { val = grp[0]; koff = 0; mine = i2 == 0 && h == 0; }
+            // only one register per group carries a distinct value: skip the head reduction for the rest
+            const bool distinct = npf == 1 || (npf == 2 && !(i2 & 1)) || (npf == 4 && !(i2 & 3)) || (npf == 8 && !(i2 & 3)) ||
+                                  (npf == 16 && !(i2 & 7)) || (npf == 32 && i2 == 0);
+            if (!distinct) continue;
+            if (P.share) {
+              for (int mk = 1; mk < P.g; mk <<= 1) val += __shfl_xor(val, mk, 64);
+            }
+            const int jblk = (kb0 + 32 * kt + koff) / npf;
+            const bool writer = mine && valid && jblk < P.nb && (!P.share || g == 0);
+            if (writer) {
+              float Lv = val * kLn2 / (float)(npf * (P.share ? P.g : 1));      // scores are in log2 units here
+              if (P.mask_own && jblk == i / P.B) Lv = -INFINITY;
+              const long prow = P.share ? ((long)bh * P.n + i) : (((long)b * P.hkv * P.g + hq) * P.n + i);
+              pooled[prow * P.nb + jblk] = Lv;
+            }
+          }
         }
       }
-    }
 
-    tmax = fmaxf(tmax, xor32(tmax));
-    const float mnew = fmaxf(m, tmax);
-    const float mref = (mnew == -INFINITY) ? 0.f : mnew;
-    const float alpha = fast_exp2(m - mref);
-    float rs = 0.f;
+      tmax = fmaxf(tmax, xor32(tmax));
+      const float mnew = fmaxf(m, tmax);
+      const float mref = (mnew == -INFINITY) ? 0.f : mnew;
+      const float alpha = fast_exp2(m - mref);
+      float rs = 0.f;
 #pragma unroll
-    for (int i2 = 0; i2 < 16; ++i2) {
-      const float p = fast_exp2(Sa[i2] - mref);
-      Sa[i2] = p;
-      rs += p;
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i2 = 0; i2 < 16; ++i2) {
+          const float p = fast_exp2(Sa[kt][i2] - mref);
+          Sa[kt][i2] = p;
+          rs += p;
+        }
+      rs += xor32(rs);
+      l = l * alpha + rs;
+      m = mnew;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) Oa[dt][e] *= alpha;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int u2 = 0; u2 < 2; ++u2) {
+          const bf16x8 Pf = pack8(Sa[kt], 8 * u2);
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+            Oa[dt] = mfma32(lds_transposed_operand(v_s, RS, 32 * kt + 16 * u2, 32 * dt, lane), Pf, Oa[dt]);
+        }
     }
-    rs += xor32(rs);
-    l = l * alpha + rs;
-    m = mnew;
-    const bf16x8 Pf0 = pack8(Sa, 0), Pf1 = pack8(Sa, 8);
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      floatx16 tv = mfma32(Vv[2 * dt], ilo, zero_acc());
-      tv = mfma32(Vv[2 * dt + 1], ihi, tv);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) Oa[dt][e] *= alpha;
-      Oa[dt] = mfma32(pack8(tv, 0), Pf0, Oa[dt]);
-      Oa[dt] = mfma32(pack8(tv, 8), Pf1, Oa[dt]);
-    }
+    __syncthreads();
   }
 
   if (P.pool) {
-    // fine blocks whose compressed keys no query of this tile can see were never visited
-    const int jstart = min(P.nb, (32 * (t_last + 1)) / P.npf);
+    // fine blocks whose compressed keys no query of this wave's tile can see were never visited
+    const int last_visited = my_hi >= 0 ? min(walk.t_hi, my_hi / kBK) : -1;
+    const int jstart = min(P.nb, (kBK * (last_visited + 1)) / P.npf);
     const int cntj = P.nb - jstart;
-    const int rows_here = min(ppt, P.n - i0) * (P.share ? 1 : P.g);
+    const int rows_here = max(0, min(ppt, P.n - i0)) * (P.share ? 1 : P.g);
     for (int e = lane; e < rows_here * cntj; e += 64) {
       const int rr = e / cntj, jj = jstart + e % cntj;
       const int qi = i0 + (P.share ? rr : rr / P.g);
@@ -212,24 +277,26 @@ __global__ __launch_bounds__(256) void dense_delta_kernel(const DensePlan P, con
   if (row < rows && (tid % LPR) == 0) delta[row] = s;
 }
 
-// dQ, query-stationary (same walk as the forward)
+// dQ, query-stationary (same tile walk as the forward): dS^T = P^T o (V dO^T - delta),
+// dQ^T += K^T dS^T with K^T read through the LDS transpose load.
 template <int D>
-__global__ __launch_bounds__(64) void dense_bwd_dq_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
-                                                          const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
-                                                          const float* __restrict__ lse, const float* __restrict__ delta, __bf16* __restrict__ dq) {
-  constexpr int KS = D / 16, DT = D / 32;
-  const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
+__global__ __launch_bounds__(256) void dense_bwd_dq_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+                                                           const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
+                                                           const float* __restrict__ lse, const float* __restrict__ delta, __bf16* __restrict__ dq) {
+  constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
+  __shared__ __align__(16) __bf16 k_s[kBK * RS];
+  __shared__ __align__(16) __bf16 v_s[kBK * RS];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
   const int ppt = 32 >> P.lg;
-  const int i0 = blockIdx.x * ppt;
+  const int q0 = blockIdx.x * 4 * ppt;
+  const int i0 = q0 + wave * ppt;
   const int pq = n_ >> P.lg, g = n_ & (P.g - 1);
   const bool valid = i0 + pq < P.n;
-  const int i = valid ? i0 + pq : P.n - 1;
-  const int ilast = min(P.n - 1, i0 + ppt - 1);
+  const int i = min(i0 + pq, P.n - 1);
   const int hq = hk * P.g + g;
 
-  bf16x8 Qf[KS], Gf[KS], ilo, ihi;
-  make_ident(lane, ilo, ihi);
+  bf16x8 Qf[KS], Gf[KS];
   {
     const __bf16* qp = q + b * P.sq[0] + (long)hq * P.sq[1] + (long)i * P.sq[2] + 8 * h;
     const __bf16* gp = dout + b * P.sdo[0] + (long)hq * P.sdo[1] + (long)i * P.sdo[2] + 8 * h;
@@ -239,50 +306,65 @@ __global__ __launch_bounds__(64) void dense_bwd_dq_kernel(const DensePlan P, con
   const long srow = ((long)b * P.hkv * P.g + hq) * P.n + i;
   const float lse_r = lse[srow] * kLog2e, del_r = delta[srow];
   const Interval me = visible_range(P, i);
-  const int tile_lo = visible_range(P, i0).lo, tile_hi = visible_range(P, ilast).hi;
+  const TileWalk walk = make_walk(P, q0, min(P.n - 1, q0 + 4 * ppt - 1));
+  const int my_hi = visible_range(P, min(P.n - 1, i0 + ppt - 1)).hi, my_lo = visible_range(P, min(i0, P.n - 1)).lo;
   const float sc = P.scale * kLog2e;
   floatx16 Qa[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) Qa[dt] = zero_acc();
-  const __bf16* kbase = k + b * P.sk[0] + hk * P.sk[1] + 8 * h;
-  const __bf16* vbase = v + b * P.sv[0] + hk * P.sv[1] + 8 * h;
-  const int t_first = (P.mem > 0) ? -1 : (tile_lo >> 5);
-  const int t_last = tile_hi >> 5;
 
-  for (int t = t_first; t <= t_last; ++t) {
-    if (t == 0 && t_first == -1) t = tile_lo >> 5;
+  const __bf16* kbase = k + b * P.sk[0] + hk * P.sk[1];
+  const __bf16* vbase = v + b * P.sv[0] + hk * P.sv[1];
+  TileRegs<D, 256> kr, vr;
+  auto load_tile = [&](int t) {
+    const long first = t < 0 ? 0 : (long)P.mem + (long)t * kBK;
+    const long limit = t < 0 ? P.mem : (long)P.mem + P.nkeys;
+    kr.load(kbase, P.sk[2], first, limit, tid);
+    vr.load(vbase, P.sv[2], first, limit, tid);
+  };
+  int t = walk.t_first;
+  if (t <= walk.t_hi || t < 0) load_tile(t);
+
+  for (; t <= walk.t_hi; t = walk.next(t)) {
+    kr.commit(k_s, RS, tid);
+    vr.commit(v_s, RS, tid);
+    __syncthreads();
+    const int tn = walk.next(t);
+    if (tn <= walk.t_hi) load_tile(tn);
     const bool memtile = t < 0;
-    const int kk = memtile ? n_ : 32 * t + n_;
-    const bool kok = memtile ? (n_ < P.mem) : (kk < P.nkeys);
-    const long krow = kok ? (memtile ? kk : kk + P.mem) : 0;
-    bf16x8 Kf[KS], Vf[KS];
+    const int kb0 = memtile ? 0 : t * kBK;
+    const bool active = memtile || (kb0 <= my_hi && kb0 + kBK - 1 >= my_lo);
+    if (active) {
+      floatx16 Sa[2], Pa[2];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      Kf[ks] = kok ? load8(kbase + krow * P.sk[2] + 16 * ks) : zero_frag();
-      Vf[ks] = kok ? load8(vbase + krow * P.sv[2] + 16 * ks) : zero_frag();
-    }
-    floatx16 Sa = zero_acc(), Pa = zero_acc();
+      for (int kt = 0; kt < 2; ++kt) {
+        Sa[kt] = zero_acc(); Pa[kt] = zero_acc();
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      Sa = mfma32(Kf[ks], Qf[ks], Sa);
-      Pa = mfma32(Vf[ks], Gf[ks], Pa);
-    }
-    const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
-    const int kb0 = memtile ? 0 : 32 * t;
+        for (int ks = 0; ks < KS; ++ks) {
+          Sa[kt] = mfma32(lds_row_operand(k_s + 32 * kt * RS, RS, ks, lane), Qf[ks], Sa[kt]);
+          Pa[kt] = mfma32(lds_row_operand(v_s + 32 * kt * RS, RS, ks, lane), Gf[ks], Pa[kt]);
+        }
+      }
+      const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
 #pragma unroll
-    for (int i2 = 0; i2 < 16; ++i2) {
-      const int key = kb0 + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
-      const float p = (key >= klo && key <= khi) ? fast_exp2(Sa[i2] * sc - lse_r) : 0.f;
-      Sa[i2] = p * (Pa[i2] - del_r);
-    }
-    const bf16x8 Sf0 = pack8(Sa, 0), Sf1 = pack8(Sa, 8);
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      floatx16 tk = mfma32(Kf[2 * dt], ilo, zero_acc());
-      tk = mfma32(Kf[2 * dt + 1], ihi, tk);
-      Qa[dt] = mfma32(pack8(tk, 0), Sf0, Qa[dt]);
-      Qa[dt] = mfma32(pack8(tk, 8), Sf1, Qa[dt]);
+        for (int i2 = 0; i2 < 16; ++i2) {
+          const int key = kb0 + 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
+          const float p = (key >= klo && key <= khi) ? fast_exp2(Sa[kt][i2] * sc - lse_r) : 0.f;
+          Sa[kt][i2] = p * (Pa[kt][i2] - del_r);
+        }
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int u2 = 0; u2 < 2; ++u2) {
+          const bf16x8 Sf = pack8(Sa[kt], 8 * u2);
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+            Qa[dt] = mfma32(lds_transposed_operand(k_s, RS, 32 * kt + 16 * u2, 32 * dt, lane), Sf, Qa[dt]);
+        }
     }
+    __syncthreads();
   }
   if (valid) {
     __bf16* op = dq + srow * D + 4 * h;
@@ -295,45 +377,47 @@ __global__ __launch_bounds__(64) void dense_bwd_dq_kernel(const DensePlan P, con
   }
 }
 
-// Query range [qlo, qhi) that can see any key of key tile t (t = -1: the memory tile).
-__device__ __forceinline__ void tile_query_range(const DensePlan& P, int t, int& qlo, int& qhi) {
-  if (t < 0) { qlo = 0; qhi = P.n; return; }
+// Query range [qlo, qhi) that can see any key of the 64-row tile T of k/v (rows counted from the
+// start of the arrays, memory slots included).
+__device__ __forceinline__ void tile_query_range(const DensePlan& P, int T, int& qlo, int& qhi) {
+  qhi = P.n;
   if (P.mode == 0) {
-    qlo = max(0, 32 * t - P.wf);
-    qhi = min(P.n, 32 * t + 31 + P.wb + 1);
+    qlo = max(0, kBK * T - P.wf);
+    qhi = min(P.n, kBK * T + kBK - 1 + P.wb + 1);
+  } else if (!P.causal || kBK * T < P.mem) {
+    qlo = 0;
   } else {
-    qlo = P.causal ? min(P.n, (32 * t + 1) * P.st) : 0;      // key kk visible iff i >= (kk+1)*st
-    qhi = P.n;
+    qlo = (int)min((long)P.n, ((long)kBK * T - P.mem + 1) * P.st);      // compressed key c is visible iff i >= (c+1)*st
   }
 }
 
-// dK/dV of one 32-key tile over one chunk of the queries that can see it (key-stationary);
-// same register scheme as sel_bwd_dkv_kernel.
+// dK/dV of one 64-row tile of k/v over one chunk of the queries that can see it (key-stationary);
+// wave kt owns rows 32kt .. 32kt+31 of the tile.  Rows are indexed from the start of the arrays,
+// so in stride mode row r is visible to query i iff r <= hi(i) + mem.
 template <int D>
-__global__ __launch_bounds__(64) void dense_bwd_dkv_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
-                                                           const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
-                                                           const float* __restrict__ lse, const float* __restrict__ delta, float* __restrict__ part) {
-  constexpr int KS = D / 16, DT = D / 32;
+__global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+                                                            const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
+                                                            const float* __restrict__ lse, const float* __restrict__ delta, float* __restrict__ part) {
+  constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
   __shared__ __align__(16) float lse_s[32];
   __shared__ __align__(16) float del_s[32];
   __shared__ __align__(16) int lo_s[32];
   __shared__ __align__(16) int hi_s[32];
-  const int lane = threadIdx.x, n_ = lane & 31, h = lane >> 5;
+  __shared__ __align__(16) __bf16 xq_s[32 * RS];
+  __shared__ __align__(16) __bf16 xg_s[32 * RS];
+  const int kt = threadIdx.x >> 6, lane = threadIdx.x & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
-  const int tix = blockIdx.x / P.chunks, c = blockIdx.x % P.chunks;
-  const int t = tix - (P.mem > 0 ? 1 : 0);
-  const bool memtile = t < 0;
+  const int T = blockIdx.x / P.chunks, c = blockIdx.x % P.chunks;
   int qlo, qhi;
-  tile_query_range(P, t, qlo, qhi);
+  tile_query_range(P, T, qlo, qhi);
   const int c0 = qlo + c * P.chunk_q, c1 = min(qhi, c0 + P.chunk_q);
   if (c0 >= c1) return;
 
-  const int kk = memtile ? n_ : 32 * t + n_;              // this lane's key (index space of the mask)
-  const bool kok = memtile ? (n_ < P.mem) : (kk < P.nkeys);
-  bf16x8 Kf[KS], Vf[KS], ilo, ihi;
-  make_ident(lane, ilo, ihi);
+  const int kr_ = kBK * T + 32 * kt + n_;                // this lane's row of k/v
+  const bool kok = kr_ < P.krows;
+  bf16x8 Kf[KS], Vf[KS];
   {
-    const long krow = kok ? (memtile ? kk : kk + P.mem) : 0;
+    const long krow = kok ? kr_ : 0;
     const __bf16* kp = k + b * P.sk[0] + hk * P.sk[1] + krow * P.sk[2] + 8 * h;
     const __bf16* vp = v + b * P.sv[0] + hk * P.sv[1] + krow * P.sv[2] + 8 * h;
 #pragma unroll
@@ -349,29 +433,60 @@ __global__ __launch_bounds__(64) void dense_bwd_dkv_kernel(const DensePlan P, co
   const int ppt = 32 >> P.lg;
   const int pq = n_ >> P.lg, g = n_ & (P.g - 1);
   const int hq = hk * P.g + g;
+  const __bf16* qbase = q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1];
+  const __bf16* gbase = dout + b * P.sdo[0] + (long)(hk * P.g) * P.sdo[1];
+  constexpr int CPR = D / 8, RPI = 64 / CPR, NT = 32 / RPI;
 
+  // wave 0 gathers the tile's Q rows, wave 1 its dO rows (coalesced), one tile ahead
+  bf16x8 raw[NT];
+  auto issue = [&](int i0) {
+    const __bf16* base = kt == 0 ? qbase : gbase;
+    const long sh = kt == 0 ? P.sq[1] : P.sdo[1], sn = kt == 0 ? P.sq[2] : P.sdo[2];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int rr = t * RPI + lane / CPR;
+      const int qi = min(i0 + (rr >> P.lg), P.n - 1);
+      raw[t] = load8(base + (long)(rr & (P.g - 1)) * sh + (long)qi * sn + 8 * (lane % CPR));
+    }
+  };
+  issue(c0);
+  float lse_r, del_r;
+  {
+    const int qi = min(c0 + pq, P.n - 1);
+    const long srow = ((long)b * P.hkv * P.g + hq) * P.n + qi;
+    lse_r = lse[srow] * kLog2e; del_r = delta[srow];
+  }
+  wait_all_loads();
   for (int i0 = c0; i0 < c1; i0 += ppt) {
     const bool valid = i0 + pq < c1;
-    const int i = valid ? i0 + pq : i0;
-    const __bf16* qp = q + b * P.sq[0] + (long)hq * P.sq[1] + (long)i * P.sq[2] + 8 * h;
-    const __bf16* gp = dout + b * P.sdo[0] + (long)hq * P.sdo[1] + (long)i * P.sdo[2] + 8 * h;
-    bf16x8 Qf[KS], Gf[KS];
+    const int i = min(i0 + pq, P.n - 1);
+    {
+      __bf16* dst = kt == 0 ? xq_s : xg_s;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) { Qf[ks] = load8(qp + 16 * ks); Gf[ks] = load8(gp + 16 * ks); }
-    if (h == 0) {
-      const long srow = ((long)b * P.hkv * P.g + hq) * P.n + i;
-      lse_s[n_] = valid ? lse[srow] * kLog2e : INFINITY;
-      del_s[n_] = delta[srow];
+      for (int t = 0; t < NT; ++t) *reinterpret_cast<bf16x8*>(dst + (t * RPI + lane / CPR) * RS + 8 * (lane % CPR)) = raw[t];
+    }
+    if (kt == 0 && h == 0) {
+      lse_s[n_] = valid ? lse_r : INFINITY;                // +inf: a padding row gets p = 0
+      del_s[n_] = del_r;
       const Interval me = visible_range(P, i);
-      lo_s[n_] = memtile ? 0 : me.lo;
-      hi_s[n_] = memtile ? P.mem - 1 : me.hi;
+      lo_s[n_] = P.mode == 0 ? me.lo : 0;
+      hi_s[n_] = P.mode == 0 ? me.hi : me.hi + P.mem;
     }
     __syncthreads();
+    issue(i0 + ppt);
+    float lse_n, del_n;
+    {
+      const int qi = min(i0 + ppt + pq, P.n - 1);
+      const long srow = ((long)b * P.hkv * P.g + hq) * P.n + qi;
+      lse_n = lse[srow] * kLog2e; del_n = delta[srow];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
     floatx16 Sa = zero_acc(), Pa = zero_acc();
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      Sa = mfma32(Qf[ks], Kf[ks], Sa);
-      Pa = mfma32(Gf[ks], Vf[ks], Pa);
+      Sa = mfma32(lds_row_operand(xq_s, RS, ks, lane), Kf[ks], Sa);     // [row][key]: lane <-> key, registers <-> rows
+      Pa = mfma32(lds_row_operand(xg_s, RS, ks, lane), Vf[ks], Pa);
     }
     floatx16 dSa;
 #pragma unroll
@@ -383,7 +498,7 @@ __global__ __launch_bounds__(64) void dense_bwd_dkv_kernel(const DensePlan P, co
 #pragma unroll
       for (int bb = 0; bb < 4; ++bb) {
         const int i2 = 4 * a + bb;
-        const float p = (kk >= lo4[bb] && kk <= hi4[bb]) ? fast_exp2(Sa[i2] * sc - l4[bb]) : 0.f;
+        const float p = (kr_ >= lo4[bb] && kr_ <= hi4[bb]) ? fast_exp2(Sa[i2] * sc - l4[bb]) : 0.f;
         Sa[i2] = p;
         dSa[i2] = p * (Pa[i2] - d4[bb]);
       }
@@ -392,19 +507,17 @@ __global__ __launch_bounds__(64) void dense_bwd_dkv_kernel(const DensePlan P, co
     const bf16x8 Sf0 = pack8(dSa, 0), Sf1 = pack8(dSa, 8);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      floatx16 tt = mfma32(Gf[2 * dt], ilo, zero_acc());
-      tt = mfma32(Gf[2 * dt + 1], ihi, tt);
-      dVa[dt] = mfma32(pack8(tt, 0), Pf0, dVa[dt]);
-      dVa[dt] = mfma32(pack8(tt, 8), Pf1, dVa[dt]);
-      tt = mfma32(Qf[2 * dt], ilo, zero_acc());
-      tt = mfma32(Qf[2 * dt + 1], ihi, tt);
-      dKa[dt] = mfma32(pack8(tt, 0), Sf0, dKa[dt]);
-      dKa[dt] = mfma32(pack8(tt, 8), Sf1, dKa[dt]);
+      dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 0, 32 * dt, lane), Pf0, dVa[dt]);
+      dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 16, 32 * dt, lane), Pf1, dVa[dt]);
+      dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 0, 32 * dt, lane), Sf0, dKa[dt]);
+      dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 16, 32 * dt, lane), Sf1, dKa[dt]);
     }
     __syncthreads();
+    lse_r = lse_n; del_r = del_n;
   }
-  float* pk = part + (((size_t)bh * P.key_tiles + tix) * P.chunks + c) * (2 * 32 * D) + (size_t)n_ * D + 4 * h;
-  float* pv = pk + 32 * D;
+  // partial [bh][tile][chunk][2][64][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][row 32kt + n_]
+  float* pk = part + (((size_t)bh * P.key_tiles + T) * P.chunks + c) * (2 * kBK * D) + (size_t)(32 * kt + n_) * D + 4 * h;
+  float* pv = pk + kBK * D;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -419,23 +532,21 @@ __global__ __launch_bounds__(64) void dense_bwd_dkv_kernel(const DensePlan P, co
 
 template <int D>
 __global__ __launch_bounds__(256) void dense_bwd_dkv_reduce_kernel(const DensePlan P, const float* __restrict__ part, __bf16* __restrict__ dk, __bf16* __restrict__ dv) {
-  const int tix = blockIdx.x, bh = blockIdx.y;
-  const int t = tix - (P.mem > 0 ? 1 : 0);
+  const int T = blockIdx.x, bh = blockIdx.y;
   int qlo, qhi;
-  tile_query_range(P, t, qlo, qhi);
+  tile_query_range(P, T, qlo, qhi);
   const int live = qhi > qlo ? (qhi - qlo + P.chunk_q - 1) / P.chunk_q : 0;
-  const int keys = t < 0 ? P.mem : min(32, P.nkeys - 32 * t);
-  const long row0 = t < 0 ? 0 : (long)P.mem + 32 * t;
-  const float* base = part + ((size_t)bh * P.key_tiles + tix) * P.chunks * (2 * 32 * D);
+  const int keys = min(kBK, P.krows - kBK * T);
+  const float* base = part + ((size_t)bh * P.key_tiles + T) * P.chunks * (2 * kBK * D);
   constexpr int CPR = D / 4;
   for (int e = threadIdx.x; e < 2 * keys * CPR; e += 256) {
     const int which = e / (keys * CPR), rem = e % (keys * CPR);
     const int key = rem / CPR, dd = (rem % CPR) * 4;
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
     for (int c = 0; c < live; ++c)
-      acc += *reinterpret_cast<const floatx4*>(base + (size_t)c * (2 * 32 * D) + (size_t)which * 32 * D + (size_t)key * D + dd);
+      acc += *reinterpret_cast<const floatx4*>(base + (size_t)c * (2 * kBK * D) + (size_t)which * kBK * D + (size_t)key * D + dd);
     const float s = which == 0 ? P.scale : 1.0f;
-    __bf16* dst = (which == 0 ? dk : dv) + ((size_t)bh * P.krows + row0 + key) * D + dd;
+    __bf16* dst = (which == 0 ? dk : dv) + ((size_t)bh * P.krows + (size_t)kBK * T + key) * D + dd;
     store4_bf16(dst, acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s);
   }
 }
@@ -460,8 +571,8 @@ extern "C" int nsa_dense_workspace_bytes(const nsa_dense_desc* d, size_t* bwd_by
 
 template <int D>
 static int dense_fwd_launch(const DensePlan& P, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, hipStream_t st) {
-  const int ppt = 32 >> P.lg;
-  hipLaunchKernelGGL((dense_fwd_kernel<D>), dim3((P.n + ppt - 1) / ppt, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+  const int qpw = 4 * (32 >> P.lg);                 // queries per work-group
+  hipLaunchKernelGGL((dense_fwd_kernel<D>), dim3((P.n + qpw - 1) / qpw, P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (__bf16*)out, lse, pooled);
   NSA_LAUNCH_CHECK();
   return 0;
@@ -486,11 +597,11 @@ static int dense_bwd_launch(const DensePlan& P, const void* q, const void* k, co
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((dense_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, delta);
   NSA_LAUNCH_CHECK();
-  const int ppt = 32 >> P.lg;
-  hipLaunchKernelGGL((dense_bwd_dq_kernel<D>), dim3((P.n + ppt - 1) / ppt, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+  const int qpw = 4 * (32 >> P.lg);
+  hipLaunchKernelGGL((dense_bwd_dq_kernel<D>), dim3((P.n + qpw - 1) / qpw, P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (const __bf16*)dout, lse, delta, (__bf16*)dq);
   NSA_LAUNCH_CHECK();
-  hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(P.key_tiles * P.chunks, P.bh), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+  hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(P.key_tiles * P.chunks, P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
   NSA_LAUNCH_CHECK();
   hipLaunchKernelGGL((dense_bwd_dkv_reduce_kernel<D>), dim3(P.key_tiles, P.bh), dim3(256), 0, st, P, part, (__bf16*)dk, (__bf16*)dv);

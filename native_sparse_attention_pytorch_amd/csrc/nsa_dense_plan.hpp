@@ -53,14 +53,16 @@ static inline int make_dense_plan(const nsa_dense_desc* d, DensePlan& P) {
     P.sq[t] = d->q_stride[t]; P.sk[t] = d->k_stride[t]; P.sv[t] = d->v_stride[t]; P.so[t] = d->o_stride[t]; P.sdo[t] = d->do_stride[t];
     if ((P.sq[t] | P.sk[t] | P.sv[t] | P.so[t] | P.sdo[t]) & 7) return NSA_E_ARG;
   }
-  P.key_tiles = (P.mem > 0 ? 1 : 0) + (P.nkeys + 31) / 32;
+  // dK/dV walk: 64-row tiles of k/v (memory slots included), the queries that can see a tile
+  // are cut into chunks of chunk_q; smaller chunks when there would be too few work-groups
+  P.key_tiles = (P.krows + 63) / 64;
+  const long span = P.mode == 0 ? ((long)64 + P.wb + P.wf < P.n ? (long)64 + P.wb + P.wf : P.n) : P.n;
   P.chunk_q = 1024;
-  const int span = P.mode == 0 ? (32 + P.wb + P.wf) : P.n;      // queries that can see one key tile
-  P.chunks = (span < P.n ? span : P.n) / P.chunk_q + 2;
-  if (P.mode == 1) P.chunks = (P.n + P.chunk_q - 1) / P.chunk_q;
+  while (P.chunk_q > 128 && bh * P.key_tiles * ((span + P.chunk_q - 1) / P.chunk_q) < 2048) P.chunk_q /= 2;
+  P.chunks = (int)((span + P.chunk_q - 1) / P.chunk_q);
   size_t o = 0;
   P.off_delta = o; o = dense_align_up(o + (size_t)bh * P.g * P.n * 4);
-  P.off_part = o;  o = dense_align_up(o + (size_t)bh * P.key_tiles * P.chunks * 2 * 32 * P.D * 4);
+  P.off_part = o;  o = dense_align_up(o + (size_t)bh * P.key_tiles * P.chunks * 2 * 64 * P.D * 4);
   P.bwd_total = o;
   return 0;
 }

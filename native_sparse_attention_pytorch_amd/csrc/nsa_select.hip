@@ -279,11 +279,6 @@ __device__ __forceinline__ void commit_tile(const bf16x8 (&raw)[D / 16], __bf16*
   }
 }
 
-// MFMA operand (lane <-> row n_, k <-> 8 consecutive features) of k-step ks from a row-major tile
-__device__ __forceinline__ bf16x8 lds_row_operand(const __bf16* tile_s, int RS, int ks, int lane) {
-  return *reinterpret_cast<const bf16x8*>(tile_s + (lane & 31) * RS + 16 * ks + 8 * (lane >> 5));
-}
-
 // Write a wave's 32-row x D accumulator tile (transposed MFMA layout: lane <-> row n_,
 // register (dt, a, b) <-> feature 32dt + 8a + 4h + b) as bf16 rows through LDS, so that every
 // global store instruction covers whole 2*D-byte rows (16 bytes per lane, consecutive lanes
