@@ -102,6 +102,14 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
+// value of lane ^ 1 / lane ^ 2 (DPP quad permutes: VALU speed, no LDS round trip)
+__device__ __forceinline__ float dpp_quad_xor1(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ float dpp_quad_xor2(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+}
+
 // store 4 floats as 4 bf16 (8 bytes)
 __device__ __forceinline__ void store4_bf16(__bf16* p, float a, float b, float c, float d) {
   bf16x4 r;

@@ -73,13 +73,17 @@ __device__ __forceinline__ TileWalk make_walk(const DensePlan& P, int i_first, i
 }
 
 // ------------------------------------------------------------------------------- forward
-template <int D>
+// NPF = selection block / compress stride when the importance logits are wanted, 0 otherwise
+template <int D, int NPF>
 __global__ __launch_bounds__(256) void dense_fwd_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                         const __bf16* __restrict__ v, __bf16* __restrict__ out, float* __restrict__ lse,
                                                         float* __restrict__ pooled) {
   constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
   __shared__ __align__(16) __bf16 k_s[kBK * RS];
   __shared__ __align__(16) __bf16 v_s[kBK * RS];
+  constexpr bool POOL = NPF > 0;
+  constexpr int NBT = POOL ? kBK / (POOL ? NPF : 1) : 1;        // fine blocks per key tile
+  __shared__ float pool_s[POOL ? 4 * 32 * NBT : 1];   // per wave: [rows or queries of the tile][fine blocks of the key tile]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
   const int ppt = 32 >> P.lg;                       // queries per wave tile
@@ -138,6 +142,8 @@ __global__ __launch_bounds__(256) void dense_fwd_kernel(const DensePlan P, const
         for (int ks = 0; ks < KS; ++ks) Sa[kt] = mfma32(lds_row_operand(k_s + 32 * kt * RS, RS, ks, lane), Qf[ks], Sa[kt]);
       }
       const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
+      floatx16 Sraw[2];
+      if (POOL) { Sraw[0] = Sa[0]; Sraw[1] = Sa[1]; }
       float tmax = -INFINITY;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
@@ -149,9 +155,13 @@ __global__ __launch_bounds__(256) void dense_fwd_kernel(const DensePlan P, const
           tmax = fmaxf(tmax, s);
         }
 
-      if (P.pool && !memtile) {
-        // block-importance logits: groups of npf consecutive keys, then the G heads of the group
-        const int npf = P.npf;
+      if (POOL && !memtile) {
+        // Block-importance logits of this 64-key tile: sum the raw scaled logits over the npf keys
+        // of a fine block (in registers / one exchange between the lane halves) and over the G
+        // heads of the group (adjacent lanes: DPP quad permutes for G <= 4), stage the sums in
+        // LDS and write them with coalesced stores; visibility is index arithmetic at store time.
+        constexpr int npf = POOL ? NPF : 1, nbt = NBT;
+        float* pw = pool_s + wave * (32 * nbt);
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
           float grp[4];
@@ -159,7 +169,7 @@ __global__ __launch_bounds__(256) void dense_fwd_kernel(const DensePlan P, const
           for (int a = 0; a < 4; ++a) grp[a] = 0.f;
           if (npf >= 4) {
 #pragma unroll
-            for (int a = 0; a < 4; ++a) grp[a] = (Sa[kt][4 * a] + Sa[kt][4 * a + 1]) + (Sa[kt][4 * a + 2] + Sa[kt][4 * a + 3]);
+            for (int a = 0; a < 4; ++a) grp[a] = (Sraw[kt][4 * a] + Sraw[kt][4 * a + 1]) + (Sraw[kt][4 * a + 2] + Sraw[kt][4 * a + 3]);
             if (npf >= 8) {
 #pragma unroll
               for (int a = 0; a < 4; ++a) grp[a] += xor32(grp[a]);
@@ -169,30 +179,48 @@ __global__ __launch_bounds__(256) void dense_fwd_kernel(const DensePlan P, const
           }
 #pragma unroll
           for (int i2 = 0; i2 < 16; ++i2) {
-            float val; int koff; bool mine;
-            if (npf == 1) { val = Sa[kt][i2]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 3); mine = true; }
-            else if (npf == 2) { val = Sa[kt][i2 & ~1] + Sa[kt][i2 | 1]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 2); mine = (i2 & 1) == 0; }
-            else if (npf == 4) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2) + 4 * h; mine = (i2 & 3) == 0; }
-            else if (npf == 8) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2); mine = (i2 & 3) == 0 && h == 0; }
-            else if (npf == 16) { val = grp[(i2 >> 3) * 2]; koff = 16 * (i2 >> 3); mine = (i2 & 7) == 0 && h == 0; }
-            else { val = grp[0]; koff = 0; mine = i2 == 0 && h == 0; }
-            // only one register per group carries a distinct value: skip the head reduction for the rest
             const bool distinct = npf == 1 || (npf == 2 && !(i2 & 1)) || (npf == 4 && !(i2 & 3)) || (npf == 8 && !(i2 & 3)) ||
                                   (npf == 16 && !(i2 & 7)) || (npf == 32 && i2 == 0);
             if (!distinct) continue;
+            float val; int koff; bool mine;
+            if (npf == 1) { val = Sraw[kt][i2]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 3); mine = true; }
+            else if (npf == 2) { val = Sraw[kt][i2] + Sraw[kt][i2 | 1]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 2); mine = true; }
+            else if (npf == 4) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2) + 4 * h; mine = true; }
+            else if (npf == 8) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2); mine = h == 0; }
+            else if (npf == 16) { val = grp[(i2 >> 3) * 2]; koff = 16 * (i2 >> 3); mine = h == 0; }
+            else { val = grp[0]; koff = 0; mine = h == 0; }
+            int prow_local = n_;                         // row inside the wave tile (per head) ...
             if (P.share) {
-              for (int mk = 1; mk < P.g; mk <<= 1) val += __shfl_xor(val, mk, 64);
+              if (P.g == 2) {
+                val += dpp_quad_xor1(val);
+              } else if (P.g == 4) {
+                val += dpp_quad_xor1(val);
+                val += dpp_quad_xor2(val);
+              } else {
+                for (int mk = 1; mk < P.g; mk <<= 1) val += __shfl_xor(val, mk, 64);
+              }
+              prow_local = pq;                           // ... or query inside the wave tile (shared)
+              mine = mine && g == 0;
             }
-            const int jblk = (kb0 + 32 * kt + koff) / npf;
-            const bool writer = mine && valid && jblk < P.nb && (!P.share || g == 0);
-            if (writer) {
-              float Lv = val * kLn2 / (float)(npf * (P.share ? P.g : 1));      // scores are in log2 units here
-              if (P.mask_own && jblk == i / P.B) Lv = -INFINITY;
-              const long prow = P.share ? ((long)bh * P.n + i) : (((long)b * P.hkv * P.g + hq) * P.n + i);
-              pooled[prow * P.nb + jblk] = Lv;
-            }
+            if (mine) pw[prow_local * nbt + (32 * kt + koff) / npf] = val;
           }
         }
+        __builtin_amdgcn_wave_barrier();
+        const int rows_here = P.share ? ppt : 32;
+        const float norm = P.scale / (float)(npf * (P.share ? P.g : 1));
+        for (int e = lane; e < rows_here * nbt; e += 64) {
+          const int rr = e / nbt, jj = e % nbt;
+          const int qi = i0 + (P.share ? rr : (rr >> P.lg));
+          const int jblk = (kb0 / npf) + jj;
+          if (qi < P.n && jblk < P.nb) {
+            // all npf keys of the block visible: (jblk+1)*npf - 1 <= qi/st - 1  <=>  (jblk+1)*B <= qi
+            const bool own = (long)jblk * P.B <= qi && qi < (long)(jblk + 1) * P.B;
+            const bool vis = (!P.causal || (long)(jblk + 1) * P.B <= qi) && !(P.mask_own && own);
+            const long prow = P.share ? ((long)bh * P.n + qi) : (((long)b * P.hkv * P.g + hk * P.g + (rr & (P.g - 1))) * P.n + qi);
+            pooled[prow * P.nb + jblk] = vis ? pw[rr * nbt + jj] * norm : -INFINITY;
+          }
+        }
+        __builtin_amdgcn_wave_barrier();
       }
 
       tmax = fmaxf(tmax, xor32(tmax));
@@ -228,10 +256,10 @@ __global__ __launch_bounds__(256) void dense_fwd_kernel(const DensePlan P, const
     __syncthreads();
   }
 
-  if (P.pool) {
+  if (POOL) {
     // fine blocks whose compressed keys no query of this wave's tile can see were never visited
     const int last_visited = my_hi >= 0 ? min(walk.t_hi, my_hi / kBK) : -1;
-    const int jstart = min(P.nb, (kBK * (last_visited + 1)) / P.npf);
+    const int jstart = min(P.nb, (kBK * (last_visited + 1)) / (POOL ? NPF : 1));
     const int cntj = P.nb - jstart;
     const int rows_here = max(0, min(ppt, P.n - i0)) * (P.share ? 1 : P.g);
     for (int e = lane; e < rows_here * cntj; e += 64) {
@@ -569,13 +597,27 @@ extern "C" int nsa_dense_workspace_bytes(const nsa_dense_desc* d, size_t* bwd_by
   return 0;
 }
 
-template <int D>
-static int dense_fwd_launch(const DensePlan& P, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, hipStream_t st) {
+template <int D, int NPF>
+static int dense_fwd_launch2(const DensePlan& P, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, hipStream_t st) {
   const int qpw = 4 * (32 >> P.lg);                 // queries per work-group
-  hipLaunchKernelGGL((dense_fwd_kernel<D>), dim3((P.n + qpw - 1) / qpw, P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+  hipLaunchKernelGGL((dense_fwd_kernel<D, NPF>), dim3((P.n + qpw - 1) / qpw, P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (__bf16*)out, lse, pooled);
   NSA_LAUNCH_CHECK();
   return 0;
+}
+
+template <int D>
+static int dense_fwd_launch(const DensePlan& P, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, hipStream_t st) {
+  switch (P.pool ? P.npf : 0) {
+    case 0: return dense_fwd_launch2<D, 0>(P, q, k, v, out, lse, pooled, st);
+    case 1: return dense_fwd_launch2<D, 1>(P, q, k, v, out, lse, pooled, st);
+    case 2: return dense_fwd_launch2<D, 2>(P, q, k, v, out, lse, pooled, st);
+    case 4: return dense_fwd_launch2<D, 4>(P, q, k, v, out, lse, pooled, st);
+    case 8: return dense_fwd_launch2<D, 8>(P, q, k, v, out, lse, pooled, st);
+    case 16: return dense_fwd_launch2<D, 16>(P, q, k, v, out, lse, pooled, st);
+    case 32: return dense_fwd_launch2<D, 32>(P, q, k, v, out, lse, pooled, st);
+  }
+  return NSA_E_UNSUPPORTED;
 }
 
 extern "C" int nsa_dense_fwd(const nsa_dense_desc* d, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, void* stream) {
