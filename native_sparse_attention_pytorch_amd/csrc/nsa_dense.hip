@@ -419,6 +419,23 @@ __device__ __forceinline__ void tile_query_range(const DensePlan& P, int T, int&
   }
 }
 
+__device__ __forceinline__ void chunk_range(const DensePlan& P, int T, int c, int& qlo, int& qhi, int& c0, int& c1) {
+  tile_query_range(P, T, qlo, qhi);
+  if (P.mode == 0) {
+    c0 = qlo + c * P.chunk_q;
+    c1 = min(qhi, c0 + P.chunk_q);
+  } else {
+    c0 = max(qlo, c * P.chunk_q);
+    c1 = min(qhi, (c + 1) * P.chunk_q);
+  }
+}
+
+__device__ __forceinline__ void chunk_of(const DensePlan& P, int x, int& T, int& c, int& qlo, int& qhi, int& c0, int& c1) {
+  if (P.mode == 0) { T = x / P.chunks; c = x % P.chunks; }
+  else { c = x / P.key_tiles; T = x % P.key_tiles; }
+  chunk_range(P, T, c, qlo, qhi, c0, c1);
+}
+
 // dK/dV of one 64-row tile of k/v over one chunk of the queries that can see it (key-stationary);
 // wave kt owns rows 32kt .. 32kt+31 of the tile.  Rows are indexed from the start of the arrays,
 // so in stride mode row r is visible to query i iff r <= hi(i) + mem.
@@ -435,10 +452,12 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
   __shared__ __align__(16) __bf16 xg_s[32 * RS];
   const int kt = threadIdx.x >> 6, lane = threadIdx.x & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
-  const int T = blockIdx.x / P.chunks, c = blockIdx.x % P.chunks;
-  int qlo, qhi;
-  tile_query_range(P, T, qlo, qhi);
-  const int c0 = qlo + c * P.chunk_q, c1 = min(qhi, c0 + P.chunk_q);
+  // band mode: chunks are counted from the tile's first visible query, tile-major order (adjacent
+  // tiles see almost the same queries).  Stride mode: chunks are absolute query ranges in
+  // chunk-major order, so that work-groups running together read the same Q/dO chunk (L2 reuse
+  // across the key tiles) instead of each streaming its own.
+  int T, c, qlo, qhi, c0, c1;
+  chunk_of(P, blockIdx.x, T, c, qlo, qhi, c0, c1);
   if (c0 >= c1) return;
 
   const int kr_ = kBK * T + 32 * kt + n_;                // this lane's row of k/v
@@ -561,9 +580,6 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
 template <int D>
 __global__ __launch_bounds__(256) void dense_bwd_dkv_reduce_kernel(const DensePlan P, const float* __restrict__ part, __bf16* __restrict__ dk, __bf16* __restrict__ dv) {
   const int T = blockIdx.x, bh = blockIdx.y;
-  int qlo, qhi;
-  tile_query_range(P, T, qlo, qhi);
-  const int live = qhi > qlo ? (qhi - qlo + P.chunk_q - 1) / P.chunk_q : 0;
   const int keys = min(kBK, P.krows - kBK * T);
   const float* base = part + ((size_t)bh * P.key_tiles + T) * P.chunks * (2 * kBK * D);
   constexpr int CPR = D / 4;
@@ -571,8 +587,11 @@ __global__ __launch_bounds__(256) void dense_bwd_dkv_reduce_kernel(const DensePl
     const int which = e / (keys * CPR), rem = e % (keys * CPR);
     const int key = rem / CPR, dd = (rem % CPR) * 4;
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int c = 0; c < live; ++c)
-      acc += *reinterpret_cast<const floatx4*>(base + (size_t)c * (2 * kBK * D) + (size_t)which * kBK * D + (size_t)key * D + dd);
+    for (int c = 0; c < P.chunks; ++c) {
+      int qlo, qhi, c0, c1;
+      chunk_range(P, T, c, qlo, qhi, c0, c1);
+      if (c0 < c1) acc += *reinterpret_cast<const floatx4*>(base + (size_t)c * (2 * kBK * D) + (size_t)which * kBK * D + (size_t)key * D + dd);
+    }
     const float s = which == 0 ? P.scale : 1.0f;
     __bf16* dst = (which == 0 ? dk : dv) + ((size_t)bh * P.krows + (size_t)kBK * T + key) * D + dd;
     store4_bf16(dst, acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s);
