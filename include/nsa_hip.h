@@ -73,11 +73,14 @@ int nsa_select_fwd(const nsa_select_desc* d, const void* q, const void* k, const
 /* dq: bf16 contiguous [batch, kv_heads*group, seq, dim_head]; dk, dv: bf16 contiguous
  * [batch, kv_heads, seq, dim_head].  Atomic-free and bit-reproducible: dK/dV of a KV block are
  * accumulated on chip by the work-groups that own the block, dQ is reduced over a query's slots.
- * (The reference accumulates all three through global fp32 atomics, TRI.py:758-788, 1395-1425.) */
+ * (The reference accumulates all three through global fp32 atomics, TRI.py:758-788, 1395-1425.)
+ * sel_grads: NULL, or fp32 contiguous [batch, kv_heads, seq, num_sel] receiving the gradient of a
+ * multiplier of value 1 on each slot's keys (the straight-through top-k gates `sel_scale`,
+ * TRI.py:1061-1080, NSA.py:793-797); dead slots get 0. */
 int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const void* v,
                    const void* out, const void* d_out, const float* lse,
                    const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
-                   void* dq, void* dk, void* dv, void* stream);
+                   void* dq, void* dk, void* dv, float* sel_grads, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Interval-masked GQA flash attention: one kernel family for
@@ -146,7 +149,7 @@ int nsa_select_fwd_timed(const nsa_select_desc* d, const void* q, const void* k,
 int nsa_select_bwd_timed(const nsa_select_desc* d, const void* q, const void* k, const void* v,
                          const void* out, const void* d_out, const float* lse,
                          const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
-                         void* dq, void* dk, void* dv, void* stream, void* const* events, int num_events);
+                         void* dq, void* dk, void* dv, float* sel_grads, void* stream, void* const* events, int num_events);
 
 #ifdef __cplusplus
 }

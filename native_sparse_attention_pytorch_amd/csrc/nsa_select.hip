@@ -523,11 +523,14 @@ __global__ __launch_bounds__(256) void sel_delta_kernel(const SelPlan P, const _
 }
 
 // dQ partial of every (query, slot) pair; same walk and register layout as the forward
-template <int D, int KT>
+// With GATE the kernel also writes sel_grads[b,h,i,slot] = sum over the group's heads and the
+// slot's keys of dS * (scaled logit): the gradient of a multiplier of 1 applied to the slot's
+// keys (the straight-through top-k gates of NSA.py:715, 793-797; TRI.py:1061-1080).
+template <int D, int KT, bool GATE>
 __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                         const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
                                                         const float* __restrict__ lse, const float* __restrict__ delta,
-                                                        const char* __restrict__ iws, char* __restrict__ bws) {
+                                                        const char* __restrict__ iws, char* __restrict__ bws, float* __restrict__ sel_grads) {
   constexpr int KS = D / 16, DT = D / 32, TBL = 1;
   constexpr int RS = D + 8;
   __shared__ __align__(16) __bf16 tile_s[32 * RS];    // output staging
@@ -619,14 +622,23 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
         Pa[kt] = mfma32(Vf[kt][ks], Gf[ks], Pa[kt]);
       }
     }
+    float gs = 0.f;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int i2 = 0; i2 < 16; ++i2) {
         const int kl = 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
-        const float p = (kl <= r.lim) ? fast_exp2(Sa[kt][i2] * sc - lse_r) : 0.f;
-        Sa[kt][i2] = p * (Pa[kt][i2] - del_r);
+        const float sraw = Sa[kt][i2];
+        const float p = (kl <= r.lim) ? fast_exp2(sraw * sc - lse_r) : 0.f;
+        const float ds = p * (Pa[kt][i2] - del_r);
+        Sa[kt][i2] = ds;
+        if (GATE) gs += ds * sraw;
       }
+    if (GATE) {
+      gs += xor32(gs);
+      for (int mk = 1; mk < P.g; mk <<= 1) gs += __shfl_xor(gs, mk, 64);      // the G heads of a pair are adjacent lanes
+      if (r.valid && r.g == 0 && h == 0 && r.slot < P.S) sel_grads[((size_t)bh * P.n + r.i) * P.S + r.slot] = gs * P.scale;
+    }
     floatx16 Qa[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) Qa[dt] = zero_acc();
@@ -649,13 +661,15 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
 
 template <int D>
 __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, const char* __restrict__ bws,
-                                                                __bf16* __restrict__ dq) {
+                                                                __bf16* __restrict__ dq, float* __restrict__ sel_grads) {
   const int lane = threadIdx.x & 63;
   const long qi = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (qi >= (long)P.bh * P.n) return;
   const int bh = (int)(qi / P.n), i = (int)(qi % P.n);
   const int b = bh / P.hkv, hk = bh % P.hkv;
   const unsigned long long live = live_slots(P, idx, fmask, bh, i, lane);
+  // slots the walk never visited carry no gradient
+  if (sel_grads && lane < P.S && !((live >> lane) & 1)) sel_grads[((size_t)bh * P.n + i) * P.S + lane] = 0.f;
   const __bf16* dqpart = reinterpret_cast<const __bf16*>(bws + P.off_dqpart);
   constexpr int CPR = D / 8;
   for (int c = lane; c < P.g * CPR; c += 64) {
@@ -926,7 +940,7 @@ extern "C" int nsa_select_fwd(const nsa_select_desc* d, const void* q, const voi
 
 template <int D, int KT>
 static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
-                      const void* idx, const uint8_t* fmask, const void* iws, void* bws, void* dq, void* dk, void* dv, hipStream_t st, void* const* ev, int nev) {
+                      const void* idx, const uint8_t* fmask, const void* iws, void* bws, void* dq, void* dk, void* dv, float* sel_grads, hipStream_t st, void* const* ev, int nev) {
   mark(ev, nev, 0, st);
   float* delta = reinterpret_cast<float*>((char*)bws + P.off_delta);
   const long rows = (long)P.bh * P.g * P.n;
@@ -934,12 +948,17 @@ static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void
   hipLaunchKernelGGL((sel_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, delta);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 1, st);
-  hipLaunchKernelGGL((sel_bwd_dq_kernel<D, KT>), dim3(xcd_grid(P, 1)), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
-                     (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
+  if (sel_grads) {
+    hipLaunchKernelGGL((sel_bwd_dq_kernel<D, KT, true>), dim3(xcd_grid(P, 1)), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+                       (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws, sel_grads);
+  } else {
+    hipLaunchKernelGGL((sel_bwd_dq_kernel<D, KT, false>), dim3(xcd_grid(P, 1)), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+                       (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws, sel_grads);
+  }
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 2, st);
   const long nq = (long)P.bh * P.n;
-  hipLaunchKernelGGL((sel_bwd_dq_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)bws, (__bf16*)dq);
+  hipLaunchKernelGGL((sel_bwd_dq_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)bws, (__bf16*)dq, sel_grads);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 3, st);
   hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT>), dim3(P.ub_kv, P.bh), dim3(64 * KT), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
@@ -954,7 +973,7 @@ static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void
 
 extern "C" int nsa_select_bwd_timed(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* out, const void* d_out,
                                     const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
-                                    void* dq, void* dk, void* dv, void* stream, void* const* ev, int nev) {
+                                    void* dq, void* dk, void* dv, float* sel_grads, void* stream, void* const* ev, int nev) {
   SelPlan P;
   const int rc = make_plan(d, P);
   if (rc) return rc;
@@ -962,17 +981,17 @@ extern "C" int nsa_select_bwd_timed(const nsa_select_desc* d, const void* q, con
   if (!q || !k || !v || !out || !d_out || !lse || !index_ws || !bwd_ws || !dq || !dk || !dv) return NSA_E_ARG;
   hipStream_t st = (hipStream_t)stream;
   const int KT = (P.B + 31) / 32;
-  if (P.D == 64 && KT == 1) return launch_bwd<64, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st, ev, nev);
-  if (P.D == 64 && KT == 2) return launch_bwd<64, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st, ev, nev);
-  if (P.D == 128 && KT == 1) return launch_bwd<128, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st, ev, nev);
-  if (P.D == 128 && KT == 2) return launch_bwd<128, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, st, ev, nev);
+  if (P.D == 64 && KT == 1) return launch_bwd<64, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
+  if (P.D == 64 && KT == 2) return launch_bwd<64, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
+  if (P.D == 128 && KT == 1) return launch_bwd<128, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
+  if (P.D == 128 && KT == 2) return launch_bwd<128, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
   return NSA_E_UNSUPPORTED;
 }
 
 extern "C" int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* out, const void* d_out,
                               const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
-                              void* dq, void* dk, void* dv, void* stream) {
-  return nsa_select_bwd_timed(d, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, bwd_bytes, dq, dk, dv, stream, nullptr, 0);
+                              void* dq, void* dk, void* dv, float* sel_grads, void* stream) {
+  return nsa_select_bwd_timed(d, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, bwd_bytes, dq, dk, dv, sel_grads, stream, nullptr, 0);
 }
 
-extern "C" int nsa_abi_version(void) { return 1; }
+extern "C" int nsa_abi_version(void) { return 2; }

@@ -9,6 +9,7 @@ missing library raise.
 from __future__ import annotations
 
 import ctypes as C
+from typing import Optional
 
 import torch
 from torch import Tensor
@@ -62,7 +63,9 @@ def _ws_sizes(dsc) -> tuple[int, int, int]:
 # ------------------------------------------------------------------------------- selection
 
 @torch.library.custom_op("nsa_amd::select_fwd", mutates_args=())
-def select_fwd(q: Tensor, k: Tensor, v: Tensor, idx: Tensor, fmask: Tensor, block: int, causal: bool, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+def select_fwd(q: Tensor, k: Tensor, v: Tensor, idx: Tensor, fmask: Tensor, sel_scale: Optional[Tensor], block: int, causal: bool,
+               scale: float) -> tuple[Tensor, Tensor, Tensor]:
+    # sel_scale only takes part in the backward (its value is 1 by contract, TRI.py:1861)
     q, k, v = _prep(q), _prep(k), _prep(v)
     b, hq, n, d = q.shape
     idx = idx.contiguous()
@@ -84,14 +87,14 @@ def select_fwd(q: Tensor, k: Tensor, v: Tensor, idx: Tensor, fmask: Tensor, bloc
 
 
 @select_fwd.register_fake
-def _(q, k, v, idx, fmask, block, causal, scale):
+def _(q, k, v, idx, fmask, sel_scale, block, causal, scale):
     b, hq, n, d = q.shape
     return (q.new_empty((b, hq, n, d)), q.new_empty((b, hq, n), dtype=torch.float32), q.new_empty((1,), dtype=torch.uint8))
 
 
 @torch.library.custom_op("nsa_amd::select_bwd", mutates_args=())
 def select_bwd(q: Tensor, k: Tensor, v: Tensor, out: Tensor, dout: Tensor, lse: Tensor, idx: Tensor, fmask: Tensor,
-               index_ws: Tensor, block: int, causal: bool, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+               index_ws: Tensor, block: int, causal: bool, scale: float, want_sel_grads: bool) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     q, k, v = _prep(q), _prep(k), _prep(v)
     out = out.contiguous()
     dout = dout.contiguous()
@@ -109,28 +112,31 @@ def select_bwd(q: Tensor, k: Tensor, v: Tensor, out: Tensor, dout: Tensor, lse: 
     if index_ws.numel() < ib:
         raise RuntimeError("inverse index workspace does not belong to these shapes")
     bwd_ws = torch.empty(wb, dtype=torch.uint8, device=q.device)
+    dsel = torch.empty(idx.shape if want_sel_grads else (0,), dtype=torch.float32, device=q.device)
     _lib.check(_lib.lib().nsa_select_bwd(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(idx), _ptr(fm),
-                                         _ptr(index_ws), _ptr(bwd_ws), wb, _ptr(dq), _ptr(dk), _ptr(dv), _stream()), "nsa_select_bwd")
-    return dq, dk, dv
+                                         _ptr(index_ws), _ptr(bwd_ws), wb, _ptr(dq), _ptr(dk), _ptr(dv),
+                                         _ptr(dsel) if want_sel_grads else 0, _stream()), "nsa_select_bwd")
+    return dq, dk, dv, dsel
 
 
 @select_bwd.register_fake
-def _(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale):
-    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+def _(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale, want_sel_grads):
+    return (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+            q.new_empty(idx.shape if want_sel_grads else (0,), dtype=torch.float32))
 
 
 def _select_setup(ctx, inputs, output):
-    q, k, v, idx, fmask, block, causal, scale = inputs
+    q, k, v, idx, fmask, sel_scale, block, causal, scale = inputs
     out, lse, index_ws = output
     ctx.save_for_backward(q, k, v, out, lse, idx, fmask, index_ws)
-    ctx.args = (block, causal, scale)
+    ctx.args = (block, causal, scale, sel_scale is not None and sel_scale.requires_grad, None if sel_scale is None else sel_scale.dtype)
 
 
 def _select_backward(ctx, dout, dlse, dws):
     q, k, v, out, lse, idx, fmask, index_ws = ctx.saved_tensors
-    block, causal, scale = ctx.args
-    dq, dk, dv = select_bwd(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale)
-    return dq, dk, dv, None, None, None, None, None
+    block, causal, scale, want, sdtype = ctx.args
+    dq, dk, dv, dsel = select_bwd(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale, want)
+    return dq, dk, dv, None, None, (dsel.to(sdtype) if want else None), None, None, None
 
 
 select_fwd.register_autograd(_select_backward, setup_context=_select_setup)
@@ -142,7 +148,10 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     """Drop-in for native_sparse_attend (TRI.py:1938-1987): fq [b,Hq,n,d], fk/fv [b,Hkv,n,d],
     selected_block_indices / fmask [b,Hkv|Hq,n,S].  Returns out [b,Hq,n,d] in fq's dtype and,
     on request, lse [b,Hq,n] (fp32).  Inputs are computed in bf16 (the reference computes in
-    fp16, TRI.py:1845).  `block_dk_dv_use_dot` is accepted and ignored (a Triton tuning switch)."""
+    fp16, TRI.py:1845).  `sel_scale` must be all ones (straight-through gates, as the reference
+    asserts at TRI.py:1861 - not re-checked here to avoid a device sync); it receives the gradient
+    TRI.py:1061-1080 computes.  `block_dk_dv_use_dot` is accepted and ignored (a Triton tuning
+    switch)."""
     q_heads, kv_heads, sel_heads = fq.shape[1], fk.shape[1], selected_block_indices.shape[1]
     assert q_heads % kv_heads == 0
     assert sel_heads in (q_heads, kv_heads)
@@ -150,14 +159,12 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     if return_sliding_window_out:
         raise NotImplementedError("the fused sliding-window output is experimental in the reference "
                                   "(test_triton_nsa.py:144) and is served by sliding_attend here")
-    if sel_scale is not None:
-        raise NotImplementedError("sel_scale (differentiable top-k gates) is not implemented in the HIP path yet")
     dtype = fq.dtype
     if kv_heads != sel_heads:                         # per-query-head selection: TRI.py:1961-1962
         g = q_heads // kv_heads
         fk, fv = fk.repeat_interleave(g, dim=1), fv.repeat_interleave(g, dim=1)
     scale = fq.shape[-1] ** -0.5
-    out, lse, _ = select_fwd(fq.to(_BF16), fk.to(_BF16), fv.to(_BF16), selected_block_indices, fmask,
+    out, lse, _ = select_fwd(fq.to(_BF16), fk.to(_BF16), fv.to(_BF16), selected_block_indices, fmask, sel_scale,
                              int(block_size), bool(include_block_causal), float(scale))
     out = out.to(dtype)
     return (out, lse) if return_lse else out
@@ -235,13 +242,46 @@ def _dense_setup(ctx, inputs, output):
     q, k, v, mode, causal, window, stride, num_mem, pool, sel_block, share, scale = inputs
     out, lse, _ = output
     ctx.save_for_backward(q, k, v, out, lse)
-    ctx.args = (mode, causal, window, stride, num_mem, scale)
+    ctx.args = (mode, causal, window, stride, num_mem, scale, sel_block, share)
+    ctx.set_materialize_grads(False)
+
+
+def _importance_backward(q, ck, dpooled, num_mem, stride, sel_block, share, scale):
+    """Gradient of the importance logits (NSA.py:652-680: mean of the scaled logits over a fine
+    block's npf compressed keys and, if shared, the group's heads) with respect to q and ck.  The
+    logits are linear in both, so this is two small dense GEMMs per (batch, kv head); entries that
+    were -inf carry zero gradient by construction of the softmax that follows."""
+    b, hq, n, d = q.shape
+    hk = ck.shape[1]
+    g = hq // hk
+    nb = dpooled.shape[-1]
+    npf = sel_block // stride
+    dp = torch.nan_to_num(dpooled.float(), nan=0.0, posinf=0.0, neginf=0.0)
+    ckb = ck[:, :, num_mem:num_mem + nb * npf].float().reshape(b, hk, nb, npf, d).sum(dim=3)       # [b,hk,nb,d]
+    qf = q.float()
+    if share:
+        c = scale / (g * npf)
+        dq = (c * torch.matmul(dp, ckb)).repeat_interleave(g, dim=1)                                # every head of the group
+        dckb = c * torch.matmul(dp.transpose(-1, -2), qf.reshape(b, hk, g, n, d).sum(dim=2))         # [b,hk,nb,d]
+    else:
+        c = scale / npf
+        dq = c * torch.matmul(dp, ckb.repeat_interleave(g, dim=1))
+        dckb = c * torch.matmul(dp.transpose(-1, -2), qf).reshape(b, hk, g, nb, d).sum(dim=2)
+    dck = torch.zeros_like(ck, dtype=torch.float32)
+    dck[:, :, num_mem:num_mem + nb * npf] = dckb.repeat_interleave(npf, dim=2)
+    return dq, dck
 
 
 def _dense_backward(ctx, dout, dlse, dpooled):
     q, k, v, out, lse = ctx.saved_tensors
-    mode, causal, window, stride, num_mem, scale = ctx.args
-    dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale)
+    mode, causal, window, stride, num_mem, scale, sel_block, share = ctx.args
+    dq = dk = dv = None
+    if dout is not None:
+        dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale)
+    if dpooled is not None and dpooled.numel() > 0:
+        dq2, dk2 = _importance_backward(q, k, dpooled, num_mem, stride, sel_block, share, scale)
+        dq = dq2.to(q.dtype) if dq is None else (dq.float() + dq2).to(q.dtype)
+        dk = dk2.to(k.dtype) if dk is None else (dk.float() + dk2).to(k.dtype)
     return (dq, dk, dv) + (None,) * 9
 
 
@@ -291,10 +331,35 @@ def _(scores, k, apply_softmax):
     return (scores.new_empty(shp, dtype=torch.int32), scores.new_empty(shp), scores.new_empty(shp, dtype=torch.uint8))
 
 
+class _ImportanceTopk(torch.autograd.Function):
+    """HIP top-k in the forward; the backward of `values` through the padded softmax (plain
+    elementwise torch, O(rows * nb)) - only used for the differentiable top-k gates."""
+
+    @staticmethod
+    def forward(ctx, logits, k):
+        idx, vals, fm = topk_op(logits, k, True)
+        ctx.save_for_backward(logits, idx)
+        ctx.mark_non_differentiable(idx, fm)
+        return vals, idx, fm
+
+    @staticmethod
+    def backward(ctx, dvals, _didx, _dfm):
+        logits, idx = ctx.saved_tensors
+        padded = torch.nn.functional.pad(logits, (1, 0), value=-1e3)
+        p = padded.softmax(dim=-1)[..., 1:]                     # -inf entries -> exactly 0
+        dfull = torch.zeros_like(p).scatter_add_(-1, idx.long(), dvals.to(p.dtype))
+        dl = p * (dfull - (p * dfull).sum(dim=-1, keepdim=True))
+        return dl, None
+
+
 def importance_topk(importance_logits: Tensor, num_selected: int):
     """softmax with the -1e3 pad column (NSA.py:693-695) + topk (NSA.py:713) + `> 1e-10` mask
-    (NSA.py:721).  Returns (values fp32, indices int32, fmask bool), each [..., num_selected]."""
-    idx, vals, fm = topk_op(importance_logits, int(num_selected), True)
+    (NSA.py:721).  Returns (values fp32, indices int32, fmask bool), each [..., num_selected];
+    `values` is differentiable with respect to the logits."""
+    if importance_logits.requires_grad:
+        vals, idx, fm = _ImportanceTopk.apply(importance_logits, int(num_selected))
+    else:
+        idx, vals, fm = topk_op(importance_logits, int(num_selected), True)
     return vals, idx, fm.view(torch.bool)
 
 

@@ -156,8 +156,6 @@ class SparseAttention(nn.Module):
         assert not (not self.causal and return_cache)
         if sliding_window_flex_mask is not None or fine_selection_flex_mask is not None:
             raise NotImplementedError("flex-attention masks are a different backend; the HIP kernels implement the same masks directly")
-        if self.use_diff_topk:
-            raise NotImplementedError("use_diff_topk (gradient through the selection gates) is not implemented in the HIP path")
         if not inp.is_cuda:
             raise RuntimeError("SparseAttention runs on the GPU only (HIP kernels, no CPU fallback)")
 
@@ -192,8 +190,10 @@ class SparseAttention(nn.Module):
 
         num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
         if num_sel > 0:
-            _, idx, fmask = ops.importance_topk(imp, num_sel)
-            f_out = ops.native_sparse_attend(rq16, rk16, v16, B, idx, fmask, include_block_causal=self.causal)
+            vals, idx, fmask = ops.importance_topk(imp, num_sel)
+            # straight-through gates (NSA.py:715): value 1, gradient flows into the importance scores
+            gates = (vals + (1. - vals).detach()) if self.use_diff_topk else None
+            f_out = ops.native_sparse_attend(rq16, rk16, v16, B, idx, fmask, sel_scale=gates, include_block_causal=self.causal)
         elif self.causal:
             # nothing selectable: block-diagonal causal attention (NSA.py:821-837)
             idx = torch.zeros((b, self.kv_heads, n, 0), dtype=torch.int32, device=inp.device)

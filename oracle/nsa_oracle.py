@@ -416,9 +416,14 @@ class SparseAttentionOracle(nn.Module):
         rq, rk = self.rotary_emb.rotate_queries_with_cached_keys(q, k)
         sel = self.select(csim)
         if selection_override is not None:
+            # the discrete choice comes from outside; values (for the gates) are re-read from this
+            # module's own importance scores at the given indices
             idx, live = selection_override
-            vals = None
-            f_out = select_attend(rq, rk, v, idx, live, B, causal=self.causal)
+            imp = importance_from_csim(csim, self.num_mem_compress_kv, self.num_grouped_queries,
+                                       self.query_heads_share_selected_kv, st, B)
+            vals = imp.gather(-1, idx.long())
+            gates = (vals + (1.0 - vals).detach()) if self.use_diff_topk else None
+            f_out = select_attend(rq, rk, v, idx, live, B, causal=self.causal, gates=gates)
         elif sel is not None:
             vals, idx = sel
             gates = (vals + (1.0 - vals).detach()) if self.use_diff_topk else None

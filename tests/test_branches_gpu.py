@@ -93,6 +93,29 @@ def test_compress_matches_oracle(b, hq, hk, n, d, st, B, mem, causal, share):
     assert_close(imp[~dead], want[~dead], 2e-3, 1e-3, "importance logits")
 
 
+def test_importance_logits_gradient_matches_oracle():
+    """gradient of the importance logits with respect to q and the compressed keys (needed by the
+    differentiable top-k, NSA.py:715) against autograd through the oracle's NSA.py:652-691."""
+    from native_sparse_attention_pytorch_amd.ops import compress_attend
+    for (b, hq, hk, n, d, st, B, mem, share) in [(1, 4, 2, 200, 64, 4, 16, 1, True), (1, 4, 2, 160, 64, 4, 32, 2, False)]:
+        g = torch.Generator().manual_seed(n)
+        nc = n // st
+        q = _rand((b, hq, n, d), g, d ** -0.25)
+        ck, cv = _rand((b, hk, mem + nc, d), g, d ** -0.25), _rand((b, hk, mem + nc, d), g)
+        qr, kr = q.float().requires_grad_(), ck.float().requires_grad_()
+        _, csim = O.attend(qr, kr, cv.float(), mask=O.compress_mask(n, nc, st, mem, True), return_sim=True)
+        want = O.importance_logits(csim, mem, hq // hk, share, st, B)
+        w = torch.randn(want.shape, generator=g)
+        live = want > -1e30
+        (want * w).masked_fill(~live, 0.0).sum().backward()
+        qg, kg = q.to(DEV).requires_grad_(), ck.to(DEV).requires_grad_()
+        _, imp = compress_attend(qg, kg, cv.to(DEV), mem, st, True, sel_block=B, share=share)
+        (imp * w.to(DEV)).masked_fill(~live.to(DEV), 0.0).sum().backward()
+        torch.cuda.synchronize()
+        _grad_close(qg.grad, qr.grad, "dq via importance")
+        _grad_close(kg.grad, kr.grad, "dck via importance")
+
+
 def test_topk_bit_exact_on_given_scores():
     from native_sparse_attention_pytorch_amd.ops import topk_op
     g = torch.Generator().manual_seed(0)

@@ -33,6 +33,8 @@ def _pair(seed, **kw):
 
 CONFIGS = [
     dict(dim=256, dim_head=64, heads=8, kv_heads=2, sliding_window_size=64, compress_block_size=16,
+         compress_block_sliding_stride=8, selection_block_size=32, num_selected_blocks=4, causal=True, use_diff_topk=True),
+    dict(dim=256, dim_head=64, heads=8, kv_heads=2, sliding_window_size=64, compress_block_size=16,
          compress_block_sliding_stride=8, selection_block_size=32, num_selected_blocks=4, causal=True),
     dict(dim=256, dim_head=128, heads=4, kv_heads=2, sliding_window_size=32, compress_block_size=32,
          compress_block_sliding_stride=16, selection_block_size=64, num_selected_blocks=3, causal=True),

@@ -90,6 +90,29 @@ def test_select_reference_script_contract():
     assert_close(kg.grad, kr.grad, 2e-2 * kr.grad.abs().max().item(), 5e-2, "dk")
 
 
+def test_select_gate_gradient_matches_oracle():
+    """sel_scale (straight-through top-k gates, value 1): its gradient against the oracle's
+    gather path with gates multiplying the selected keys (NSA.py:793-797); tolerance of
+    test_triton_nsa.py:194 scaled to the gradient's magnitude."""
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    for (b, hq, hk, n, d, B, S) in [(2, 4, 2, 300, 64, 16, 3), (1, 8, 2, 512, 128, 64, 4)]:
+        q, k, v, do = _inputs(b, hq, hk, n, d, seed=n)
+        idx, msk = causal_random_selection(b, hk, n, B, S, seed=5)
+        gr = torch.ones(b, hk, n, S, requires_grad=True)
+        qr, kr, vr = (t.float().requires_grad_() for t in (q, k, v))
+        ref = O.select_attend(qr, kr, vr, idx, msk, B, causal=True, gates=gr)
+        (ref * do.float()).sum().backward()
+        gg = torch.ones(b, hk, n, S, device=DEV, requires_grad=True)
+        qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+        out = native_sparse_attend(qg, kg, vg, B, idx.to(DEV), msk.to(DEV), sel_scale=gg)
+        (out.float() * do.to(DEV).float()).sum().backward()
+        torch.cuda.synchronize()
+        want = gr.grad * msk                       # dead slots: the oracle's masked logits carry no gradient either
+        assert_close(gg.grad, want, 2e-2 * want.abs().max().item() + 1e-6, 5e-2, "d sel_scale")
+        assert_close(qg.grad, qr.grad, 2e-2 * qr.grad.abs().max().item(), 5e-2, "dq with gates")
+        assert (gg.grad.cpu()[~msk] == 0).all()
+
+
 def test_select_strided_views_and_per_head_selection():
     """q/k/v as 'b n (h d) -> b h n d' views of one projection output (NSA.py:583-585) and
     selection per query head (query_heads_share_selected_kv=False, TRI.py:1961-1962)."""
