@@ -29,6 +29,11 @@ HBM_PEAK_GBS = 8000.0
 
 CFG = dict(batch=1, seq=32768, heads=32, kv_heads=8, dim_head=128, block=64, num_sel=15)
 
+# HBM bytes per launch on this workload, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
+# scaled by streaming kernels of known size (profiles/select_fwd_bwd_seq32k_hbm_traffic.txt)
+MEASURED_TRAFFIC_BYTES = {"fwd_block_walk": 7.391e9, "fwd_merge": 4.627e9, "bwd_dq_walk": 9.666e9, "bwd_dq_merge": 4.546e9,
+                          "bwd_dkv_walk": 9.207e9, "bwd_dkv_reduce": 0.547e9, "bwd_delta": 0.541e9}
+
 
 def selection(b, h, n, B, S, seed, device):
     """15 distinct causal blocks per query, uniform over the blocks before the query's own
@@ -166,9 +171,13 @@ def main():
     kflop = {"fwd_block_walk": 2 * flop_unit, "bwd_dkv_walk": 4 * flop_unit, "bwd_dq_walk": 1 * flop_unit}
     dom = max(kflop, key=lambda nm: kern[nm])
     achieved = kflop[dom] / (kern[dom] * 1e-3) / 1e12
+    traffic = MEASURED_TRAFFIC_BYTES.get(dom)
     roofline = dict(bound="mfma", kernel=dom, achieved=round(achieved, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
-                    frac=round(achieved / MFMA_PEAK_TFLOPS, 4), traffic=None,
-                    step_frac=round(value / MFMA_PEAK_TFLOPS, 4))
+                    frac=round(achieved / MFMA_PEAK_TFLOPS, 4), traffic=traffic,
+                    step_frac=round(value / MFMA_PEAK_TFLOPS, 4),
+                    # the kernels are HBM-bound in practice: measured bytes / measured time against 8 TB/s
+                    hbm_GBs={nm: round(MEASURED_TRAFFIC_BYTES[nm] / (kern[nm] * 1e-3) / 1e9, 1) for nm in MEASURED_TRAFFIC_BYTES},
+                    hbm_frac_step=round(sum(MEASURED_TRAFFIC_BYTES.values()) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4))
 
     res = dict(metric="NSA selection-attention fwd+bwd TFLOP/s at seq 32k (bf16)", value=round(value, 2), unit="TFLOP/s",
                n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_step, 4), higher_is_better=True,
