@@ -166,6 +166,21 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     scale = fq.shape[-1] ** -0.5
     out, lse, _ = select_fwd(fq.to(_BF16), fk.to(_BF16), fv.to(_BF16), selected_block_indices, fmask, sel_scale,
                              int(block_size), bool(include_block_causal), float(scale))
+    if not include_block_causal and selected_block_indices.shape[-1] > 0:
+        # A query whose slots are all dead attends nothing in the kernel.  The reference's torch
+        # path (NSA.py:809-815) fills every logit of such a row with the same value, i.e. it
+        # attends uniformly over the keys of the (dead) slots' blocks, zero padding included;
+        # reproduce that corner with a few elementwise ops (no sync, differentiable in v).
+        b, hs, n, S = selected_block_indices.shape
+        hk2, d = fk.shape[1], fk.shape[-1]
+        W = (n + block_size - 1) // block_size
+        vpad = torch.nn.functional.pad(fv, (0, 0, 0, W * block_size - n)).reshape(b, hk2, W, block_size, d)
+        vmean = vpad.float().mean(dim=3)                                                  # [b,hk,W,d]
+        gi = selected_block_indices.long().clamp(0, W - 1).reshape(b, hs, n * S, 1).expand(-1, -1, -1, d)
+        avg = vmean.gather(2, gi).reshape(b, hs, n, S, d).mean(dim=3)                     # [b,hk,n,d]
+        dead = ~fmask.bool().any(dim=-1)                                                  # [b,hk,n]
+        g = q_heads // hs
+        out = torch.where(dead.repeat_interleave(g, dim=1)[..., None], avg.repeat_interleave(g, dim=1).to(out.dtype), out)
     out = out.to(dtype)
     return (out, lse) if return_lse else out
 
