@@ -141,8 +141,8 @@ int nsa_gate_bwd(int32_t batch, int32_t heads, int32_t seq, int32_t dim_head, co
 /* Same as nsa_select_fwd / nsa_select_bwd, additionally recording the caller's hipEvent_t
  * handles (created with timing enabled) between the kernels of the call, so that a benchmark
  * can time each kernel on the launch stream.  Events: fwd {start, after block walk, after
- * merge}; bwd {start, after delta, after dQ walk, after dQ merge, after dK/dV walk, after dK/dV
- * reduce}.  NULL entries are skipped.  No reference counterpart (measurement hook). */
+ * merge}; bwd {start, after delta, after the separate dQ walk (only run when sel_grads is
+ * requested), after the dK/dV(+dQ) walk, after dQ merge, after dK/dV reduce}.  NULL entries are skipped.  No reference counterpart (measurement hook). */
 int nsa_select_fwd_timed(const nsa_select_desc* d, const void* q, const void* k, const void* v,
                          const void* idx, const uint8_t* fmask, const void* index_ws, void* fwd_ws, size_t fwd_bytes,
                          void* out, float* lse, void* stream, void* const* events, int num_events);

@@ -699,17 +699,29 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 // lane <-> key and registers <-> rows, which is the B-operand layout of dV^T = dO^T P and
 // dK^T = Q^T dS; dO^T and Q^T (lane <-> feature, k <-> rows) are read from the LDS tiles with
 // the hardware transpose load.
-template <int D, int KT>
+//
+// With FUSE_DQ the walk also produces the dQ partial of every pair (so the separate dQ walk and
+// its second gather of Q and dO are not needed): each wave stores its dS (32 keys x 32 rows) as
+// [key][row] in LDS; dQ^T = K^T dS^T is then formed with both operands read through the
+// transpose load (K block row-major in LDS, loaded once per unit), each wave taking half of the
+// features, and the finished 32 x D tile leaves through coalesced row stores.
+template <int D, int KT, bool FUSE_DQ>
 __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                               const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
                                                               const float* __restrict__ lse, const float* __restrict__ delta,
                                                               const char* __restrict__ iws, char* __restrict__ bws) {
   constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
+  constexpr int RST = 32 + 8;                  // row stride of the [key][row] dS tile
+  constexpr int DTW = DT / KT;                 // feature tiles of dQ per wave
   __shared__ __align__(16) float lse_s[32];
   __shared__ __align__(16) float del_s[32];
   __shared__ __align__(16) int lim_s[32];
   __shared__ __align__(16) __bf16 xq_s[32 * RS];
   __shared__ __align__(16) __bf16 xg_s[32 * RS];
+  __shared__ __align__(16) __bf16 kb_s[FUSE_DQ ? 32 * KT * RS : 8];     // the K block, row-major
+  __shared__ __align__(16) __bf16 ds_s[FUSE_DQ ? 32 * KT * RST : 8];    // dS^T: [key][row]
+  __shared__ __align__(16) __bf16 dq_s[FUSE_DQ ? 32 * RS : 8];          // finished dQ tile, row-major
+  __shared__ size_t row_s[32];
   const int kt = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
@@ -732,6 +744,10 @@ __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, c
       Kf[ks] = ok ? load8(kp + 16 * ks) : zero_frag();
       Vf[ks] = ok ? load8(vp + 16 * ks) : zero_frag();
     }
+    if (FUSE_DQ) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<bf16x8*>(kb_s + kl * RS + 16 * ks + 8 * h) = Kf[ks];
+    }
   }
   floatx16 dKa[DT], dVa[DT];
 #pragma unroll
@@ -742,6 +758,7 @@ __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, c
   const int HQ = P.hkv * P.g;
   const __bf16* qbase = q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1];
   const __bf16* gbase = dout + b * P.so[0] + (long)(hk * P.g) * P.so[1];
+  __bf16* dqpart = reinterpret_cast<__bf16*>(bws + P.off_dqpart);
 
   RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + ppt, n_);
   RowInfo r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0, n_), n_);
@@ -764,6 +781,7 @@ __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, c
       lse_s[n_] = r.valid ? lse_r : INFINITY;              // +inf: a padding row gets p = 0
       del_s[n_] = del_r;
       lim_s[n_] = r.lim;
+      if (FUSE_DQ) row_s[n_] = r.valid ? (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g : P.prow;
     }
     __syncthreads();
 
@@ -802,6 +820,16 @@ __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, c
     }
     const bf16x8 Pf0 = pack8(Sa, 0), Pf1 = pack8(Sa, 8);
     const bf16x8 Sf0 = pack8(dSa, 0), Sf1 = pack8(dSa, 8);
+    if (FUSE_DQ) {
+      // dS^T[key kl][row 8a + 4h + bb]: four consecutive rows per 8-byte store
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        bf16x4 t4;
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) t4[bb] = (__bf16)dSa[4 * a + bb];
+        *reinterpret_cast<bf16x4*>(ds_s + kl * RST + 8 * a + 4 * h) = t4;
+      }
+    }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 0, 32 * dt, lane), Pf0, dVa[dt]);
@@ -810,6 +838,38 @@ __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, c
       dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 16, 32 * dt, lane), Sf1, dKa[dt]);
     }
     __syncthreads();
+    if (FUSE_DQ) {
+      // dQ^T[feature][row] = sum_key K^T[feature][key] dS^T[key][row]; this wave: features 32*DTW*kt ...
+      floatx16 Qa[DTW];
+#pragma unroll
+      for (int w = 0; w < DTW; ++w) Qa[w] = zero_acc();
+#pragma unroll
+      for (int k0 = 0; k0 < 32 * KT; k0 += 16) {
+        const bf16x8 Sf = lds_transposed_operand(ds_s, RST, k0, 0, lane);          // lane <-> row, k <-> keys k0 ..
+#pragma unroll
+        for (int w = 0; w < DTW; ++w)
+          Qa[w] = mfma32(lds_transposed_operand(kb_s, RS, k0, 32 * (DTW * kt + w), lane), Sf, Qa[w]);
+      }
+      // Qa[w][4a + bb] = dQ[row n_][feature 32(DTW kt + w) + 8a + 4h + bb]
+#pragma unroll
+      for (int w = 0; w < DTW; ++w)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          bf16x4 t4;
+#pragma unroll
+          for (int bb = 0; bb < 4; ++bb) t4[bb] = (__bf16)(Qa[w][4 * a + bb] * P.scale);
+          *reinterpret_cast<bf16x4*>(dq_s + n_ * RS + 32 * (DTW * kt + w) + 8 * a + 4 * h) = t4;
+        }
+      __syncthreads();
+      constexpr int CPR = D / 8, RPI = (64 * KT) / CPR;
+#pragma unroll
+      for (int t = 0; t < 32 / RPI; ++t) {
+        const int rr = t * RPI + (int)threadIdx.x / CPR, c = threadIdx.x % CPR;
+        const bf16x8 vv = *reinterpret_cast<const bf16x8*>(dq_s + rr * RS + 8 * c);
+        *reinterpret_cast<bf16x8*>(dqpart + row_s[rr] * D + 8 * c) = vv;
+      }
+      __syncthreads();
+    }
     lse_r = lse_n; del_r = del_n;
     r = rn; e_n = e_nn;
   }
@@ -948,21 +1008,26 @@ static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void
   hipLaunchKernelGGL((sel_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, delta);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 1, st);
-  if (sel_grads) {
+  // without gate gradients the dQ partials come out of the dK/dV walk (one gather of Q and dO
+  // instead of two); with them the separate dQ walk, which also emits sel_grads, is used
+  const bool fused = sel_grads == nullptr;
+  if (!fused) {
     hipLaunchKernelGGL((sel_bwd_dq_kernel<D, KT, true>), dim3(xcd_grid(P, 1)), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                        (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws, sel_grads);
+    NSA_LAUNCH_CHECK();
+  }
+  mark(ev, nev, 2, st);
+  if (fused) {
+    hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT, true>), dim3(P.ub_kv, P.bh), dim3(64 * KT), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+                       (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
   } else {
-    hipLaunchKernelGGL((sel_bwd_dq_kernel<D, KT, false>), dim3(xcd_grid(P, 1)), dim3(64), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
-                       (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws, sel_grads);
+    hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT, false>), dim3(P.ub_kv, P.bh), dim3(64 * KT), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+                       (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
   }
   NSA_LAUNCH_CHECK();
-  mark(ev, nev, 2, st);
+  mark(ev, nev, 3, st);
   const long nq = (long)P.bh * P.n;
   hipLaunchKernelGGL((sel_bwd_dq_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)bws, (__bf16*)dq, sel_grads);
-  NSA_LAUNCH_CHECK();
-  mark(ev, nev, 3, st);
-  hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT>), dim3(P.ub_kv, P.bh), dim3(64 * KT), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
-                     (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 4, st);
   hipLaunchKernelGGL((sel_bwd_dkv_reduce_kernel<D, KT>), dim3(P.W, P.bh), dim3(256), 0, st, P, (const char*)iws, (const char*)bws, (__bf16*)dk, (__bf16*)dv);
