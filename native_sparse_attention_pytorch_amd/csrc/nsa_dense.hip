@@ -75,7 +75,7 @@ __device__ __forceinline__ TileWalk make_walk(const DensePlan& P, int i_first, i
 // ------------------------------------------------------------------------------- forward
 // NPF = selection block / compress stride when the importance logits are wanted, 0 otherwise
 template <int D, int NPF>
-__global__ __launch_bounds__(256) void dense_fwd_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+__global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                         const __bf16* __restrict__ v, __bf16* __restrict__ out, float* __restrict__ lse,
                                                         float* __restrict__ pooled) {
   constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
@@ -308,7 +308,7 @@ __global__ __launch_bounds__(256) void dense_delta_kernel(const DensePlan P, con
 // dQ, query-stationary (same tile walk as the forward): dS^T = P^T o (V dO^T - delta),
 // dQ^T += K^T dS^T with K^T read through the LDS transpose load.
 template <int D>
-__global__ __launch_bounds__(256) void dense_bwd_dq_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+__global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                            const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
                                                            const float* __restrict__ lse, const float* __restrict__ delta, __bf16* __restrict__ dq) {
   constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
