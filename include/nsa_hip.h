@@ -138,6 +138,14 @@ int nsa_gate_bwd(int32_t batch, int32_t heads, int32_t seq, int32_t dim_head, co
                  const void* s, const int64_t* s_stride, const void* d_out,
                  void* d_logits, void* dc, void* df, void* ds, void* stream);
 
+/* Rotary position embedding of queries or keys.  Replaces rotary_emb.rotate_queries_with_cached_keys
+ * (NSA.py:643; third-party rotary_embedding_torch defaults: feature pairs (2k, 2k+1) rotated by
+ * (i + offset) * freqs[k], fp32 arithmetic).  x: bf16 [batch, heads, seq, d] with element strides
+ * {batch, head, token}; freqs: fp32 [d/2]; out: bf16 contiguous.  inverse != 0 rotates by the negative
+ * angle (the backward). */
+int nsa_rope(const void* x, const int64_t* x_stride, int32_t batch, int32_t heads, int32_t seq, int32_t dim_head,
+             const float* freqs, int32_t offset, int32_t inverse, void* out, void* stream);
+
 /* Same as nsa_select_fwd / nsa_select_bwd, additionally recording the caller's hipEvent_t
  * handles (created with timing enabled) between the kernels of the call, so that a benchmark
  * can time each kernel on the launch stream.  Events: fwd {start, after block walk, after

@@ -60,6 +60,8 @@ def lib():
         i3 = C.POINTER(C.c_int64)
         L.nsa_gate_fwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp]
         L.nsa_gate_bwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp, vp, vp, vp, vp]
+        L.nsa_rope.argtypes = [vp, i3, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, C.c_int32, C.c_int32, vp, vp]
+        L.nsa_rope.restype = C.c_int
         for name in ("nsa_dense_workspace_bytes", "nsa_dense_fwd", "nsa_dense_bwd", "nsa_topk", "nsa_gate_fwd", "nsa_gate_bwd"):
             getattr(L, name).restype = C.c_int
         for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):

@@ -439,3 +439,40 @@ def gate_combine(logits: Tensor, compressed: Tensor, selected: Tensor, sliding: 
     """sigmoid(logits) 'b n (h s) -> b h n s' weighted sum of the three branches, merged to
     'b n (h d)' (NSA.py:323-327, 854-860).  logits are the pre-sigmoid gate projection."""
     return gate_fwd(logits.to(_BF16), compressed, selected, sliding)
+
+
+# ---------------------------------------------------------------------------------- rotary
+
+@torch.library.custom_op("nsa_amd::rope", mutates_args=())
+def rope_op(x: Tensor, freqs: Tensor, offset: int, inverse: bool) -> Tensor:
+    x = _prep(x)
+    b, h, n, d = x.shape
+    freqs = freqs.detach().to(torch.float32).contiguous()
+    out = torch.empty((b, h, n, d), dtype=_BF16, device=x.device)
+    _lib.check(_lib.lib().nsa_rope(_ptr(x), _s3(x), b, h, n, d, _ptr(freqs), int(offset), int(inverse), _ptr(out), _stream()), "nsa_rope")
+    return out
+
+
+@rope_op.register_fake
+def _(x, freqs, offset, inverse):
+    return x.new_empty(x.shape)
+
+
+def _rope_setup(ctx, inputs, output):
+    _, freqs, offset, inverse = inputs
+    ctx.save_for_backward(freqs)
+    ctx.args = (offset, inverse)
+
+
+def _rope_backward(ctx, dout):
+    (freqs,) = ctx.saved_tensors
+    offset, inverse = ctx.args
+    return rope_op(dout if dout.dtype == _BF16 else dout.to(_BF16), freqs, offset, not inverse), None, None, None
+
+
+rope_op.register_autograd(_rope_backward, setup_context=_rope_setup)
+
+
+def rotary(x: Tensor, freqs: Tensor, offset: int = 0) -> Tensor:
+    """Rotary embedding of 'b h n d' queries or keys at positions offset .. offset+n-1 (NSA.py:643)."""
+    return rope_op(x, freqs, int(offset), False)

@@ -185,8 +185,10 @@ class SparseAttention(nn.Module):
         c_out, imp = ops.compress_attend(q.to(bf16), ck.to(bf16), cv.to(bf16), M, st, self.causal,
                                          sel_block=B if want_sel else None, share=share)
 
-        rq, rk = self.rotary_emb.rotate_queries_with_cached_keys(q, k)
-        rq16, rk16, v16 = rq.to(bf16), rk.to(bf16), v.to(bf16)
+        # rotary positions for the selection and sliding branches (NSA.py:643), one HIP kernel each
+        rq16 = ops.rotary(q.to(bf16), self.rotary_emb.freqs)
+        rk16 = ops.rotary(k.to(bf16), self.rotary_emb.freqs)
+        v16 = v.to(bf16)
 
         num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
         if num_sel > 0:
@@ -216,4 +218,4 @@ class SparseAttention(nn.Module):
         run_k, run_v = k, v
         if co > 0:
             run_k, run_v = F.pad(run_k, (0, 0, co, 0)), F.pad(run_v, (0, 0, co, 0))
-        return out, ((rk, v), ((ck0, cv0), (run_k[..., L:, :], run_v[..., L:, :])))
+        return out, ((rk16.to(k.dtype), v), ((ck0, cv0), (run_k[..., L:, :], run_v[..., L:, :])))

@@ -171,3 +171,29 @@ def test_gate_combine_matches_oracle(b, h, n, d):
     assert_close(out, ref, 2e-2, 1e-2, "gate out")
     for name, a, r in zip(("dlogits", "dc", "df", "ds"), gins, ins):
         _grad_close(a.grad, r.grad, name)
+
+
+@pytest.mark.parametrize("b,h,n,d,offset,view", [(2, 4, 300, 64, 0, False), (1, 2, 515, 128, 0, True), (1, 4, 64, 64, 40000, False)])
+def test_rotary_matches_oracle(b, h, n, d, offset, view):
+    """Rotary kernel against the oracle's fp32 restatement, forward and backward, on a contiguous
+    tensor and on the 'b n (h d) -> b h n d' view the qkv projection hands over; large positions
+    exercise the sine / cosine range reduction.  One bf16 rounding of an O(1) value: 1e-2 abs."""
+    from native_sparse_attention_pytorch_amd.ops import rotary
+    g = torch.Generator().manual_seed(n + d)
+    rot = O.RotaryEmbedding(d)
+    if view:
+        base = _rand((b, n, h * d), g)
+        x = base.view(b, n, h, d).permute(0, 2, 1, 3)
+    else:
+        x = _rand((b, h, n, d), g)
+    do = _rand((b, h, n, d), g)
+    xr = x.float().requires_grad_()
+    ref = rot.rotate(xr, offset=offset)
+    (ref * do.float()).sum().backward()
+    xg = x.to(DEV).requires_grad_()
+    out = rotary(xg, rot.freqs.to(DEV), offset)
+    (out.float() * do.to(DEV).float()).sum().backward()
+    torch.cuda.synchronize()
+    assert out.is_contiguous()
+    assert_close(out, ref, 1.6e-2 * ref.abs().max().item(), 1e-2, "rotary out")
+    _grad_close(xg.grad, xr.grad, "rotary dx")
