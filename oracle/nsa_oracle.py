@@ -320,8 +320,10 @@ def sliding_attend(q, k, v, window, causal=True, chunk=1024):
 
 class SparseAttentionOracle(nn.Module):
     """Restatement of SparseAttention (NSA.py:188-336 construction, :549-867 forward) with
-    identical constructor arguments, parameter names and creation order.  Training / prefill
-    path only (no cache)."""
+    identical constructor arguments, parameter names and creation order, plus the
+    single-token decode step over the three caches (NSA.py:338-547).  The decode restatement
+    is pinned by the reference's own criterion (tests/test_sparse_attn.py:50-86): token-by-
+    token outputs equal the parallel forward to 1e-5 in fp32."""
 
     def __init__(self, dim, dim_head, heads, sliding_window_size, compress_block_size,
                  compress_block_sliding_stride, selection_block_size, num_selected_blocks,
@@ -403,9 +405,14 @@ class SparseAttentionOracle(nn.Module):
             return None
         return topk_lower_index_first(imp, num_sel)
 
-    def forward(self, inp, return_parts=False, selection_override=None):
+    def forward(self, inp, return_parts=False, selection_override=None, cache=None, return_cache=False):
         """selection_override = (idx, fmask) replaces the module's own top-k result (used to
-        compare implementations under an identical discrete selection)."""
+        compare implementations under an identical discrete selection).  With `cache` the
+        input is one token and the decode step runs (NSA.py:559-563)."""
+        if cache is not None:
+            assert inp.shape[1] == 1
+            return self.forward_inference(inp, cache, return_cache=return_cache, selection_override=selection_override)
+        assert self.causal or not return_cache
         b, n, _ = inp.shape
         st, B = self.compress_block_sliding_stride, self.selection_block_size
         x, q, k, v = self.project(inp)
@@ -438,7 +445,98 @@ class SparseAttentionOracle(nn.Module):
         if return_parts:
             return y, dict(q=q, k=k, v=v, rq=rq, rk=rk, ck=ck, cv=cv, csim=csim, c_out=c_out,
                            idx=idx, vals=vals, f_out=f_out, s_out=s_out, gate=gate)
+        if return_cache:
+            # NSA.py:605-619, 863-867: rotated keys and values; compressed keys without the
+            # memory slots; the raw tokens after the last complete stride, preceded by the
+            # window overlap (zeros left of token 0)
+            M, cbs = self.num_mem_compress_kv, self.compress_block_size
+            L = (n // st) * st
+            run_k = F.pad(k, (0, 0, cbs - st, 0))[..., L:, :]
+            run_v = F.pad(v, (0, 0, cbs - st, 0))[..., L:, :]
+            return y, ((rk, v), ((ck[..., M:, :], cv[..., M:, :]), (run_k, run_v)))
         return y
+
+    def forward_inference(self, inp, cache, return_cache=True, selection_override=None):
+        """One decode step (NSA.py:338-547).  inp [b,1,dim]; cache as returned by `forward`.
+        The token at position t = cached length attends to: every cached compressed key (plus the
+        memory slots, unless there is none cached: then that branch is zero); the top blocks
+        by importance plus the keys of its own block up to itself; its last window+1 keys."""
+        assert self.causal
+        (cache_k, cache_v), ((ck, cv), (run_k, run_v)) = cache
+        b, t = inp.shape[0], cache_k.shape[-2]
+        G, B, st, cbs, M = self.num_grouped_queries, self.selection_block_size, self.compress_block_sliding_stride, self.compress_block_size, self.num_mem_compress_kv
+        x, q, k, v = self.project(inp)
+        run_k, run_v = torch.cat((run_k, k), dim=-2), torch.cat((run_v, v), dim=-2)     # un-rotated (NSA.py:377-380)
+        rq, rk = self.rotary_emb.rotate(q, offset=t), self.rotary_emb.rotate(k, offset=t)
+        keys, vals_ = torch.cat((cache_k, rk), dim=-2), torch.cat((cache_v, v), dim=-2)
+
+        # compressed branch (NSA.py:396-420): no mask, every cached block is complete
+        nc = ck.shape[-2]
+        if nc > 0:
+            ak = torch.cat((self.compress_mem_kv[0][None].expand(b, -1, -1, -1), ck), dim=-2)
+            av = torch.cat((self.compress_mem_kv[1][None].expand(b, -1, -1, -1), cv), dim=-2)
+            csim = torch.einsum('bhgd,bhjd->bhgj', q.reshape(b, self.kv_heads, G, -1), ak) * self.scale
+            c_out = torch.einsum('bhgj,bhjd->bhgd', csim.softmax(dim=-1), av).reshape(b, self.heads, 1, -1)
+            imp = csim[..., M:]                                                        # [b, hk, G, nc]
+        else:
+            c_out = torch.zeros_like(q)
+            imp = q.new_zeros(b, self.kv_heads, G, 0)
+
+        # a window of cbs raw tokens is complete: compress it and keep the overlap (NSA.py:422-441)
+        if run_k.shape[-2] % cbs == 0:
+            nk = self.k_compress((run_k + self.k_intrablock_positions)[:, :, None])
+            nv = self.v_compress((run_v + self.v_intrablock_positions)[:, :, None])
+            keep = cbs - st
+            run_k, run_v = run_k[..., cbs - keep:, :], run_v[..., cbs - keep:, :]
+            ck, cv = torch.cat((ck, nk), dim=-2), torch.cat((cv, nv), dim=-2)
+
+        # selection branch (NSA.py:446-515)
+        npf = B // st
+        nb = nc // npf if st != B else nc
+        imp = imp[..., :nb * npf].reshape(b, self.kv_heads, G, nb, npf).mean(dim=-1) if st != B else imp
+        num_sel = min(self.num_selected_blocks, nb)
+        own = (t % B) + 1                                                              # keys of the own block, itself included
+        seg_k, seg_v = [keys[..., -own:, :]], [vals_[..., -own:, :]]
+        live = None
+        qg = rq.reshape(b, self.kv_heads, G, -1)
+        if num_sel > 0:
+            if self.query_heads_share_selected_kv:
+                imp = imp.mean(dim=2, keepdim=True)                                    # [b, hk, 1, nb]
+            probs = F.pad(imp, (1, 0), value=-1e3).softmax(dim=-1)[..., 1:]
+            if selection_override is not None:
+                idx, lv = selection_override
+                idx, lv = idx.reshape(probs.shape[:-1] + (-1,)).long(), lv.reshape(probs.shape[:-1] + (-1,))
+            else:
+                sv, idx = topk_lower_index_first(probs, num_sel)
+                lv = sv > 1e-10
+            W = -(-(t + 1) // B)
+            kb = F.pad(keys, (0, 0, 0, W * B - (t + 1))).reshape(b, self.kv_heads, 1, W, B, -1)
+            vb = F.pad(vals_, (0, 0, 0, W * B - (t + 1))).reshape(b, self.kv_heads, 1, W, B, -1)
+            gi = idx[..., None, None].expand(-1, -1, -1, -1, B, kb.shape[-1])
+            sk = kb.expand(-1, -1, idx.shape[2], -1, -1, -1).gather(3, gi).flatten(3, 4)   # [b, hk, 1|G, sel*B, d]
+            sv_ = vb.expand(-1, -1, idx.shape[2], -1, -1, -1).gather(3, gi).flatten(3, 4)
+            live = torch.cat((lv.repeat_interleave(B, dim=-1), lv.new_ones(lv.shape[:-1] + (own,))), dim=-1)
+            fk = torch.cat((sk, seg_k[0][:, :, None].expand(-1, -1, sk.shape[2], -1, -1)), dim=-2)
+            fv = torch.cat((sv_, seg_v[0][:, :, None].expand(-1, -1, sk.shape[2], -1, -1)), dim=-2)
+            fsim = torch.einsum('bhgd,bhgjd->bhgj', qg, fk.expand(-1, -1, G, -1, -1)) * self.scale
+            fsim = fsim.masked_fill(~live.expand_as(fsim), _neg_max(fsim))
+            f_out = torch.einsum('bhgj,bhgjd->bhgd', fsim.softmax(dim=-1), fv.expand(-1, -1, G, -1, -1))
+        else:
+            fsim = torch.einsum('bhgd,bhjd->bhgj', qg, seg_k[0]) * self.scale
+            f_out = torch.einsum('bhgj,bhjd->bhgd', fsim.softmax(dim=-1), seg_v[0])
+        f_out = f_out.reshape(b, self.heads, 1, -1)
+
+        # sliding branch (NSA.py:519-530): the last window+1 keys
+        wk, wv = keys[..., -(self.sliding_window_size + 1):, :], vals_[..., -(self.sliding_window_size + 1):, :]
+        ssim = torch.einsum('bhgd,bhjd->bhgj', qg, wk) * self.scale
+        s_out = torch.einsum('bhgj,bhjd->bhgd', ssim.softmax(dim=-1), wv).reshape(b, self.heads, 1, -1)
+
+        gate = self.to_strategy_combine(x).reshape(b, 1, self.heads, 3).permute(0, 2, 1, 3)
+        out = gate[..., 0:1] * c_out + gate[..., 1:2] * f_out + gate[..., 2:3] * s_out
+        y = self.combine_heads(merge_heads(out))
+        if not return_cache:
+            return y
+        return y, ((keys, vals_), ((ck, cv), (run_k, run_v)))
 
 
 def gate_combine(logits, c_out, f_out, s_out):
@@ -460,7 +558,9 @@ def _feed_forward(dim, expansion_factor=4.0):
 class TransformerOracle(nn.Module):
     """Restatement of the reference's training forward, transformer.py:142-211 (construction
     order: token_emb, per layer [attention, feed-forward], norm, to_logits) and :254-330
-    (ids[:, :-1] -> logits, cross entropy against ids[:, 1:])."""
+    (ids[:, :-1] -> logits, cross entropy against ids[:, 1:]; with a cache only the last token
+    is embedded and every layer takes its decode step), and of greedy / temperature sampling
+    with or without the caches (transformer.py:213-252)."""
 
     def __init__(self, num_tokens, dim, depth, dim_head=64, heads=8, kv_heads=None, ff_expansion_factor=4.0,
                  causal=True, sparse_attn_kwargs=None):
@@ -474,14 +574,43 @@ class TransformerOracle(nn.Module):
         self.norm = nn.RMSNorm(dim)
         self.to_logits = nn.Linear(dim, num_tokens, bias=False)
 
-    def forward(self, ids, return_loss=False):
+    def forward(self, ids, return_loss=False, cache=None, return_cache=False):
         if return_loss:
             ids, labels = ids[:, :-1], ids[:, 1:]
-        tokens = self.token_emb(ids)
+        tokens = self.token_emb(ids if cache is None else ids[:, -1:])
+        layer_caches = iter(cache or [])
+        next_cache = []
         for attn, ff in self.layers:
-            tokens = attn(tokens) + tokens
+            if return_cache or cache is not None:
+                attn_out, lc = attn(tokens, cache=next(layer_caches, None), return_cache=True)
+                next_cache.append(lc)
+            else:
+                attn_out = attn(tokens)
+            tokens = attn_out + tokens
             tokens = ff(tokens) + tokens
         logits = self.to_logits(self.norm(tokens))
         if not return_loss:
-            return logits
+            return (logits, next_cache) if return_cache else logits
         return F.cross_entropy(logits.transpose(1, 2), labels)
+
+    @torch.no_grad()
+    def sample(self, prompt, seq_len, temperature=1.0, filter_thres=0.9, use_cache_kv=False):
+        """transformer.py:213-252: extend `prompt` to seq_len tokens; temperature <= 0 is greedy,
+        otherwise gumbel sampling over the top (1 - filter_thres) share of the vocabulary
+        (transformer.py:45-62).  Returns only the new tokens."""
+        out, cache = prompt.clone(), None
+        for _ in range(max(0, seq_len - prompt.shape[-1])):
+            logits, next_cache = self.forward(out, cache=cache, return_cache=True)
+            if use_cache_kv:
+                cache = next_cache
+            logits = logits[:, -1]
+            if temperature <= 0.0:
+                tok = logits.argmax(dim=-1, keepdim=True)
+            else:
+                kk = math.ceil((1.0 - filter_thres) * logits.shape[-1])
+                val, ind = logits.topk(kk, dim=-1)
+                logits = torch.full_like(logits, float('-inf')).scatter(-1, ind, val)
+                noise = -torch.log(-torch.log(torch.rand_like(logits).clamp_min(1e-20)).clamp_min(1e-20))
+                tok = (logits / max(temperature, 1e-10) + noise).argmax(dim=-1, keepdim=True)
+            out = torch.cat((out, tok), dim=-1)
+        return out[..., prompt.shape[-1]:]

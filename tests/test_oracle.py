@@ -367,3 +367,66 @@ def test_gate_combine_closed_form():
         g = torch.sigmoid(logits[:, :, hh * 3:hh * 3 + 3])                  # column h*3+s
         want = g[..., 0:1] * c[:, hh] + g[..., 1:2] * f[:, hh] + g[..., 2:3] * s[:, hh]
         assert torch.allclose(got[:, :, hh * d:(hh + 1) * d], want, atol=1e-6)
+
+
+# ------------------------------------------------------------------ decode step (NSA.py:338-547)
+
+@pytest.mark.parametrize("seq_len", (2, 8, 16, 45))
+@pytest.mark.parametrize("num_selected_blocks", (0, 2))
+@pytest.mark.parametrize("stride", (2, 4))
+@pytest.mark.parametrize("block", (8, 16, 20))
+@pytest.mark.parametrize("share,kv_heads", ((True, 8), (True, 2), (False, 4)))
+def test_decode_steps_equal_parallel_forward(seq_len, num_selected_blocks, stride, block, share, kv_heads):
+    """The reference's own criterion for its decode path (tests/test_sparse_attn.py:50-86, same
+    grid plus a longer sequence, grouped heads and per-head selection): feeding the tokens one at
+    a time through the caches reproduces the parallel forward to 1e-5.  The two code paths share
+    no masking or gathering logic, so an off-by-one in either shows up here."""
+    torch.manual_seed(seq_len + stride + block)
+    m = O.SparseAttentionOracle(dim=64, dim_head=16, heads=8, kv_heads=kv_heads, causal=True, sliding_window_size=2,
+                                compress_block_size=5, selection_block_size=block, num_selected_blocks=num_selected_blocks,
+                                compress_block_sliding_stride=stride, query_heads_share_selected_kv=share)
+    with torch.no_grad():       # away from the symmetric init, but memory slots stay zero as the reference's test has them
+        m.to_strategy_combine[0].weight.normal_(std=0.3)
+        m.k_intrablock_positions.normal_()
+        m.v_intrablock_positions.normal_()
+    x = torch.randn(2, seq_len, 64)
+    parallel = m(x)
+    cache, outs = None, []
+    for i in range(seq_len):
+        o, cache = m(x[:, i:i + 1], cache=cache, return_cache=True)
+        outs.append(o)
+    (ck, cv), (run_k, run_v) = cache[1]
+    assert cache[0][0].shape[-2] == seq_len and ck.shape[-2] == seq_len // stride
+    assert run_k.shape[-2] == (5 - stride) + seq_len % stride
+    assert torch.allclose(parallel, torch.cat(outs, dim=1), atol=1e-5)
+
+
+def test_decode_from_prefill_cache():
+    """A prompt through the parallel forward with return_cache, then decode steps: the outputs
+    equal the parallel forward of the whole sequence (cache layout of NSA.py:605-619, 863-867)."""
+    torch.manual_seed(3)
+    m = O.SparseAttentionOracle(dim=64, dim_head=16, heads=4, kv_heads=2, causal=True, sliding_window_size=3,
+                                compress_block_size=8, selection_block_size=8, num_selected_blocks=2, compress_block_sliding_stride=4)
+    x = torch.randn(1, 37, 64)
+    full = m(x)
+    for p in (1, 6, 19, 32):
+        y, cache = m(x[:, :p], return_cache=True)
+        outs = [y]
+        for i in range(p, 37):
+            o, cache = m(x[:, i:i + 1], cache=cache, return_cache=True)
+            outs.append(o)
+        assert torch.allclose(full, torch.cat(outs, dim=1), atol=1e-5), p
+
+
+@pytest.mark.parametrize("block", (4, 8))
+def test_transformer_sampling_with_and_without_cache(block):
+    """tests/test_sparse_attn.py:88-118: greedy sampling gives the same tokens whether every step
+    re-runs the whole prefix or advances the caches."""
+    torch.manual_seed(0)
+    model = O.TransformerOracle(num_tokens=256, dim=64, depth=2, dim_head=16, heads=4, causal=True,
+                                sparse_attn_kwargs=dict(sliding_window_size=16, compress_block_size=4, compress_block_sliding_stride=2,
+                                                        selection_block_size=block, num_selected_blocks=2))
+    prompt = torch.randint(0, 256, (1, 1))
+    a = model.sample(prompt, 48, temperature=0.0, use_cache_kv=False)
+    c = model.sample(prompt, 48, temperature=0.0, use_cache_kv=True)
+    assert a.shape == (1, 47) and torch.equal(a, c)
