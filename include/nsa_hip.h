@@ -141,10 +141,39 @@ int nsa_gate_bwd(int32_t batch, int32_t heads, int32_t seq, int32_t dim_head, co
 /* Rotary position embedding of queries or keys.  Replaces rotary_emb.rotate_queries_with_cached_keys
  * (NSA.py:643; third-party rotary_embedding_torch defaults: feature pairs (2k, 2k+1) rotated by
  * (i + offset) * freqs[k], fp32 arithmetic).  x: bf16 [batch, heads, seq, d] with element strides
- * {batch, head, token}; freqs: fp32 [d/2]; out: bf16 contiguous.  inverse != 0 rotates by the negative
- * angle (the backward). */
+ * {batch, head, token}; freqs: fp32 [d/2]; out: bf16 with element strides out_stride (NULL: contiguous;
+ * a slot of a key cache otherwise, NSA.py:384-390).  inverse != 0 rotates by the negative angle (the
+ * backward). */
 int nsa_rope(const void* x, const int64_t* x_stride, int32_t batch, int32_t heads, int32_t seq, int32_t dim_head,
-             const float* freqs, int32_t offset, int32_t inverse, void* out, void* stream);
+             const float* freqs, int32_t offset, int32_t inverse, void* out, const int64_t* out_stride, void* stream);
+
+/* Single-token decode attention over cached keys / values.  Replaces the three attention
+ * computations of SparseAttention.forward_inference (NSA.py:396-420 compressed, :446-515 selected
+ * blocks + own block, :519-530 sliding window).
+ *   mode 0: the group's query heads attend keys [start, start + count) of the caches, preceded by
+ *           num_mem memory rows (mem_k / mem_v: bf16 [kv_heads, num_mem, d], contiguous; NSA.py:401-405).
+ *           logits (optional): fp32 [batch, heads, count] = scale * q.k of the cache keys, the
+ *           importance scores of NSA.py:444.
+ *   mode 1: keys of blocks idx[slot] (where fmask[slot] != 0 and the block starts before kv_len) plus
+ *           the block holding position kv_len - 1 up to that position.  idx / fmask:
+ *           [batch, kv_heads, num_sel] or, with per_head_sel, [batch, heads, num_sel].
+ * q: bf16 [batch, heads, d] with element strides {batch, head}; k, v: bf16 caches [batch, kv_heads,
+ * capacity, d] with element strides {batch, head, token}; out: bf16 [batch, heads, d] contiguous.
+ * ws: nsa_decode_workspace_bytes() bytes of device memory (split-K partials).  The caller
+ * guarantees start + count <= capacity and kv_len <= capacity. */
+typedef struct nsa_decode_desc {
+  int32_t batch, kv_heads, group, dim_head;
+  int32_t mode;
+  int32_t start, count, num_mem;          /* mode 0 */
+  int32_t block, num_sel, kv_len;         /* mode 1 */
+  int32_t per_head_sel, idx_is_int64;     /* mode 1 */
+  float scale;
+  int64_t q_stride[2], k_stride[3], v_stride[3];
+} nsa_decode_desc;
+int nsa_decode_workspace_bytes(const nsa_decode_desc* desc, size_t* bytes);
+int nsa_decode_attend(const nsa_decode_desc* desc, const void* q, const void* k, const void* v, const void* mem_k,
+                      const void* mem_v, const void* idx, const uint8_t* fmask, void* ws, size_t ws_bytes, void* out,
+                      float* logits, void* stream);
 
 /* Same as nsa_select_fwd / nsa_select_bwd, additionally recording the caller's hipEvent_t
  * handles (created with timing enabled) between the kernels of the call, so that a benchmark

@@ -31,6 +31,16 @@ class DenseDesc(C.Structure):
     ]
 
 
+class DecodeDesc(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("kv_heads", C.c_int32), ("group", C.c_int32), ("dim_head", C.c_int32),
+        ("mode", C.c_int32), ("start", C.c_int32), ("count", C.c_int32), ("num_mem", C.c_int32),
+        ("block", C.c_int32), ("num_sel", C.c_int32), ("kv_len", C.c_int32),
+        ("per_head_sel", C.c_int32), ("idx_is_int64", C.c_int32), ("scale", C.c_float),
+        ("q_stride", C.c_int64 * 2), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
+    ]
+
+
 _ERR = {-1: "invalid argument", -2: "shape not supported by the compiled kernels", -3: "workspace too small"}
 
 
@@ -60,8 +70,11 @@ def lib():
         i3 = C.POINTER(C.c_int64)
         L.nsa_gate_fwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp]
         L.nsa_gate_bwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp, vp, vp, vp, vp]
-        L.nsa_rope.argtypes = [vp, i3, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, C.c_int32, C.c_int32, vp, vp]
+        L.nsa_rope.argtypes = [vp, i3, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, C.c_int32, C.c_int32, vp, i3, vp]
         L.nsa_rope.restype = C.c_int
+        L.nsa_decode_workspace_bytes.argtypes = [C.POINTER(DecodeDesc), C.POINTER(sz)]
+        L.nsa_decode_attend.argtypes = [C.POINTER(DecodeDesc)] + [vp] * 8 + [sz, vp, vp, vp]
+        L.nsa_decode_workspace_bytes.restype = L.nsa_decode_attend.restype = C.c_int
         for name in ("nsa_dense_workspace_bytes", "nsa_dense_fwd", "nsa_dense_bwd", "nsa_topk", "nsa_gate_fwd", "nsa_gate_bwd"):
             getattr(L, name).restype = C.c_int
         for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):

@@ -449,7 +449,7 @@ def rope_op(x: Tensor, freqs: Tensor, offset: int, inverse: bool) -> Tensor:
     b, h, n, d = x.shape
     freqs = freqs.detach().to(torch.float32).contiguous()
     out = torch.empty((b, h, n, d), dtype=_BF16, device=x.device)
-    _lib.check(_lib.lib().nsa_rope(_ptr(x), _s3(x), b, h, n, d, _ptr(freqs), int(offset), int(inverse), _ptr(out), _stream()), "nsa_rope")
+    _lib.check(_lib.lib().nsa_rope(_ptr(x), _s3(x), b, h, n, d, _ptr(freqs), int(offset), int(inverse), _ptr(out), None, _stream()), "nsa_rope")
     return out
 
 
@@ -476,3 +476,93 @@ rope_op.register_autograd(_rope_backward, setup_context=_rope_setup)
 def rotary(x: Tensor, freqs: Tensor, offset: int = 0) -> Tensor:
     """Rotary embedding of 'b h n d' queries or keys at positions offset .. offset+n-1 (NSA.py:643)."""
     return rope_op(x, freqs, int(offset), False)
+
+
+def rotary_into(x: Tensor, freqs: Tensor, offset: int, out: Tensor) -> None:
+    """Rotate 'b h n d' `x` at positions offset.. and write the result into `out`, a strided
+    'b h n d' view (a slot of a key cache, NSA.py:384-390).  Inference only (no autograd)."""
+    x = _prep(x)
+    b, h, n, d = x.shape
+    if out.dtype != _BF16 or out.shape != x.shape or not _rows_ok(out):
+        raise RuntimeError("rotary_into: `out` must be a bf16 'b h n d' view with 16-byte aligned rows")
+    freqs = freqs.detach().to(torch.float32).contiguous()
+    _lib.check(_lib.lib().nsa_rope(_ptr(x), _s3(x), b, h, n, d, _ptr(freqs), int(offset), 0, _ptr(out), _s3(out), _stream()), "nsa_rope")
+
+
+# ---------------------------------------------------------------------------------- decode
+
+def _decode_call(dsc, q, k, v, mem_k, mem_v, idx, fmask, logits):
+    L = _lib.lib()
+    nbytes = C.c_size_t()
+    _lib.check(L.nsa_decode_workspace_bytes(C.byref(dsc), C.byref(nbytes)), "nsa_decode_workspace_bytes")
+    ws = torch.empty(max(nbytes.value, 16), dtype=torch.uint8, device=q.device)
+    out = torch.empty((q.shape[0], q.shape[1], 1, q.shape[3]), dtype=_BF16, device=q.device)
+    _lib.check(L.nsa_decode_attend(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(mem_k), _ptr(mem_v), _ptr(idx), _ptr(fmask),
+                                   _ptr(ws), nbytes, _ptr(out), _ptr(logits), _stream()), "nsa_decode_attend")
+    return out
+
+
+def _decode_desc(q: Tensor, k: Tensor | None, v: Tensor | None, hk: int):
+    b, hq, one, d = q.shape
+    if one != 1:
+        raise RuntimeError("decode attention takes one query token")
+    if hq % hk:
+        raise RuntimeError("query heads must be a multiple of kv heads")
+    dsc = _lib.DecodeDesc()
+    dsc.batch, dsc.kv_heads, dsc.group, dsc.dim_head = b, hk, hq // hk, d
+    dsc.scale = d ** -0.5
+    dsc.q_stride[:] = (q.stride(0), q.stride(1))
+    for name, t in (("k_stride", k), ("v_stride", v)):
+        if t is not None:
+            if t.dtype != _BF16 or not t.is_cuda or not _rows_ok(t):
+                raise RuntimeError("key / value caches must be bf16 device tensors with unit feature stride and 16-byte aligned rows")
+            getattr(dsc, name)[:] = t.stride()[:3]
+    return dsc
+
+
+@torch.no_grad()
+def decode_range_attend(q: Tensor, k: Tensor, v: Tensor, start: int, count: int, mem_k: Tensor | None = None,
+                        mem_v: Tensor | None = None, return_logits: bool = False):
+    """One query token 'b hq 1 d' attends keys [start, start+count) of the caches 'b hk cap d',
+    preceded by the memory rows mem_k / mem_v 'hk m d' (compressed branch NSA.py:396-420; sliding
+    branch NSA.py:519-530).  With return_logits also scale * q.k over the cache keys, fp32
+    'b hq count' (NSA.py:444)."""
+    q = _prep(q)
+    hk = k.shape[1]
+    if start < 0 or count < 0 or start + count > k.shape[2] or k.shape != v.shape:
+        raise RuntimeError("decode_range_attend: key range outside the caches")
+    dsc = _decode_desc(q, k if count else None, v if count else None, hk)
+    dsc.mode, dsc.start, dsc.count = 0, int(start), int(count)
+    m = 0
+    if mem_k is not None:
+        mem_k, mem_v = mem_k.to(_BF16).contiguous(), mem_v.to(_BF16).contiguous()
+        m = mem_k.shape[-2]
+        if mem_k.shape != (hk, m, q.shape[-1]) or mem_v.shape != mem_k.shape:
+            raise RuntimeError("decode_range_attend: memory rows must be 'hk m d'")
+    dsc.num_mem = m
+    logits = torch.empty((q.shape[0], q.shape[1], count), dtype=torch.float32, device=q.device) if return_logits else None
+    out = _decode_call(dsc, q, k if count else None, v if count else None, mem_k, mem_v, None, None, logits)
+    return (out, logits) if return_logits else out
+
+
+@torch.no_grad()
+def decode_select_attend(q: Tensor, k: Tensor, v: Tensor, kv_len: int, block: int, idx: Tensor, fmask: Tensor):
+    """One query token at position kv_len-1 attends the blocks idx[..., slot] (where fmask) and
+    its own block up to itself (NSA.py:446-515).  idx / fmask: 'b hk 1 S' or, for per-head
+    selection, 'b hq 1 S'."""
+    q = _prep(q)
+    b, hq = q.shape[:2]
+    hk = k.shape[1]
+    if kv_len < 1 or kv_len > k.shape[2] or k.shape != v.shape:
+        raise RuntimeError("decode_select_attend: kv_len outside the caches")
+    if idx.shape[:3] not in ((b, hk, 1), (b, hq, 1)) or fmask.shape != idx.shape:
+        raise RuntimeError("decode_select_attend: idx / fmask must be 'b hk 1 S' or 'b hq 1 S'")
+    if idx.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError("decode_select_attend: idx must be int32 or int64")
+    dsc = _decode_desc(q, k, v, hk)
+    dsc.mode, dsc.block, dsc.num_sel, dsc.kv_len = 1, int(block), idx.shape[-1], int(kv_len)
+    dsc.per_head_sel = int(idx.shape[1] == hq and hq != hk)
+    dsc.idx_is_int64 = int(idx.dtype == torch.int64)
+    idx = idx.contiguous()
+    fm = fmask.contiguous().view(torch.uint8) if fmask.dtype == torch.bool else fmask.to(torch.uint8).contiguous()
+    return _decode_call(dsc, q, k, v, None, None, idx if idx.numel() else None, fm if fm.numel() else None, None)

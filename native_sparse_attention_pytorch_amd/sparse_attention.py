@@ -10,6 +10,11 @@ training / prefill forward runs the four NSA subsystems as gfx950 HIP kernels:
 
 The dense projections (qkv, compression MLP, gate logits, output) stay `nn.Linear` GEMMs.  There
 is no non-HIP path: CPU tensors, a missing library or an unsupported shape raise.
+
+Single-token decoding over the caches (NSA.py:338-547) runs the same branches through
+ops.decode_range_attend / ops.decode_select_attend.  The key / value and compressed caches the
+module hands back are prefixes of buffers with spare capacity: the next step writes its row in
+place instead of re-concatenating the whole cache (amortised O(1) per token rather than O(n)).
 """
 from __future__ import annotations
 
@@ -41,6 +46,24 @@ class RotaryEmbedding(nn.Module):
 
     def rotate_queries_with_cached_keys(self, q, k):
         return self.rotate(q, offset=k.shape[-2] - q.shape[-2]), self.rotate(k)
+
+
+def _append_rows(t: torch.Tensor, extra: int = 1):
+    """Grow the 'b h n d' cache `t` by `extra` rows.  Returns (view of n+extra rows, view of the
+    new rows).  When `t` is the filled prefix of a buffer made here, the rows are taken from the
+    buffer's spare capacity; otherwise (a cache from the parallel forward, a branch point that
+    re-uses an older cache, no capacity left) the contents move to a new bf16 buffer of twice
+    the size first, so a caller that keeps an old cache tuple never sees it change."""
+    b, h, n, d = t.shape
+    base = t._base
+    ok = (base is not None and getattr(base, "_nsa_filled", -1) == n and base.dtype == torch.bfloat16
+          and base.dim() == 4 and base.shape[2] >= n + extra and base.shape[:2] == t.shape[:2] and base.shape[3] == d
+          and t.data_ptr() == base.data_ptr() and t.stride() == base.stride())
+    if not ok:
+        base = torch.empty((b, h, max(2 * (n + extra), 128), d), dtype=torch.bfloat16, device=t.device)
+        base[:, :, :n].copy_(t)
+    base._nsa_filled = n + extra
+    return base[:, :, :n + extra], base[:, :, n:n + extra]
 
 
 class _FlattenWindow(nn.Module):
@@ -145,8 +168,79 @@ class SparseAttention(nn.Module):
             return t.reshape(b, h, 0, cbs, d)
         return F.pad(t, (0, 0, cbs - st, 0)).unfold(2, cbs, st).permute(0, 1, 2, 4, 3)
 
+    @torch.no_grad()
     def forward_inference(self, inp, cache, return_cache=True):
-        raise NotImplementedError("single-token decode with caches (NSA.py:338-547) is outside the accelerated hot path")
+        """One decode step (NSA.py:338-547): `inp` 'b 1 dim' is the token at position t = cached
+        length; returns the output and the advanced caches."""
+        assert self.causal, 'inference only relevant for autoregressive'
+        if not inp.is_cuda:
+            raise RuntimeError("SparseAttention runs on the GPU only (HIP kernels, no CPU fallback)")
+        (cache_k, cache_v), ((cache_ck, cache_cv), (run_k, run_v)) = cache
+        b, t = inp.shape[0], cache_k.shape[-2]
+        st, cbs, B = self.compress_block_sliding_stride, self.compress_block_size, self.selection_block_size
+        G, bf16 = self.num_grouped_queries, torch.bfloat16
+        freqs = self.rotary_emb.freqs
+
+        x = self.norm(inp)
+        q, k, v = self.to_qkv(x).split(self.qkv_split, dim=-1)
+        q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
+        q16, k16 = q.to(bf16), k.to(bf16)
+
+        # raw tokens of the open compression window (not rotated, NSA.py:377-380)
+        run_k, run_v = torch.cat((run_k, k.to(run_k.dtype)), dim=-2), torch.cat((run_v, v.to(run_v.dtype)), dim=-2)
+
+        # the rotated key and the value go into row t of the caches (NSA.py:384-393)
+        keys, k_row = _append_rows(cache_k)
+        vals, v_row = _append_rows(cache_v)
+        ops.rotary_into(k16, freqs, t, k_row)
+        v_row.copy_(v)
+        rq16 = ops.rotary(q16, freqs, t)
+
+        # 1. compressed branch: every cached compressed key, no mask (NSA.py:396-420)
+        nc = cache_ck.shape[-2]
+        logits = None
+        if nc > 0:
+            ck16 = cache_ck if cache_ck.dtype == bf16 else cache_ck.to(bf16)
+            cv16 = cache_cv if cache_cv.dtype == bf16 else cache_cv.to(bf16)
+            c_out, logits = ops.decode_range_attend(q16, ck16, cv16, 0, nc, self.compress_mem_kv[0], self.compress_mem_kv[1],
+                                                    return_logits=True)
+        else:
+            c_out = torch.zeros_like(q16)
+
+        # a compression window is complete: compress it, keep the overlap (NSA.py:422-441)
+        ck, cv = cache_ck, cache_cv
+        if run_k.shape[-2] % cbs == 0:
+            next_ck = self.k_compress((run_k + self.k_intrablock_positions)[:, :, None])
+            next_cv = self.v_compress((run_v + self.v_intrablock_positions)[:, :, None])
+            run_k, run_v = run_k[..., st:, :], run_v[..., st:, :]
+            ck, ck_row = _append_rows(cache_ck)
+            cv, cv_row = _append_rows(cache_cv)
+            ck_row.copy_(next_ck)
+            cv_row.copy_(next_cv)
+
+        # 2. selection branch (NSA.py:446-515): top blocks by importance + own block up to t
+        npf = B // st
+        nb = nc // npf
+        num_sel = min(self.num_selected_blocks, nb)
+        if num_sel > 0:
+            imp = logits[..., :nb * npf].reshape(b, self.kv_heads, G, 1, nb, npf).mean(dim=-1)
+            imp = imp.mean(dim=2) if self.query_heads_share_selected_kv else imp.reshape(b, self.heads, 1, nb)
+            _, idx, fmask = ops.importance_topk(imp.contiguous(), num_sel)
+        else:
+            idx = torch.zeros((b, self.kv_heads, 1, 0), dtype=torch.int32, device=inp.device)
+            fmask = idx.bool()
+        f_out = ops.decode_select_attend(rq16, keys, vals, t + 1, B, idx, fmask)
+
+        # 3. sliding branch: the last window + 1 keys (NSA.py:519-530)
+        w = min(t + 1, self.sliding_window_size + 1)
+        s_out = ops.decode_range_attend(rq16, keys, vals, t + 1 - w, w)
+
+        logits_g = self.to_strategy_combine[0](x)
+        merged = ops.gate_combine(logits_g, c_out, f_out, s_out)
+        out = self.combine_heads(merged.to(x.dtype))
+        if not return_cache:
+            return out
+        return out, ((keys, vals), ((ck, cv), (run_k, run_v)))
 
     def forward(self, inp, cache=None, disable_triton_kernel=False, sliding_window_flex_mask=None,
                 fine_selection_flex_mask=None, return_cache=False):

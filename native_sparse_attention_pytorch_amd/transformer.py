@@ -1,8 +1,10 @@
 """Decoder-only transformer around `SparseAttention`: the training-forward harness of the
 reference (native_sparse_attention_pytorch/transformer.py:130-138 FeedForward, :142-211
-construction, :254-330 forward) with the same constructor arguments and parameter names.
-Sampling / cached decoding (transformer.py:213-252) is outside the accelerated hot path."""
+construction, :254-330 forward, :213-252 sampling with or without the per-layer caches) with the
+same constructor arguments and parameter names."""
 from __future__ import annotations
+
+import math
 
 import torch
 import torch.nn.functional as F
@@ -40,15 +42,17 @@ class Transformer(nn.Module):
         self.to_logits = nn.Linear(dim, num_tokens, bias=False)
 
     def forward(self, ids, return_loss=False, disable_flex=False, disable_triton_kernel=False, cache=None, return_cache=False):
-        if cache is not None:
-            raise NotImplementedError("cached decoding is outside the accelerated hot path")
         if return_loss:
             ids, labels = ids[:, :-1], ids[:, 1:]
-        tokens = self.token_emb(ids)
+        # with caches only the newest token is embedded and every layer takes one decode step
+        tokens = self.token_emb(ids if cache is None else ids[:, -1:])
+        layer_caches = iter(cache or [])
         caches = []
         for attn, ff in self.layers:
-            # the reference always asks the attention layer for its cache (transformer.py:308-313)
-            attn_out, layer_cache = attn(tokens, return_cache=True) if return_cache else (attn(tokens), None)
+            if return_cache or cache is not None:
+                attn_out, layer_cache = attn(tokens, cache=next(layer_caches, None), return_cache=True)
+            else:
+                attn_out, layer_cache = attn(tokens), None
             caches.append(layer_cache)
             tokens = attn_out + tokens
             tokens = ff(tokens) + tokens
@@ -56,3 +60,26 @@ class Transformer(nn.Module):
         if not return_loss:
             return (logits, caches) if return_cache else logits
         return F.cross_entropy(logits.transpose(1, 2).float(), labels)
+
+
+    @torch.no_grad()
+    def sample(self, prompt, seq_len, temperature=1., filter_thres=0.9, use_cache_kv=False):
+        """Extend `prompt` to seq_len tokens and return the new ones (transformer.py:213-252).
+        temperature <= 0 is greedy; otherwise gumbel sampling over the top (1 - filter_thres)
+        share of the vocabulary.  With use_cache_kv every step after the first is a decode step."""
+        out, cache = prompt.clone(), None
+        for _ in range(max(0, seq_len - prompt.shape[-1])):
+            logits, next_cache = self.forward(out, cache=cache, return_cache=True)
+            if use_cache_kv:
+                cache = next_cache
+            logits = logits[:, -1].float()
+            if temperature <= 0.:
+                tok = logits.argmax(dim=-1, keepdim=True)
+            else:
+                kk = math.ceil((1 - filter_thres) * logits.shape[-1])
+                val, ind = logits.topk(kk, dim=-1)
+                logits = torch.full_like(logits, float('-inf')).scatter_(-1, ind, val)
+                noise = -torch.log(-torch.log(torch.rand_like(logits).clamp_min(1e-20)).clamp_min(1e-20))
+                tok = (logits / max(temperature, 1e-10) + noise).argmax(dim=-1, keepdim=True)
+            out = torch.cat((out, tok), dim=-1)
+        return out[..., prompt.shape[-1]:]
