@@ -175,6 +175,26 @@ int nsa_decode_attend(const nsa_decode_desc* desc, const void* q, const void* k,
                       const void* mem_v, const void* idx, const uint8_t* fmask, void* ws, size_t ws_bytes, void* out,
                       float* logits, void* stream);
 
+/* Decode step, after three nsa_decode_attend calls with out == NULL (their partials left in the
+ * three workspaces): merges each branch, applies the sigmoid strategy gate and writes the merged
+ * heads.  Replaces to_strategy_combine's sigmoid + rearrange, the stack / einsum and merge_heads of
+ * NSA.py:534-545.  gate_logits: bf16 [batch, 3 * heads], column 3 * head + {0 compressed, 1 selected,
+ * 2 sliding}; out: bf16 [batch, heads * d].  A branch whose workspace is NULL contributes zero (the
+ * compressed branch before the first compressed key exists, NSA.py:401). */
+int nsa_decode_combine(const nsa_decode_desc* compressed, const void* ws_compressed, const nsa_decode_desc* selected,
+                       const void* ws_selected, const nsa_decode_desc* sliding, const void* ws_sliding,
+                       const void* gate_logits, void* out, void* stream);
+
+/* Decode step: rotates the new token's queries (-> rq, bf16 [batch, heads, d] contiguous) and keys to
+ * position pos, writes the rotated keys into row pos of the key cache and the values into row pos
+ * of the value cache.  Replaces rotate_queries_or_keys x2 and the two cache concatenations of
+ * NSA.py:384-393.  q, k, v: bf16 [batch, heads|kv_heads, d] with element strides {batch, head};
+ * k_row / v_row: address of row pos of head 0 of batch 0 in the caches, strides {batch, head}. */
+int nsa_decode_prep(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v,
+                    const int64_t* v_stride, int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head,
+                    const float* freqs, int32_t pos, void* rq, void* k_row, const int64_t* k_row_stride, void* v_row,
+                    const int64_t* v_row_stride, void* stream);
+
 /* Same as nsa_select_fwd / nsa_select_bwd, additionally recording the caller's hipEvent_t
  * handles (created with timing enabled) between the kernels of the call, so that a benchmark
  * can time each kernel on the launch stream.  Events: fwd {start, after block walk, after

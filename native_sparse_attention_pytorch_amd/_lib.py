@@ -75,6 +75,11 @@ def lib():
         L.nsa_decode_workspace_bytes.argtypes = [C.POINTER(DecodeDesc), C.POINTER(sz)]
         L.nsa_decode_attend.argtypes = [C.POINTER(DecodeDesc)] + [vp] * 8 + [sz, vp, vp, vp]
         L.nsa_decode_workspace_bytes.restype = L.nsa_decode_attend.restype = C.c_int
+        dd = C.POINTER(DecodeDesc)
+        L.nsa_decode_combine.argtypes = [dd, vp, dd, vp, dd, vp, vp, vp, vp]
+        i2 = C.POINTER(C.c_int64)
+        L.nsa_decode_prep.argtypes = [vp, i2, vp, i2, vp, i2, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, C.c_int32, vp, vp, i2, vp, i2, vp]
+        L.nsa_decode_combine.restype = L.nsa_decode_prep.restype = C.c_int
         for name in ("nsa_dense_workspace_bytes", "nsa_dense_fwd", "nsa_dense_bwd", "nsa_topk", "nsa_gate_fwd", "nsa_gate_bwd"):
             getattr(L, name).restype = C.c_int
         for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):

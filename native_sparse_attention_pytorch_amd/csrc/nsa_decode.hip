@@ -7,7 +7,10 @@
 // (batch, kv head) are cut into 32-key tiles that are dealt round-robin to the waves of
 // `nsplit` work-groups (split-K), so that a single long sequence still fills the chip; every
 // wave keeps a running (max, sum, O) and writes one fp32 partial, and a second kernel merges the
-// partials of a head.  Scores are computed transposed, S^T = K Q^T on the 32x32x16 MFMA with the
+// partials of a head.  Rows are fetched one tile ahead with whole-row coalesced loads and become
+// MFMA operands through a per-wave LDS tile (row operand for K, transposing LDS load for V^T):
+// reading each row in 32-byte pieces straight into the operand layout touches every cache line
+// from several instructions and re-fetches it from L2 once the L1 thrashes.  Scores are computed transposed, S^T = K Q^T on the 32x32x16 MFMA with the
 // query heads as (zero-padded) columns: a lane then owns one head, the softmax statistics are
 // per-lane scalars and the rescaling of O^T = V^T P needs no cross-lane traffic.
 #include "nsa_common.hpp"
@@ -27,18 +30,72 @@ struct DecodePlan {
   long sq[2], sk[3], sv[3];
 };
 
+constexpr int kDecodeWaves = 2;      // waves per work-group; each stages its own K / V tile in LDS
+
+struct DecodeTile {
+  const __bf16 *kb, *vb;             // row 0 of the tile
+  long ks, vs;                       // row strides
+  int nvalid, lcol;                  // rows in use; column of row 0 in the logits row (-1: not written)
+};
+
+// tile t of unit (b, hk, ug) -> its rows; nvalid <= 0 for tiles with nothing to attend
+__device__ __forceinline__ DecodeTile decode_tile(const DecodePlan& P, int D, int t, int b, int hk, int ug, const __bf16* k, const __bf16* v,
+                                                  const __bf16* mem_k, const __bf16* mem_v, const void* idx, const unsigned char* fmask) {
+  DecodeTile T;
+  T.lcol = -1;
+  if (P.mode == 0) {
+    const int mem_tiles = (P.mem + 31) >> 5;
+    if (t < mem_tiles) {
+      T.kb = mem_k + ((long)hk * P.mem + 32 * t) * D;
+      T.vb = mem_v + ((long)hk * P.mem + 32 * t) * D;
+      T.ks = T.vs = D;
+      T.nvalid = min(32, P.mem - 32 * t);
+    } else {
+      const int tt = t - mem_tiles;
+      T.kb = k + b * P.sk[0] + hk * P.sk[1] + (long)(P.start + 32 * tt) * P.sk[2];
+      T.vb = v + b * P.sv[0] + hk * P.sv[1] + (long)(P.start + 32 * tt) * P.sv[2];
+      T.ks = P.sk[2]; T.vs = P.sv[2];
+      T.nvalid = min(32, P.count - 32 * tt);
+      T.lcol = 32 * tt;
+    }
+  } else {
+    const int slot = t / P.tps, sub = t % P.tps;
+    long blk;
+    bool live = true;
+    if (slot < P.S) {
+      const long e = (long)ug * P.S + slot;
+      blk = P.idx64 ? reinterpret_cast<const long*>(idx)[e] : (long)reinterpret_cast<const int*>(idx)[e];
+      live = fmask[e] != 0 && blk >= 0 && blk * P.B < P.kv_len;
+      if (!live) blk = 0;
+    } else {
+      blk = (P.kv_len - 1) / P.B;                     // the query's own block, up to itself
+    }
+    const long key0 = blk * P.B + 32 * sub;
+    T.kb = k + b * P.sk[0] + hk * P.sk[1] + key0 * P.sk[2];
+    T.vb = v + b * P.sv[0] + hk * P.sv[1] + key0 * P.sv[2];
+    T.ks = P.sk[2]; T.vs = P.sv[2];
+    T.nvalid = live ? (int)min((long)32, min((long)P.B - 32 * sub, (long)P.kv_len - key0)) : 0;
+  }
+  return T;
+}
+
 template <int D>
-__global__ __launch_bounds__(256) void decode_attend_kernel(const DecodePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
-                                                            const __bf16* __restrict__ v, const __bf16* __restrict__ mem_k,
-                                                            const __bf16* __restrict__ mem_v, const void* __restrict__ idx,
-                                                            const unsigned char* __restrict__ fmask, float* __restrict__ part,
-                                                            float* __restrict__ logits) {
-  constexpr int KS = D / 16, DT = D / 32;
+__global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_eu(2))) void decode_attend_kernel(const DecodePlan P, const __bf16* __restrict__ q,
+                                                                          const __bf16* __restrict__ k, const __bf16* __restrict__ v,
+                                                                          const __bf16* __restrict__ mem_k, const __bf16* __restrict__ mem_v,
+                                                                          const void* __restrict__ idx, const unsigned char* __restrict__ fmask,
+                                                                          float* __restrict__ part, float* __restrict__ logits) {
+  constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
+  constexpr int LPR = D / 8, RPI = 64 / LPR, NI = 32 / RPI;      // lanes per row, rows per load instruction, instructions per tile
+  __shared__ __align__(16) __bf16 kv_s[kDecodeWaves][2][32 * RS];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_ = lane & 31, h = lane >> 5;
+  const int lr = lane / LPR, lc = lane % LPR;
+  __bf16* k_s = kv_s[wave][0];
+  __bf16* v_s = kv_s[wave][1];
   const int ug = blockIdx.y, b = ug / P.units, u = ug % P.units;
   const int hk = (P.units == P.hk) ? u : u / P.g;
   const int head0 = (P.units == P.hk) ? u * P.g : u;
-  const int wid = blockIdx.x * 4 + wave, nw = P.nsplit * 4;
+  const int wid = blockIdx.x * kDecodeWaves + wave, nw = P.nsplit * kDecodeWaves;
 
   bf16x8 Qf[KS];
   {
@@ -47,73 +104,57 @@ __global__ __launch_bounds__(256) void decode_attend_kernel(const DecodePlan P, 
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) Qf[ks] = okq ? load8(qp + 16 * ks) : zero_frag();
   }
-  bf16x8 ilo, ihi;
-  make_ident(lane, ilo, ihi);
   const float sc = P.scale * kLog2e;
-  const int mem_tiles = (P.mem + 31) >> 5;
 
   float m = -INFINITY, l = 0.f;
   floatx16 Oa[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) Oa[dt] = zero_acc();
 
-  for (int t = wid; t < P.tiles; t += nw) {
-    // tile -> rows of (kb, vb) with row stride (ks_, vs_), first row key0, nvalid rows
-    const __bf16 *kb, *vb;
-    long ks_, vs_, key0;
-    int nvalid, lcol = -1;           // lcol: column of the tile's first key in the logits row
-    if (P.mode == 0) {
-      if (t < mem_tiles) {
-        kb = mem_k + (long)hk * P.mem * D; vb = mem_v + (long)hk * P.mem * D;
-        ks_ = vs_ = D; key0 = 32 * t; nvalid = min(32, P.mem - 32 * t);
-      } else {
-        const int tt = t - mem_tiles;
-        kb = k + b * P.sk[0] + hk * P.sk[1]; vb = v + b * P.sv[0] + hk * P.sv[1];
-        ks_ = P.sk[2]; vs_ = P.sv[2]; key0 = P.start + 32 * tt; nvalid = min(32, P.count - 32 * tt);
-        lcol = 32 * tt;
-      }
-    } else {
-      const int slot = t / P.tps, sub = t % P.tps;
-      kb = k + b * P.sk[0] + hk * P.sk[1]; vb = v + b * P.sv[0] + hk * P.sv[1];
-      ks_ = P.sk[2]; vs_ = P.sv[2];
-      long blk;
-      bool live = true;
-      if (slot < P.S) {
-        const long e = (long)ug * P.S + slot;
-        blk = P.idx64 ? reinterpret_cast<const long*>(idx)[e] : (long)reinterpret_cast<const int*>(idx)[e];
-        live = fmask[e] != 0 && blk >= 0 && blk * P.B < P.kv_len;
-      } else {
-        blk = (P.kv_len - 1) / P.B;                   // the query's own block, up to itself
-      }
-      key0 = blk * P.B + 32 * sub;
-      nvalid = live ? (int)min((long)32, min((long)P.B - 32 * sub, (long)P.kv_len - key0)) : 0;
+  // rows are fetched with whole-row coalesced loads (LPR lanes per row) one tile ahead of the
+  // arithmetic, and turned into MFMA operands through the wave's private LDS tiles
+  bf16x8 kr[NI], vr[NI];
+  auto issue = [&](const DecodeTile& T) {
+#pragma unroll
+    for (int r = 0; r < NI; ++r) {
+      const int row = RPI * r + lr;
+      const long rc = row < T.nvalid ? row : 0;
+      kr[r] = load8(T.kb + rc * T.ks + 8 * lc);
+      vr[r] = load8(T.vb + rc * T.vs + 8 * lc);
     }
-    if (nvalid <= 0) continue;                        // wave-uniform
+  };
+  auto next_tile = [&](int t, DecodeTile& T) {
+    for (; t < P.tiles; t += nw) {
+      T = decode_tile(P, D, t, b, hk, ug, k, v, mem_k, mem_v, idx, fmask);
+      if (T.nvalid > 0) break;
+    }
+    return t;
+  };
 
-    const bool okr = n_ < nvalid;
-    const __bf16* kp = kb + (key0 + (okr ? n_ : 0)) * ks_ + 8 * h;
-    const __bf16* vp = vb + (key0 + (okr ? n_ : 0)) * vs_ + 8 * h;
+  DecodeTile T, Tn;
+  int t = next_tile(wid, T);
+  if (t < P.tiles) issue(T);
+  while (t < P.tiles) {
+#pragma unroll
+    for (int r = 0; r < NI; ++r) {
+      *reinterpret_cast<bf16x8*>(k_s + (RPI * r + lr) * RS + 8 * lc) = kr[r];
+      *reinterpret_cast<bf16x8*>(v_s + (RPI * r + lr) * RS + 8 * lc) = vr[r];
+    }
+    const int tn = next_tile(t + nw, Tn);
+    if (tn < P.tiles) issue(Tn);
+    __builtin_amdgcn_sched_barrier(0);
+
     floatx16 Sa = zero_acc();
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) Sa = mfma32(okr ? load8(kp + 16 * ks) : zero_frag(), Qf[ks], Sa);
-    bf16x8 VT[DT][2];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const bf16x8 va = okr ? load8(vp + 32 * dt) : zero_frag();
-      const bf16x8 vb2 = okr ? load8(vp + 32 * dt + 16) : zero_frag();
-      floatx16 tr = mfma32(va, ilo, zero_acc());
-      tr = mfma32(vb2, ihi, tr);
-      VT[dt][0] = pack8(tr, 0);
-      VT[dt][1] = pack8(tr, 8);
-    }
+    for (int ks = 0; ks < KS; ++ks) Sa = mfma32(lds_row_operand(k_s, RS, ks, lane), Qf[ks], Sa);
 
     float mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int kl = 8 * (i >> 2) + 4 * h + (i & 3);
-      if (logits != nullptr && lcol >= 0 && n_ < P.gc && kl < nvalid)
-        logits[((long)b * P.hk * P.g + head0 + n_) * P.count + lcol + kl] = Sa[i] * P.scale;
-      const float s = kl < nvalid ? Sa[i] * sc : -INFINITY;
+      if (logits != nullptr && T.lcol >= 0 && n_ < P.gc && kl < T.nvalid)
+        logits[((long)b * P.hk * P.g + head0 + n_) * P.count + T.lcol + kl] = Sa[i] * P.scale;
+      const float s = kl < T.nvalid ? Sa[i] * sc : -INFINITY;
       Sa[i] = s;
       mx = fmaxf(mx, s);
     }
@@ -134,8 +175,11 @@ __global__ __launch_bounds__(256) void decode_attend_kernel(const DecodePlan P, 
 #pragma unroll
       for (int i = 0; i < 16; ++i) Oa[dt][i] *= alpha;
 #pragma unroll
-      for (int u2 = 0; u2 < 2; ++u2) Oa[dt] = mfma32(VT[dt][u2], pack8(Sa, 8 * u2), Oa[dt]);
+      for (int u2 = 0; u2 < 2; ++u2)
+        Oa[dt] = mfma32(lds_transposed_operand(v_s, RS, 16 * u2, 32 * dt, lane), pack8(Sa, 8 * u2), Oa[dt]);
     }
+    t = tn;
+    T = Tn;
   }
   l += xor32(l);
 
@@ -176,6 +220,45 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(const DecodePlan P, con
   out[(long)bh * D + threadIdx.x] = (__bf16)(L > 0.f ? acc / L : 0.f);
 }
 
+// Merge of the three branches' partials, sigmoid strategy gate and head merge in one pass
+// (NSA.py:534-545): out[b, head*D + f] = sum_s sigmoid(logit[b, 3*head + s]) * branch_s.
+// A branch without a workspace (no compressed key cached yet) contributes zero.
+struct CombineArgs {
+  DecodePlan P[3];
+  const float* part[3];
+};
+
+template <int D>
+__global__ __launch_bounds__(D) void decode_combine_kernel(const CombineArgs A, const __bf16* __restrict__ gate_logits, __bf16* __restrict__ out) {
+  const int hq = A.P[0].hk * A.P[0].g;
+  const int bh = blockIdx.x, b = bh / hq, head = bh % hq;
+  float res = 0.f;
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    if (A.part[s] == nullptr) continue;
+    const DecodePlan& P = A.P[s];
+    const int u = (P.units == P.hk) ? head / P.g : head, gi = (P.units == P.hk) ? head % P.g : 0;
+    const float* base = A.part[s] + (long)(b * P.units + u) * P.nparts * P.rec;
+    const int om = P.gc * D + gi, ol = om + P.gc;
+    float M = -INFINITY;
+    for (int p = 0; p < P.nparts; ++p) M = fmaxf(M, base[(long)p * P.rec + om]);
+    float acc = 0.f, L = 0.f;
+    if (M > -INFINITY) {
+      for (int p = 0; p < P.nparts; ++p) {
+        const float* rec = base + (long)p * P.rec;
+        const float w = fast_exp2(rec[om] - M);
+        L += w * rec[ol];
+        acc += w * rec[gi * D + threadIdx.x];
+      }
+    }
+    // branch outputs are rounded to bf16 as when each is merged on its own
+    const float o = (float)(__bf16)(L > 0.f ? acc / L : 0.f);
+    const float gl = (float)gate_logits[((long)b * hq + head) * 3 + s];
+    res += o / (1.f + __expf(-gl));
+  }
+  out[(long)bh * D + threadIdx.x] = (__bf16)res;
+}
+
 static int make_decode_plan(const nsa_decode_desc* dsc, DecodePlan& P) {
   if (!dsc) return NSA_E_ARG;
   P = DecodePlan{};
@@ -207,12 +290,13 @@ static int make_decode_plan(const nsa_decode_desc* dsc, DecodePlan& P) {
   }
   const long units = (long)P.b * P.units;
   if (units > 65535) return NSA_E_UNSUPPORTED;
-  int ns = (P.tiles + 3) / 4;
-  const long cap = units >= 1024 ? 1 : 1024 / units;
+  // split-K: about two tiles per wave, but no more work-groups than a few per CU
+  int ns = (P.tiles + 2 * kDecodeWaves - 1) / (2 * kDecodeWaves);
+  const long cap = units >= 2048 ? 1 : 2048 / units;
   if (ns > cap) ns = (int)cap;
   if (ns > 64) ns = 64;
   if (ns < 1) ns = 1;
-  P.nsplit = ns; P.nparts = ns * 4;
+  P.nsplit = ns; P.nparts = ns * kDecodeWaves;
   P.rec = P.gc * P.d + ((2 * P.gc + 3) & ~3);
   return 0;
 }
@@ -233,7 +317,7 @@ extern "C" int nsa_decode_attend(const nsa_decode_desc* dsc, const void* q, cons
   using namespace nsa;
   DecodePlan P;
   if (int e = make_decode_plan(dsc, P)) return e;
-  if (!q || !out || !ws) return NSA_E_ARG;
+  if (!q || !ws) return NSA_E_ARG;
   if (P.mode == 0 && ((P.count > 0 && (!k || !v)) || (P.mem > 0 && (!mem_k || !mem_v)))) return NSA_E_ARG;
   if (P.mode == 1 && (!k || !v || (P.S > 0 && (!idx || !fmask)))) return NSA_E_ARG;
   if (ws_bytes < (size_t)P.b * P.units * P.nparts * P.rec * sizeof(float)) return NSA_E_WORKSPACE;
@@ -241,14 +325,44 @@ extern "C" int nsa_decode_attend(const nsa_decode_desc* dsc, const void* q, cons
   const dim3 grid(P.nsplit, P.b * P.units);
   const int heads = P.b * P.hk * P.g;
   if (P.d == 64) {
-    hipLaunchKernelGGL((decode_attend_kernel<64>), grid, dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+    hipLaunchKernelGGL((decode_attend_kernel<64>), grid, dim3(64 * kDecodeWaves), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                        (const __bf16*)mem_k, (const __bf16*)mem_v, idx, fmask, (float*)ws, logits);
-    hipLaunchKernelGGL((decode_merge_kernel<64>), dim3(heads), dim3(64), 0, st, P, (const float*)ws, (__bf16*)out);
+    if (out) hipLaunchKernelGGL((decode_merge_kernel<64>), dim3(heads), dim3(64), 0, st, P, (const float*)ws, (__bf16*)out);
   } else {
-    hipLaunchKernelGGL((decode_attend_kernel<128>), grid, dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
+    hipLaunchKernelGGL((decode_attend_kernel<128>), grid, dim3(64 * kDecodeWaves), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
                        (const __bf16*)mem_k, (const __bf16*)mem_v, idx, fmask, (float*)ws, logits);
-    hipLaunchKernelGGL((decode_merge_kernel<128>), dim3(heads), dim3(128), 0, st, P, (const float*)ws, (__bf16*)out);
+    if (out) hipLaunchKernelGGL((decode_merge_kernel<128>), dim3(heads), dim3(128), 0, st, P, (const float*)ws, (__bf16*)out);
   }
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
+
+extern "C" int nsa_decode_combine(const nsa_decode_desc* compressed, const void* ws_compressed, const nsa_decode_desc* selected,
+                                  const void* ws_selected, const nsa_decode_desc* sliding, const void* ws_sliding,
+                                  const void* gate_logits, void* out, void* stream) {
+  using namespace nsa;
+  const nsa_decode_desc* dsc[3] = {compressed, selected, sliding};
+  const void* ws[3] = {ws_compressed, ws_selected, ws_sliding};
+  if (!gate_logits || !out) return NSA_E_ARG;
+  CombineArgs A;
+  int ref = -1;
+  for (int s = 0; s < 3; ++s) {
+    A.part[s] = nullptr;
+    A.P[s] = DecodePlan{};
+    if (!ws[s]) continue;
+    if (int e = make_decode_plan(dsc[s], A.P[s])) return e;
+    A.part[s] = (const float*)ws[s];
+    if (ref < 0) ref = s;
+    else if (A.P[s].b != A.P[ref].b || A.P[s].hk != A.P[ref].hk || A.P[s].g != A.P[ref].g || A.P[s].d != A.P[ref].d) return NSA_E_ARG;
+  }
+  if (ref < 0) return NSA_E_ARG;
+  if (ref != 0) A.P[0] = A.P[ref];         // the kernel reads the head counts from slot 0
+  const int heads = A.P[ref].b * A.P[ref].hk * A.P[ref].g;
+  hipStream_t st = (hipStream_t)stream;
+  if (A.P[ref].d == 64)
+    hipLaunchKernelGGL((decode_combine_kernel<64>), dim3(heads), dim3(64), 0, st, A, (const __bf16*)gate_logits, (__bf16*)out);
+  else
+    hipLaunchKernelGGL((decode_combine_kernel<128>), dim3(heads), dim3(128), 0, st, A, (const __bf16*)gate_logits, (__bf16*)out);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
 }

@@ -33,7 +33,73 @@ __global__ __launch_bounds__(256) void rope_kernel(const __bf16* __restrict__ x,
   *reinterpret_cast<bf16x8*>(out + bb * o0 + hh * o1 + i * o2 + 8 * c) = r;
 }
 
+// Decode step: the new token's query heads rotated to position pos (-> rq), its key heads
+// rotated and written into row pos of the key cache, its value heads copied into row pos of
+// the value cache (NSA.py:384-393) - one launch instead of two rotations and a copy.
+template <int D>
+__global__ __launch_bounds__(256) void decode_prep_kernel(const __bf16* __restrict__ q, long q0, long q1, const __bf16* __restrict__ k, long k0, long k1,
+                                                          const __bf16* __restrict__ v, long v0, long v1, int b, int hq, int hk,
+                                                          const float* __restrict__ freqs, int pos, __bf16* __restrict__ rq,
+                                                          __bf16* __restrict__ krow, long kr0, long kr1, __bf16* __restrict__ vrow, long vr0, long vr1) {
+  constexpr int LPR = D / 8, RPB = 256 / LPR;
+  const int per = hq + 2 * hk;
+  const long row = (long)blockIdx.x * RPB + threadIdx.x / LPR;
+  if (row >= (long)b * per) return;
+  const int c = threadIdx.x % LPR;
+  const int bb = (int)(row / per), r = (int)(row % per);
+  const __bf16* src;
+  __bf16* dst;
+  bool rot = true;
+  if (r < hq) { src = q + bb * q0 + r * q1; dst = rq + ((long)bb * hq + r) * D; }
+  else if (r < hq + hk) { src = k + bb * k0 + (r - hq) * k1; dst = krow + bb * kr0 + (r - hq) * kr1; }
+  else { src = v + bb * v0 + (r - hq - hk) * v1; dst = vrow + bb * vr0 + (r - hq - hk) * vr1; rot = false; }
+  const bf16x8 x = load8(src + 8 * c);
+  bf16x8 o = x;
+  if (rot) {
+    const float p = (float)pos;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float sn, cs;
+      sincosf(p * freqs[4 * c + e], &sn, &cs);
+      const float a = (float)x[2 * e], bq = (float)x[2 * e + 1];
+      o[2 * e] = (__bf16)(a * cs - bq * sn);
+      o[2 * e + 1] = (__bf16)(bq * cs + a * sn);
+    }
+  }
+  *reinterpret_cast<bf16x8*>(dst + 8 * c) = o;
+}
+
 }  // namespace nsa
+
+extern "C" int nsa_decode_prep(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v,
+                               const int64_t* v_stride, int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head,
+                               const float* freqs, int32_t pos, void* rq, void* k_row, const int64_t* k_row_stride, void* v_row,
+                               const int64_t* v_row_stride, void* stream) {
+  using namespace nsa;
+  if (!q || !k || !v || !q_stride || !k_stride || !v_stride || !freqs || !rq || !k_row || !v_row || !k_row_stride || !v_row_stride)
+    return NSA_E_ARG;
+  if (batch <= 0 || heads <= 0 || kv_heads <= 0 || pos < 0) return NSA_E_ARG;
+  if ((q_stride[0] | q_stride[1] | k_stride[0] | k_stride[1] | v_stride[0] | v_stride[1] | k_row_stride[0] | k_row_stride[1] |
+       v_row_stride[0] | v_row_stride[1]) & 7)
+    return NSA_E_ARG;
+  const long rows = (long)batch * (heads + 2 * kv_heads);
+  hipStream_t st = (hipStream_t)stream;
+  if (dim_head == 64) {
+    hipLaunchKernelGGL((decode_prep_kernel<64>), dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, (const __bf16*)q, (long)q_stride[0],
+                       (long)q_stride[1], (const __bf16*)k, (long)k_stride[0], (long)k_stride[1], (const __bf16*)v, (long)v_stride[0],
+                       (long)v_stride[1], batch, heads, kv_heads, freqs, pos, (__bf16*)rq, (__bf16*)k_row, (long)k_row_stride[0],
+                       (long)k_row_stride[1], (__bf16*)v_row, (long)v_row_stride[0], (long)v_row_stride[1]);
+  } else if (dim_head == 128) {
+    hipLaunchKernelGGL((decode_prep_kernel<128>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const __bf16*)q, (long)q_stride[0],
+                       (long)q_stride[1], (const __bf16*)k, (long)k_stride[0], (long)k_stride[1], (const __bf16*)v, (long)v_stride[0],
+                       (long)v_stride[1], batch, heads, kv_heads, freqs, pos, (__bf16*)rq, (__bf16*)k_row, (long)k_row_stride[0],
+                       (long)k_row_stride[1], (__bf16*)v_row, (long)v_row_stride[0], (long)v_row_stride[1]);
+  } else {
+    return NSA_E_UNSUPPORTED;
+  }
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
 
 extern "C" int nsa_rope(const void* x, const int64_t* x_stride, int32_t batch, int32_t heads, int32_t seq, int32_t dim_head,
                         const float* freqs, int32_t offset, int32_t inverse, void* out, const int64_t* out_stride, void* stream) {

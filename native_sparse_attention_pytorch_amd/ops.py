@@ -325,8 +325,7 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
 
 # ------------------------------------------------------------------------------------ top-k
 
-@torch.library.custom_op("nsa_amd::topk", mutates_args=())
-def topk_op(scores: Tensor, k: int, apply_softmax: bool) -> tuple[Tensor, Tensor, Tensor]:
+def _topk_impl(scores: Tensor, k: int, apply_softmax: bool):
     if scores.dtype != torch.float32 or not scores.is_cuda:
         raise RuntimeError("importance scores must be fp32 device tensors")
     scores = scores.contiguous()
@@ -338,6 +337,11 @@ def topk_op(scores: Tensor, k: int, apply_softmax: bool) -> tuple[Tensor, Tensor
     fm = torch.empty(shp, dtype=torch.uint8, device=scores.device)
     _lib.check(_lib.lib().nsa_topk(_ptr(scores), rows, nb, k, int(apply_softmax), _ptr(idx), _ptr(vals), _ptr(fm), _stream()), "nsa_topk")
     return idx, vals, fm
+
+
+@torch.library.custom_op("nsa_amd::topk", mutates_args=())
+def topk_op(scores: Tensor, k: int, apply_softmax: bool) -> tuple[Tensor, Tensor, Tensor]:
+    return _topk_impl(scores, k, apply_softmax)
 
 
 @topk_op.register_fake
@@ -371,10 +375,12 @@ def importance_topk(importance_logits: Tensor, num_selected: int):
     """softmax with the -1e3 pad column (NSA.py:693-695) + topk (NSA.py:713) + `> 1e-10` mask
     (NSA.py:721).  Returns (values fp32, indices int32, fmask bool), each [..., num_selected];
     `values` is differentiable with respect to the logits."""
-    if importance_logits.requires_grad:
+    if importance_logits.requires_grad and torch.is_grad_enabled():
         vals, idx, fm = _ImportanceTopk.apply(importance_logits, int(num_selected))
-    else:
+    elif torch.compiler.is_compiling():
         idx, vals, fm = topk_op(importance_logits, int(num_selected), True)
+    else:
+        idx, vals, fm = _topk_impl(importance_logits, int(num_selected), True)     # eager inference: skip the dispatcher
     return vals, idx, fm.view(torch.bool)
 
 
@@ -491,15 +497,17 @@ def rotary_into(x: Tensor, freqs: Tensor, offset: int, out: Tensor) -> None:
 
 # ---------------------------------------------------------------------------------- decode
 
-def _decode_call(dsc, q, k, v, mem_k, mem_v, idx, fmask, logits):
+def _decode_call(dsc, q, k, v, mem_k, mem_v, idx, fmask, logits, merge=True):
+    """Runs the split-K walk; with merge the head outputs 'b hq 1 d', otherwise the workspace
+    holding the partials (for decode_combine)."""
     L = _lib.lib()
     nbytes = C.c_size_t()
     _lib.check(L.nsa_decode_workspace_bytes(C.byref(dsc), C.byref(nbytes)), "nsa_decode_workspace_bytes")
     ws = torch.empty(max(nbytes.value, 16), dtype=torch.uint8, device=q.device)
-    out = torch.empty((q.shape[0], q.shape[1], 1, q.shape[3]), dtype=_BF16, device=q.device)
+    out = torch.empty((q.shape[0], q.shape[1], 1, q.shape[3]), dtype=_BF16, device=q.device) if merge else None
     _lib.check(L.nsa_decode_attend(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(mem_k), _ptr(mem_v), _ptr(idx), _ptr(fmask),
                                    _ptr(ws), nbytes, _ptr(out), _ptr(logits), _stream()), "nsa_decode_attend")
-    return out
+    return out if merge else (dsc, ws)
 
 
 def _decode_desc(q: Tensor, k: Tensor | None, v: Tensor | None, hk: int):
@@ -522,11 +530,12 @@ def _decode_desc(q: Tensor, k: Tensor | None, v: Tensor | None, hk: int):
 
 @torch.no_grad()
 def decode_range_attend(q: Tensor, k: Tensor, v: Tensor, start: int, count: int, mem_k: Tensor | None = None,
-                        mem_v: Tensor | None = None, return_logits: bool = False):
+                        mem_v: Tensor | None = None, return_logits: bool = False, merge: bool = True):
     """One query token 'b hq 1 d' attends keys [start, start+count) of the caches 'b hk cap d',
     preceded by the memory rows mem_k / mem_v 'hk m d' (compressed branch NSA.py:396-420; sliding
     branch NSA.py:519-530).  With return_logits also scale * q.k over the cache keys, fp32
-    'b hq count' (NSA.py:444)."""
+'b hq count' (NSA.py:444).  merge=False returns a handle for decode_combine in place of
+    the output."""
     q = _prep(q)
     hk = k.shape[1]
     if start < 0 or count < 0 or start + count > k.shape[2] or k.shape != v.shape:
@@ -541,12 +550,12 @@ def decode_range_attend(q: Tensor, k: Tensor, v: Tensor, start: int, count: int,
             raise RuntimeError("decode_range_attend: memory rows must be 'hk m d'")
     dsc.num_mem = m
     logits = torch.empty((q.shape[0], q.shape[1], count), dtype=torch.float32, device=q.device) if return_logits else None
-    out = _decode_call(dsc, q, k if count else None, v if count else None, mem_k, mem_v, None, None, logits)
+    out = _decode_call(dsc, q, k if count else None, v if count else None, mem_k, mem_v, None, None, logits, merge)
     return (out, logits) if return_logits else out
 
 
 @torch.no_grad()
-def decode_select_attend(q: Tensor, k: Tensor, v: Tensor, kv_len: int, block: int, idx: Tensor, fmask: Tensor):
+def decode_select_attend(q: Tensor, k: Tensor, v: Tensor, kv_len: int, block: int, idx: Tensor, fmask: Tensor, merge: bool = True):
     """One query token at position kv_len-1 attends the blocks idx[..., slot] (where fmask) and
     its own block up to itself (NSA.py:446-515).  idx / fmask: 'b hk 1 S' or, for per-head
     selection, 'b hq 1 S'."""
@@ -565,4 +574,43 @@ def decode_select_attend(q: Tensor, k: Tensor, v: Tensor, kv_len: int, block: in
     dsc.idx_is_int64 = int(idx.dtype == torch.int64)
     idx = idx.contiguous()
     fm = fmask.contiguous().view(torch.uint8) if fmask.dtype == torch.bool else fmask.to(torch.uint8).contiguous()
-    return _decode_call(dsc, q, k, v, None, None, idx if idx.numel() else None, fm if fm.numel() else None, None)
+    return _decode_call(dsc, q, k, v, None, None, idx if idx.numel() else None, fm if fm.numel() else None, None, merge)
+
+
+@torch.no_grad()
+def decode_combine(gate_logits: Tensor, compressed, selected, sliding) -> Tensor:
+    """Merges the three branches (handles from decode_*_attend(..., merge=False); None for a
+    branch that contributes nothing), applies sigmoid(gate_logits 'b 1 (h 3)') and merges the
+    heads: 'b 1 (h d)' (NSA.py:534-545)."""
+    ref = next(h for h in (compressed, selected, sliding) if h is not None)[0]
+    b, hq, d = ref.batch, ref.kv_heads * ref.group, ref.dim_head
+    gl = gate_logits.to(_BF16).contiguous()
+    if gl.numel() != b * hq * 3:
+        raise RuntimeError("decode_combine: gate logits must be 'b 1 (h 3)'")
+    out = torch.empty((b, 1, hq * d), dtype=_BF16, device=gl.device)
+    args = []
+    for h in (compressed, selected, sliding):
+        args += [None, None] if h is None else [C.byref(h[0]), _ptr(h[1])]
+    _lib.check(_lib.lib().nsa_decode_combine(*args, _ptr(gl), _ptr(out), _stream()), "nsa_decode_combine")
+    return out
+
+
+@torch.no_grad()
+def decode_prep(q: Tensor, k: Tensor, v: Tensor, freqs: Tensor, pos: int, k_row: Tensor, v_row: Tensor) -> Tensor:
+    """New token's q 'b hq 1 d', k, v 'b hk 1 d' (bf16 views are fine): returns the rotated
+    queries and writes the rotated keys / the values into the cache rows k_row, v_row 'b hk 1 d'
+    (NSA.py:384-393)."""
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    b, hq, _, d = q.shape
+    hk = k.shape[1]
+    for t in (k_row, v_row):
+        if t.dtype != _BF16 or t.shape != (b, hk, 1, d) or not _rows_ok(t):
+            raise RuntimeError("decode_prep: cache rows must be bf16 'b hk 1 d' views with 16-byte aligned rows")
+    freqs = freqs.detach()
+    if freqs.dtype != torch.float32 or not freqs.is_contiguous():
+        freqs = freqs.to(torch.float32).contiguous()
+    rq = torch.empty((b, hq, 1, d), dtype=_BF16, device=q.device)
+    s2 = lambda t: (C.c_int64 * 2)(t.stride(0), t.stride(1))
+    _lib.check(_lib.lib().nsa_decode_prep(_ptr(q), s2(q), _ptr(k), s2(k), _ptr(v), s2(v), b, hq, hk, d, _ptr(freqs), int(pos), _ptr(rq),
+                                          _ptr(k_row), s2(k_row), _ptr(v_row), s2(v_row), _stream()), "nsa_decode_prep")
+    return rq

@@ -48,7 +48,7 @@ class RotaryEmbedding(nn.Module):
         return self.rotate(q, offset=k.shape[-2] - q.shape[-2]), self.rotate(k)
 
 
-def _append_rows(t: torch.Tensor, extra: int = 1):
+def _append_rows(t: torch.Tensor, extra: int = 1, dtype=torch.bfloat16, min_capacity: int = 128):
     """Grow the 'b h n d' cache `t` by `extra` rows.  Returns (view of n+extra rows, view of the
     new rows).  When `t` is the filled prefix of a buffer made here, the rows are taken from the
     buffer's spare capacity; otherwise (a cache from the parallel forward, a branch point that
@@ -56,11 +56,11 @@ def _append_rows(t: torch.Tensor, extra: int = 1):
     the size first, so a caller that keeps an old cache tuple never sees it change."""
     b, h, n, d = t.shape
     base = t._base
-    ok = (base is not None and getattr(base, "_nsa_filled", -1) == n and base.dtype == torch.bfloat16
+    ok = (base is not None and getattr(base, "_nsa_filled", -1) == n and base.dtype == dtype
           and base.dim() == 4 and base.shape[2] >= n + extra and base.shape[:2] == t.shape[:2] and base.shape[3] == d
           and t.data_ptr() == base.data_ptr() and t.stride() == base.stride())
     if not ok:
-        base = torch.empty((b, h, max(2 * (n + extra), 128), d), dtype=torch.bfloat16, device=t.device)
+        base = torch.empty((b, h, max(2 * (n + extra), min_capacity), d), dtype=dtype, device=t.device)
         base[:, :, :n].copy_(t)
     base._nsa_filled = n + extra
     return base[:, :, :n + extra], base[:, :, n:n + extra]
@@ -184,28 +184,27 @@ class SparseAttention(nn.Module):
         x = self.norm(inp)
         q, k, v = self.to_qkv(x).split(self.qkv_split, dim=-1)
         q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
-        q16, k16 = q.to(bf16), k.to(bf16)
+        q16, k16, v16 = q.to(bf16), k.to(bf16), v.to(bf16)
 
         # raw tokens of the open compression window (not rotated, NSA.py:377-380)
-        run_k, run_v = torch.cat((run_k, k.to(run_k.dtype)), dim=-2), torch.cat((run_v, v.to(run_v.dtype)), dim=-2)
+        run_k, rk_row = _append_rows(run_k, dtype=run_k.dtype, min_capacity=cbs)
+        run_v, rv_row = _append_rows(run_v, dtype=run_v.dtype, min_capacity=cbs)
+        rk_row.copy_(k)
+        rv_row.copy_(v)
 
         # the rotated key and the value go into row t of the caches (NSA.py:384-393)
         keys, k_row = _append_rows(cache_k)
         vals, v_row = _append_rows(cache_v)
-        ops.rotary_into(k16, freqs, t, k_row)
-        v_row.copy_(v)
-        rq16 = ops.rotary(q16, freqs, t)
+        rq16 = ops.decode_prep(q16, k16, v16, freqs, t, k_row, v_row)
 
         # 1. compressed branch: every cached compressed key, no mask (NSA.py:396-420)
         nc = cache_ck.shape[-2]
-        logits = None
+        logits = c_part = None
         if nc > 0:
             ck16 = cache_ck if cache_ck.dtype == bf16 else cache_ck.to(bf16)
             cv16 = cache_cv if cache_cv.dtype == bf16 else cache_cv.to(bf16)
-            c_out, logits = ops.decode_range_attend(q16, ck16, cv16, 0, nc, self.compress_mem_kv[0], self.compress_mem_kv[1],
-                                                    return_logits=True)
-        else:
-            c_out = torch.zeros_like(q16)
+            c_part, logits = ops.decode_range_attend(q16, ck16, cv16, 0, nc, self.compress_mem_kv[0], self.compress_mem_kv[1],
+                                                     return_logits=True, merge=False)
 
         # a compression window is complete: compress it, keep the overlap (NSA.py:422-441)
         ck, cv = cache_ck, cache_cv
@@ -229,14 +228,14 @@ class SparseAttention(nn.Module):
         else:
             idx = torch.zeros((b, self.kv_heads, 1, 0), dtype=torch.int32, device=inp.device)
             fmask = idx.bool()
-        f_out = ops.decode_select_attend(rq16, keys, vals, t + 1, B, idx, fmask)
+        f_part = ops.decode_select_attend(rq16, keys, vals, t + 1, B, idx, fmask, merge=False)
 
         # 3. sliding branch: the last window + 1 keys (NSA.py:519-530)
         w = min(t + 1, self.sliding_window_size + 1)
-        s_out = ops.decode_range_attend(rq16, keys, vals, t + 1 - w, w)
+        s_part = ops.decode_range_attend(rq16, keys, vals, t + 1 - w, w, merge=False)
 
-        logits_g = self.to_strategy_combine[0](x)
-        merged = ops.gate_combine(logits_g, c_out, f_out, s_out)
+        # merge of the split-K partials, sigmoid gate and head merge in one kernel (NSA.py:534-545)
+        merged = ops.decode_combine(self.to_strategy_combine[0](x), c_part, f_part, s_part)
         out = self.combine_heads(merged.to(x.dtype))
         if not return_cache:
             return out

@@ -97,6 +97,55 @@ def test_rotary_into_cache_slot():
     assert cache[:, :, :17].abs().max() == 0 and cache[:, :, 18:].abs().max() == 0
 
 
+def test_decode_prep_rotates_and_fills_cache_rows():
+    from native_sparse_attention_pytorch_amd.ops import decode_prep
+    g = torch.Generator().manual_seed(6)
+    b, hq, hk, d, pos = 3, 8, 2, 128, 301
+    qkv = _rand((b, 1, (hq + 2 * hk) * d), g)                     # the projection's layout: heads are views
+    q, k, v = (t.view(b, 1, -1, d).permute(0, 2, 1, 3) for t in qkv.split((hq * d, hk * d, hk * d), dim=-1))
+    rot = O.RotaryEmbedding(d)
+    kc = torch.zeros(b, hk, 400, d, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    qkv_d = qkv.to(DEV)
+    qd, kd, vd = (t.view(b, 1, -1, d).permute(0, 2, 1, 3) for t in qkv_d.split((hq * d, hk * d, hk * d), dim=-1))
+    rq = decode_prep(qd, kd, vd, rot.freqs.to(DEV), pos, kc[:, :, pos:pos + 1], vc[:, :, pos:pos + 1])
+    torch.cuda.synchronize()
+    assert_close(rq, rot.rotate(q.float(), offset=pos), 3e-2, 1e-2, "rotated queries")
+    assert_close(kc[:, :, pos:pos + 1], rot.rotate(k.float(), offset=pos), 3e-2, 1e-2, "rotated key row")
+    assert torch.equal(vc[:, :, pos].cpu(), v[:, :, 0])
+    kc[:, :, pos] = 0
+    vc[:, :, pos] = 0
+    assert kc.abs().max() == 0 and vc.abs().max() == 0, "rows other than `pos` were written"
+
+
+@pytest.mark.parametrize("with_compressed", [True, False])
+def test_decode_combine_matches_oracle_gate(with_compressed):
+    """Fused merge + sigmoid gate + head merge against the oracle's gate applied to the three
+    separately merged branch outputs."""
+    from native_sparse_attention_pytorch_amd import ops
+    g = torch.Generator().manual_seed(8)
+    b, hq, hk, d, n = 2, 8, 2, 64, 500
+    q = _rand((b, hq, 1, d), g).to(DEV)
+    k, v = _rand((b, hk, n, d), g).to(DEV), _rand((b, hk, n, d), g).to(DEV)
+    ck, cv = _rand((b, hk, 60, d), g).to(DEV), _rand((b, hk, 60, d), g).to(DEV)
+    mk, mv = _rand((hk, 1, d), g).to(DEV), _rand((hk, 1, d), g).to(DEV)
+    idx = torch.tensor([3, 0, 5], dtype=torch.int32, device=DEV).expand(b, hk, 1, 3).contiguous()
+    live = torch.ones_like(idx, dtype=torch.bool)
+    logits = _rand((b, 1, 3 * hq), g, 2.0).to(DEV)
+    outs, parts = [], []
+    for merge in (True, False):
+        c = ops.decode_range_attend(q, ck, cv, 0, 60, mk, mv, merge=merge) if with_compressed else None
+        f = ops.decode_select_attend(q, k, v, n, 64, idx, live, merge=merge)
+        s_ = ops.decode_range_attend(q, k, v, n - 33, 33, merge=merge)
+        (outs if merge else parts).extend([c, f, s_])
+    got = ops.decode_combine(logits, *parts)
+    torch.cuda.synchronize()
+    c, f, s_ = (torch.zeros(b, hq, 1, d) if t is None else t.float().cpu() for t in outs)
+    want = O.gate_combine(logits.float().cpu(), c, f, s_)
+    assert got.shape == (b, 1, hq * d)
+    assert_close(got, want, 2e-2, 1e-2, "decode combine")
+
+
 def _pair(seed, **kw):
     from native_sparse_attention_pytorch_amd.sparse_attention import SparseAttention
     torch.manual_seed(seed)
