@@ -15,6 +15,10 @@ DEV = "cuda"
 def _pair(seed, **kw):
     from native_sparse_attention_pytorch_amd.sparse_attention import SparseAttention
     torch.manual_seed(seed)
+    kw = dict(kw)
+    if kw.get("compress_mlp") == "grouped":      # per-head MLP, the network train.py:100-104 installs
+        from native_sparse_attention_pytorch_amd.compress_networks import GroupedMLP
+        kw["compress_mlp"] = GroupedMLP(dim_head=kw["dim_head"], compress_window_size=kw["compress_block_size"], heads=kw["kv_heads"])
     ref = O.SparseAttentionOracle(**kw)
     # move the module away from its symmetric init so every branch and parameter matters
     with torch.no_grad():
@@ -40,6 +44,9 @@ CONFIGS = [
          compress_block_sliding_stride=16, selection_block_size=64, num_selected_blocks=3, causal=True),
     dict(dim=128, dim_head=64, heads=4, kv_heads=4, sliding_window_size=16, compress_block_size=8,
          compress_block_sliding_stride=4, selection_block_size=16, num_selected_blocks=2, causal=False),
+    dict(dim=256, dim_head=64, heads=8, kv_heads=2, sliding_window_size=64, compress_block_size=16,
+         compress_block_sliding_stride=8, selection_block_size=32, num_selected_blocks=4, causal=True, use_diff_topk=True,
+         compress_mlp="grouped"),
 ]
 
 
