@@ -11,6 +11,10 @@ reference's pure-torch path (`use_triton_kernel=False`):
       :153-184  attend()                       -> attend
       :270-275  split_compress_window          -> compress_windows
       :549-867  SparseAttention.forward        -> SparseAttentionOracle.forward
+      :338-547  forward_inference              -> SparseAttentionOracle.forward_inference
+  native_sparse_attention_pytorch/transformer.py
+      :254-330  Transformer.forward (+ caches) -> TransformerOracle.forward
+      :213-252  Transformer.sample             -> TransformerOracle.sample
       :46-109   mask closed forms              -> sliding_mask / compress_mask / fine_mask
   test_triton_nsa.py:32-133 regular_attend     -> select_attend (functional contract of
                                                   native_sparse_attend, TRI.py:1938-1987)
@@ -24,6 +28,9 @@ What pins each function (see tests/test_oracle_*.py):
                                 S=0 -> block-diagonal; S>=W -> full causal attention
   sliding_attend              : SDPA with the band mask (NSA.py:48-56); win>=n -> causal
   gate combine                : closed form at init (sigmoid([-2,-2,2]))
+  forward_inference, caches   : the reference's own criterion (tests/test_sparse_attn.py:50-118):
+                                token-by-token decode == parallel forward to 1e-5; greedy
+                                sampling with and without caches gives the same tokens
 
 PARITY UNPINNED (third-party packages absent from the reference tree and from this
 image, so no fixture can be produced): the numeric convention of
