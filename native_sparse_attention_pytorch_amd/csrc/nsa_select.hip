@@ -314,6 +314,9 @@ __device__ __forceinline__ void store_tile_rows(const floatx16 (&acc)[D / 32], f
 
 // ------------------------------------------------------------------------------- forward
 
+#ifndef NSA_FWD_STAGES
+#define NSA_FWD_STAGES 1      // measured on MI355X (seq 32k, d 128): 1 stage 1.69 ms, 2 or 3 stages 1.77 ms
+#endif
 template <int D, int KT>
 __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                      const __bf16* __restrict__ v, const char* __restrict__ iws, char* __restrict__ fws) {
@@ -362,21 +365,30 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
   const float sc = P.scale * kLog2e;
   const int ppt = 32 >> P.lg;
 
-  // software pipeline: list entries two tiles ahead, Q rows (coalesced gather) one tile ahead
+  // software pipeline: NS tiles of Q rows (coalesced gathers) in flight, list entries one more tile
+  // ahead; a stage's registers take the loads of the tile NS steps ahead once it is committed to LDS
   const __bf16* qbase = q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1];
-  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + ppt, n_);
-  RowInfo r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0, n_), n_);
-  bf16x8 rawq[KS];
-  issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], r.i, P.g - 1, lane);
+  constexpr int NS = NSA_FWD_STAGES;
+  struct Stage {
+    RowInfo r;
+    bf16x8 raw[KS];
+  };
+  Stage stg[NS];
+#pragma unroll
+  for (int s2 = 0; s2 < NS; ++s2) {
+    stg[s2].r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0 + s2 * ppt, n_), n_);
+    issue_tile_loads<D>(stg[s2].raw, qbase, P.sq[1], P.sq[2], stg[s2].r.i, P.g - 1, lane);
+  }
+  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + NS * ppt, n_);
 
   wait_all_loads();        // enter the loop with nothing pending, so the loop itself only waits for what it needs
-  for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
-    commit_tile<D>(rawq, xq_s, RS, lane);
+  auto step = [&](int vt, Stage& cur) {
+    const RowInfo r = cur.r;
+    commit_tile<D>(cur.raw, xq_s, RS, lane);
     __syncthreads();
-    // issue the next tile's loads and the entry fetch of the tile after it
-    const RowInfo rn = decode_entry(P, ui, e_n, n_);
-    issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], rn.i, P.g - 1, lane);
-    const RawEntry e_nn = fetch_entry(P, list, ui, vt + 2 * ppt, n_);
+    cur.r = decode_entry(P, ui, e_n, n_);
+    issue_tile_loads<D>(cur.raw, qbase, P.sq[1], P.sq[2], cur.r.i, P.g - 1, lane);
+    e_n = fetch_entry(P, list, ui, vt + (NS + 1) * ppt, n_);
     __builtin_amdgcn_sched_barrier(0);
 
     bf16x8 Qf[KS];
@@ -432,7 +444,11 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
       store_tile_rows<D>(Oa, inv, row, opart, tile_s, row_s, lane);
       if (h == 0) lsepart[row] = (mx + fast_log2(l)) * kLn2;
     }
-    r = rn; e_n = e_nn;
+  };
+  for (int vt = ui.v0; vt < ui.v1; vt += NS * ppt) {
+#pragma unroll
+    for (int s2 = 0; s2 < NS; ++s2)
+      if (vt + s2 * ppt < ui.v1) step(vt + s2 * ppt, stg[s2]);
   }
 }
 
@@ -705,6 +721,9 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 // [key][row] in LDS; dQ^T = K^T dS^T is then formed with both operands read through the
 // transpose load (K block row-major in LDS, loaded once per unit), each wave taking half of the
 // features, and the finished 32 x D tile leaves through coalesced row stores.
+#ifndef NSA_BWD_STAGES
+#define NSA_BWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1 stage 3.86 ms, 2: 3.44, 3: 3.53, 4: 3.60
+#endif
 template <int D, int KT, bool FUSE_DQ>
 __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                               const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
@@ -729,7 +748,7 @@ __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, c
   UnitInfo ui;
   if (!locate_unit(P, iws, 2, bh, u, ui)) return;
   const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
-  const bool load_q = KT == 1 || kt == 0, load_g = KT == 1 || kt == 1;
+  const bool load_q = kt == 0;                 // with two waves: wave 0 gathers Q rows, wave 1 dO rows; one wave does both
 
   bf16x8 Kf[KS], Vf[KS];
   const int kl = 32 * kt + n_;                 // this lane's key inside the block
@@ -760,42 +779,53 @@ __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, c
   const __bf16* gbase = dout + b * P.so[0] + (long)(hk * P.g) * P.so[1];
   __bf16* dqpart = reinterpret_cast<__bf16*>(bws + P.off_dqpart);
 
-  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + ppt, n_);
-  RowInfo r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0, n_), n_);
-  bf16x8 rawq[KS], rawg[KS];
-  float lse_r, del_r;
-  {
-    if (load_q) issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], r.i, P.g - 1, lane);
-    if (load_g) issue_tile_loads<D>(rawg, gbase, P.so[1], P.so[2], r.i, P.g - 1, lane);
-    const size_t srow = ((size_t)b * HQ + hk * P.g + r.g) * P.n + r.i;
-    lse_r = lse[srow] * kLog2e;
-    del_r = delta[srow];
-  }
+  // software pipeline with NS tiles of rows in flight: when a stage has been committed to LDS its
+  // registers take the loads of the tile NS steps ahead.  List entries run one more tile ahead.
+  constexpr int NR = KT == 1 ? 2 : 1;
+  struct Stage {
+    RowInfo r;
+    bf16x8 raw[NR][KS];      // this wave's share of the tile: Q rows (wave 0) or dO rows (wave 1); both with one wave
+    float lse_r, del_r;
+  };
+  auto issue = [&](Stage& st, const RowInfo& rr) {
+    st.r = rr;
+    if (KT == 1) {
+      issue_tile_loads<D>(st.raw[0], qbase, P.sq[1], P.sq[2], rr.i, P.g - 1, lane);
+      issue_tile_loads<D>(st.raw[NR - 1], gbase, P.so[1], P.so[2], rr.i, P.g - 1, lane);
+    } else {
+      issue_tile_loads<D>(st.raw[0], load_q ? qbase : gbase, load_q ? P.sq[1] : P.so[1], load_q ? P.sq[2] : P.so[2], rr.i, P.g - 1, lane);
+    }
+    const size_t srow = ((size_t)b * HQ + hk * P.g + rr.g) * P.n + rr.i;
+    st.lse_r = lse[srow] * kLog2e;
+    st.del_r = delta[srow];
+  };
+  constexpr int NS = KT == 1 ? 1 : NSA_BWD_STAGES;      // a single wave gathers both tiles: no registers for a second stage
+  Stage stg[NS];
+#pragma unroll
+  for (int s2 = 0; s2 < NS; ++s2) issue(stg[s2], decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0 + s2 * ppt, n_), n_));
+  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + NS * ppt, n_);
 
   wait_all_loads();        // enter the loop with nothing pending, so the loop itself only waits for what it needs
-  for (int vt = ui.v0; vt < ui.v1; vt += ppt) {
-    // commit the current tile (loaded during the previous iteration) to LDS
-    if (load_q) commit_tile<D>(rawq, xq_s, RS, lane);
-    if (load_g) commit_tile<D>(rawg, xg_s, RS, lane);
+  auto step = [&](int vt, Stage& cur) {
+    const RowInfo r = cur.r;
+    // commit the current tile to LDS
+    if (KT == 1) {
+      commit_tile<D>(cur.raw[0], xq_s, RS, lane);
+      commit_tile<D>(cur.raw[NR - 1], xg_s, RS, lane);
+    } else {
+      commit_tile<D>(cur.raw[0], load_q ? xq_s : xg_s, RS, lane);
+    }
     if (kt == 0 && h == 0) {
-      lse_s[n_] = r.valid ? lse_r : INFINITY;              // +inf: a padding row gets p = 0
-      del_s[n_] = del_r;
+      lse_s[n_] = r.valid ? cur.lse_r : INFINITY;          // +inf: a padding row gets p = 0
+      del_s[n_] = cur.del_r;
       lim_s[n_] = r.lim;
       if (FUSE_DQ) row_s[n_] = r.valid ? (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g : P.prow;
     }
     __syncthreads();
 
-    // issue the next tile's loads and the entry fetch of the tile after it
-    const RowInfo rn = decode_entry(P, ui, e_n, n_);
-    if (load_q) issue_tile_loads<D>(rawq, qbase, P.sq[1], P.sq[2], rn.i, P.g - 1, lane);
-    if (load_g) issue_tile_loads<D>(rawg, gbase, P.so[1], P.so[2], rn.i, P.g - 1, lane);
-    float lse_n, del_n;
-    {
-      const size_t srown = ((size_t)b * HQ + hk * P.g + rn.g) * P.n + rn.i;
-      lse_n = lse[srown] * kLog2e;
-      del_n = delta[srown];
-    }
-    const RawEntry e_nn = fetch_entry(P, list, ui, vt + 2 * ppt, n_);
+    // the freed stage takes the loads of the tile two steps ahead; fetch the entry of the tile after that
+    issue(cur, decode_entry(P, ui, e_n, n_));
+    e_n = fetch_entry(P, list, ui, vt + (NS + 1) * ppt, n_);
     __builtin_amdgcn_sched_barrier(0);
 
     floatx16 Sa = zero_acc(), Pa = zero_acc();
@@ -870,8 +900,11 @@ __global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, c
       }
       __syncthreads();
     }
-    lse_r = lse_n; del_r = del_n;
-    r = rn; e_n = e_nn;
+  };
+  for (int vt = ui.v0; vt < ui.v1; vt += NS * ppt) {
+#pragma unroll
+    for (int s2 = 0; s2 < NS; ++s2)
+      if (vt + s2 * ppt < ui.v1) step(vt + s2 * ppt, stg[s2]);
   }
 
   // partial [unit][2][32*KT keys][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][key kl]
