@@ -16,6 +16,7 @@
 // reads, transposed operands (V^T, K^T) with the gfx950 LDS transpose load.  dK/dV is
 // key-stationary: two waves own a 64-key tile (32 keys each) and stream the query rows that can
 // see it, like the dK/dV walk of the block-selection kernels.
+#include <type_traits>
 #include "nsa_common.hpp"
 #include "nsa_dense_plan.hpp"
 
@@ -104,6 +105,8 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
   const TileWalk walk = make_walk(P, q0, min(P.n - 1, q0 + 4 * ppt - 1));
   // this wave's own reach (its tiles are a subset of the work-group's)
   const int my_hi = visible_range(P, min(P.n - 1, i0 + ppt - 1)).hi, my_lo = visible_range(P, min(i0, P.n - 1)).lo;
+  // keys in [all_lo, all_hi] are visible to every row of this wave: tiles inside need no per-element mask
+  const int all_hi = visible_range(P, min(i0, P.n - 1)).hi, all_lo = visible_range(P, min(P.n - 1, i0 + ppt - 1)).lo;
   const float sc = P.scale * kLog2e;
 
   float m = -INFINITY, l = 0.f;
@@ -145,15 +148,19 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
       floatx16 Sraw[2];
       if (POOL) { Sraw[0] = Sa[0]; Sraw[1] = Sa[1]; }
       float tmax = -INFINITY;
+      auto scale_scores = [&](auto masked) {
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+        for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int i2 = 0; i2 < 16; ++i2) {
-          const int key = kb0 + 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
-          const float s = (key >= klo && key <= khi) ? Sa[kt][i2] * sc : -INFINITY;
-          Sa[kt][i2] = s;
-          tmax = fmaxf(tmax, s);
-        }
+          for (int i2 = 0; i2 < 16; ++i2) {
+            const int key = kb0 + 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
+            const float s = (!decltype(masked)::value || (key >= klo && key <= khi)) ? Sa[kt][i2] * sc : -INFINITY;
+            Sa[kt][i2] = s;
+            tmax = fmaxf(tmax, s);
+          }
+      };
+      if (!memtile && kb0 >= all_lo && kb0 + kBK - 1 <= all_hi) scale_scores(std::false_type{});      // wave-uniform
+      else scale_scores(std::true_type{});
 
       if (POOL && !memtile) {
         // Block-importance logits of this 64-key tile: sum the raw scaled logits over the npf keys
@@ -336,6 +343,7 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P,
   const Interval me = visible_range(P, i);
   const TileWalk walk = make_walk(P, q0, min(P.n - 1, q0 + 4 * ppt - 1));
   const int my_hi = visible_range(P, min(P.n - 1, i0 + ppt - 1)).hi, my_lo = visible_range(P, min(i0, P.n - 1)).lo;
+  const int all_hi = visible_range(P, min(i0, P.n - 1)).hi, all_lo = visible_range(P, min(P.n - 1, i0 + ppt - 1)).lo;
   const float sc = P.scale * kLog2e;
   floatx16 Qa[DT];
 #pragma unroll
@@ -362,7 +370,7 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P,
     const bool memtile = t < 0;
     const int kb0 = memtile ? 0 : t * kBK;
     const bool active = memtile || (kb0 <= my_hi && kb0 + kBK - 1 >= my_lo);
-    if (active) {
+    auto tile_math = [&](auto masked) {
       floatx16 Sa[2], Pa[2];
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
@@ -379,7 +387,7 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P,
 #pragma unroll
         for (int i2 = 0; i2 < 16; ++i2) {
           const int key = kb0 + 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
-          const float p = (key >= klo && key <= khi) ? fast_exp2(Sa[kt][i2] * sc - lse_r) : 0.f;
+          const float p = (!decltype(masked)::value || (key >= klo && key <= khi)) ? fast_exp2(Sa[kt][i2] * sc - lse_r) : 0.f;
           Sa[kt][i2] = p * (Pa[kt][i2] - del_r);
         }
 #pragma unroll
@@ -391,6 +399,12 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P,
           for (int dt = 0; dt < DT; ++dt)
             Qa[dt] = mfma32(lds_transposed_operand(k_s, RS, 32 * kt + 16 * u2, 32 * dt, lane), Sf, Qa[dt]);
         }
+    };
+    if (active) {
+      // a tile every row of the wave sees completely needs no per-element mask (wave-uniform); each
+      // variant is one straight-line block so that VALU work and MFMAs can be interleaved
+      if (!memtile && kb0 >= all_lo && kb0 + kBK - 1 <= all_hi) tile_math(std::false_type{});
+      else tile_math(std::true_type{});
     }
     __syncthreads();
   }
@@ -529,6 +543,9 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
     }
     __builtin_amdgcn_sched_barrier(0);
 
+    // the whole tile's arithmetic as one straight-line block per variant (masked / unmasked), so that
+    // the scheduler can overlap the softmax VALU work with the MFMAs on either side of it
+    auto tile_math = [&](auto masked) {
     floatx16 Sa = zero_acc(), Pa = zero_acc();
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -536,18 +553,20 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
       Pa = mfma32(lds_row_operand(xg_s, RS, ks, lane), Vf[ks], Pa);
     }
     floatx16 dSa;
+    {
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      const floatx4 l4 = *reinterpret_cast<const floatx4*>(&lse_s[8 * a + 4 * h]);
-      const floatx4 d4 = *reinterpret_cast<const floatx4*>(&del_s[8 * a + 4 * h]);
-      const int* lo4 = &lo_s[8 * a + 4 * h];
-      const int* hi4 = &hi_s[8 * a + 4 * h];
+      for (int a = 0; a < 4; ++a) {
+        const floatx4 l4 = *reinterpret_cast<const floatx4*>(&lse_s[8 * a + 4 * h]);
+        const floatx4 d4 = *reinterpret_cast<const floatx4*>(&del_s[8 * a + 4 * h]);
+        const int* lo4 = &lo_s[8 * a + 4 * h];
+        const int* hi4 = &hi_s[8 * a + 4 * h];
 #pragma unroll
-      for (int bb = 0; bb < 4; ++bb) {
-        const int i2 = 4 * a + bb;
-        const float p = (kr_ >= lo4[bb] && kr_ <= hi4[bb]) ? fast_exp2(Sa[i2] * sc - l4[bb]) : 0.f;
-        Sa[i2] = p;
-        dSa[i2] = p * (Pa[i2] - d4[bb]);
+        for (int bb = 0; bb < 4; ++bb) {
+          const int i2 = 4 * a + bb;
+          const float p = (!decltype(masked)::value || (kr_ >= lo4[bb] && kr_ <= hi4[bb])) ? fast_exp2(Sa[i2] * sc - l4[bb]) : 0.f;
+          Sa[i2] = p;
+          dSa[i2] = p * (Pa[i2] - d4[bb]);
+        }
       }
     }
     const bf16x8 Pf0 = pack8(Sa, 0), Pf1 = pack8(Sa, 8);
@@ -558,6 +577,16 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
       dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 16, 32 * dt, lane), Pf1, dVa[dt]);
       dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 0, 32 * dt, lane), Sf0, dKa[dt]);
       dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 16, 32 * dt, lane), Sf1, dKa[dt]);
+    }
+    };
+    {
+      // rows of this wave are visible to every query of the tile iff they lie between the largest lower
+      // and the smallest upper bound, which consecutive queries take at the tile's ends (wave-uniform)
+      const Interval vf = visible_range(P, min(i0, P.n - 1)), vl = visible_range(P, min(i0 + ppt - 1, P.n - 1));
+      const int all_lo = P.mode == 0 ? vl.lo : 0, all_hi = P.mode == 0 ? vf.hi : vf.hi + P.mem;
+      const int r0 = kBK * T + 32 * kt;
+      if (r0 >= all_lo && r0 + 31 <= all_hi) tile_math(std::false_type{});
+      else tile_math(std::true_type{});
     }
     __syncthreads();
     lse_r = lse_n; del_r = del_n;
