@@ -1,32 +1,70 @@
 // Block-importance softmax and per-query top-k (NSA.py:693-713, 721): one wave per query row.
 // Input row: nb importance logits (fp32, -inf = cannot be selected).  The row is softmaxed with
 // the reference's extra -1e3 column (so a row with nothing visible becomes all zeros), then the
-// k largest probabilities are extracted in descending order, ties going to the lower block
-// index.  HBM-bound: reads nb*4 bytes per row, writes k*(4+4+1).
+// k (<= 64) largest probabilities are extracted in descending order, ties going to the lower
+// block index.  HBM-bound nominally: reads nb*4 bytes per row, writes k*(4+4+1).
+#include <type_traits>
 #include "nsa_common.hpp"
 #include "../../include/nsa_hip.h"
 
 namespace nsa {
 
+// max over the 64 lanes: DPP butterflies inside every row of 16 lanes (VALU speed, no LDS round
+// trips), then the four row maxima through readlane
+__device__ __forceinline__ float wave_max(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xF, 0xF, false));
+  };
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0xB1>{}));     // quad_perm [1,0,3,2]
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x4E>{}));     // quad_perm [2,3,0,1]
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x141>{}));    // row_half_mirror: quads of a half row
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x140>{}));    // row_mirror: the two half rows
+  const float a = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+  const float b = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+  const float c = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+  const float d = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+  return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+// Lane l holds the VPL consecutive entries l*VPL .. l*VPL+VPL-1 and, across rounds, its own best
+// remaining entry; a round is a value-only wave maximum, a ballot of the lanes that hold it (the
+// lowest lane holds the lowest index, and inside a lane the scan keeps the lower one: ties go to the
+// lower block index), and a re-scan in the winning lane.  Result s stays in lane s until the end,
+// so the outputs leave in one coalesced store each.
 template <int VPL>
-__global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in, long rows, int nb, int k, int softmax,
+__global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in, long rows, int nb, int k, int softmax, int vec4,
                                                    int* __restrict__ idx, float* __restrict__ vals, uint8_t* __restrict__ fmask) {
   const int lane = threadIdx.x & 63;
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const float* src = in + row * nb;
   float x[VPL];
+  bool loaded = false;
+  if constexpr (VPL % 4 == 0) {
+    if (vec4) {                                          // rows are 16-byte aligned and nb % 4 == 0
 #pragma unroll
-  for (int r = 0; r < VPL; ++r) {
-    const int j = lane + 64 * r;
-    x[r] = j < nb ? src[j] : -INFINITY;
+      for (int r4 = 0; r4 < VPL / 4; ++r4) {
+        const int j = lane * VPL + 4 * r4;
+        floatx4 t = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+        if (j < nb) t = *reinterpret_cast<const floatx4*>(src + j);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[4 * r4 + e] = t[e];
+      }
+      loaded = true;
+    }
+  }
+  if (!loaded) {
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+      const int j = lane * VPL + r;
+      x[r] = j < nb ? src[j] : -INFINITY;
+    }
   }
   if (softmax) {
     float mx = -1e3f;
 #pragma unroll
     for (int r = 0; r < VPL; ++r) mx = fmaxf(mx, x[r]);
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    mx = wave_max(mx);
     float sum = 0.f;
 #pragma unroll
     for (int r = 0; r < VPL; ++r) { x[r] = __expf(x[r] - mx); sum += x[r]; }
@@ -39,29 +77,36 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in,
   }
 #pragma unroll
   for (int r = 0; r < VPL; ++r)
-    if (lane + 64 * r >= nb) x[r] = -1.0f;               // padding loses against every real entry
-  for (int s = 0; s < k; ++s) {
-    float bv = x[0];
-    int bj = lane;
+    if (lane * VPL + r >= nb) x[r] = -1.0f;              // padding loses against every real entry
+
+  float bv;
+  int br;
+  auto rescan = [&]() {
+    bv = x[0]; br = 0;
 #pragma unroll
     for (int r = 1; r < VPL; ++r)
-      if (x[r] > bv) { bv = x[r]; bj = lane + 64 * r; }   // strict: ties keep the lower index
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) {
-      const float ov = __shfl_xor(bv, o, 64);
-      const int oj = __shfl_xor(bj, o, 64);
-      if (ov > bv || (ov == bv && oj < bj)) { bv = ov; bj = oj; }
-    }
-    if ((bj & 63) == lane) {
+      if (x[r] > bv) { bv = x[r]; br = r; }               // strict: ties keep the lower index
+  };
+  rescan();
+  float res_v = 0.f;
+  int res_j = 0;
+  for (int s = 0; s < k; ++s) {
+    const float m = wave_max(bv);
+    const unsigned long long holders = __ballot(bv == m);
+    const int w = __builtin_ctzll(holders);               // lowest lane = lowest index among equals
+    const int jw = __builtin_amdgcn_readlane(lane * VPL + br, w);
+    if (lane == s) { res_v = m; res_j = jw; }
+    if (lane == w) {
 #pragma unroll
       for (int r = 0; r < VPL; ++r)
-        if ((bj >> 6) == r) x[r] = -2.0f;                 // taken
+        if (r == br) x[r] = -2.0f;                        // taken
+      rescan();
     }
-    if (lane == 0) {
-      idx[row * k + s] = bj;
-      vals[row * k + s] = bv;
-      fmask[row * k + s] = bv > 1e-10f ? 1 : 0;
-    }
+  }
+  if (lane < k) {
+    idx[row * k + lane] = res_j;
+    vals[row * k + lane] = res_v;
+    fmask[row * k + lane] = res_v > 1e-10f ? 1 : 0;
   }
 }
 
@@ -71,11 +116,12 @@ extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k
                         int32_t* idx, float* vals, uint8_t* fmask, void* stream) {
   using namespace nsa;
   if (!scores || !idx || !vals || !fmask || rows <= 0 || nb <= 0 || k <= 0 || k > nb) return NSA_E_ARG;
-  if (nb > 64 * 32) return NSA_E_UNSUPPORTED;
+  if (nb > 64 * 32 || k > 64) return NSA_E_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   const int vpl = (nb + 63) / 64;
-#define NSA_TOPK(V) hipLaunchKernelGGL((topk_kernel<V>), grid, block, 0, st, scores, (long)rows, nb, k, apply_softmax, idx, vals, fmask)
+  const int vec4 = (nb % 4 == 0) && ((reinterpret_cast<uintptr_t>(scores) & 15) == 0);
+#define NSA_TOPK(V) hipLaunchKernelGGL((topk_kernel<V>), grid, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, idx, vals, fmask)
   if (vpl <= 1) NSA_TOPK(1);
   else if (vpl <= 2) NSA_TOPK(2);
   else if (vpl <= 4) NSA_TOPK(4);
