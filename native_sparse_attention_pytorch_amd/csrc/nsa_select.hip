@@ -725,7 +725,7 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 #define NSA_BWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1 stage 3.86 ms, 2: 3.44, 3: 3.53, 4: 3.60
 #endif
 template <int D, int KT, bool FUSE_DQ>
-__global__ __launch_bounds__(64 * KT) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+__global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1))) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                               const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
                                                               const float* __restrict__ lse, const float* __restrict__ delta,
                                                               const char* __restrict__ iws, char* __restrict__ bws) {
