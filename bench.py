@@ -215,6 +215,55 @@ def main():
     except Exception as ex:  # the headline must still be printed
         res["compressed_branch"] = dict(error=repr(ex))
 
+    # the callers either side of the path, reported beside the headline: the whole SparseAttention
+    # module (BASELINE configs[2]: b4 n4096 dim1024, forward + backward) and one decode step of a
+    # configs[3]-sized layer over a 32k-token cache
+    try:
+        from native_sparse_attention_pytorch_amd import SparseAttention
+        torch.manual_seed(0)
+        mod = SparseAttention(dim=1024, dim_head=64, heads=16, kv_heads=4, sliding_window_size=512, compress_block_size=32,
+                              compress_block_sliding_stride=16, selection_block_size=64, num_selected_blocks=16, causal=True).to(dev).bfloat16()
+        xm = torch.randn(4, 4096, 1024, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        dom = torch.randn_like(xm)
+        for _ in range(2):
+            mod(xm).backward(dom)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            mod(xm).backward(dom)
+        torch.cuda.synchronize()
+        tm = (time.perf_counter() - t0) / 5
+        res["module_config3"] = dict(ms_per_step=round(tm * 1e3, 3), tokens_per_s=round(4 * 4096 / tm, 1))
+        del mod, xm, dom
+    except Exception as ex:
+        res["module_config3"] = dict(error=repr(ex))
+    try:
+        from native_sparse_attention_pytorch_amd import SparseAttention
+        torch.manual_seed(0)
+        bd, ctx = 32, 32768
+        mod = SparseAttention(dim=hq * d, dim_head=d, heads=hq, kv_heads=hk, sliding_window_size=512, compress_block_size=32,
+                              compress_block_sliding_stride=16, selection_block_size=B, num_selected_blocks=S + 1, causal=True).to(dev).bfloat16()
+        def filled(rows, cap):          # a cache tensor as the module hands it back: prefix of a buffer with spare rows
+            buf = torch.randn(bd, hk, cap, d, device=dev, dtype=torch.bfloat16)
+            buf._nsa_filled = rows
+            return buf[:, :, :rows]
+        cache = ((filled(ctx, ctx + 256), filled(ctx, ctx + 256)),
+                 ((filled(ctx // 16, ctx // 16 + 64), filled(ctx // 16, ctx // 16 + 64)),
+                  (torch.zeros(bd, hk, 16, d, device=dev, dtype=torch.bfloat16), torch.zeros(bd, hk, 16, d, device=dev, dtype=torch.bfloat16))))
+        xt = torch.randn(bd, 1, hq * d, device=dev, dtype=torch.bfloat16)
+        for _ in range(40):             # includes the first compression step (one-time library initialisation)
+            _, cache = mod(xt, cache=cache, return_cache=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(100):
+            _, cache = mod(xt, cache=cache, return_cache=True)
+        torch.cuda.synchronize()
+        td = (time.perf_counter() - t0) / 100
+        res["decode_layer_32k"] = dict(batch=bd, us_per_step=round(td * 1e6, 1), tokens_per_s=round(bd / td, 1))
+        del mod, cache
+    except Exception as ex:
+        res["decode_layer_32k"] = dict(error=repr(ex))
+
     if not args.no_cpu:
         torch.set_num_threads(min(16, os.cpu_count() or 1))
         base, ref = cpu_baseline(cfg, q, k, v, do, idx, msk)
