@@ -147,6 +147,18 @@ int nsa_gate_bwd(int32_t batch, int32_t heads, int32_t seq, int32_t dim_head, co
 int nsa_rope(const void* x, const int64_t* x_stride, int32_t batch, int32_t heads, int32_t seq, int32_t dim_head,
              const float* freqs, int32_t offset, int32_t inverse, void* out, const int64_t* out_stride, void* stream);
 
+/* Compression windows.  Replaces split_compress_window (pad + unfold, NSA.py:270-275) and the
+ * intra-window position add (NSA.py:600-603).  x: bf16 [batch, heads, seq, d] with element strides
+ * {batch, head, token}; pos: bf16 [heads, block, d] or NULL; out: bf16 [batch, heads, seq / stride,
+ * block, d] contiguous, window w = tokens (w+1)*stride - block .. (w+1)*stride - 1 (zeros left of token
+ * 0) + pos.  nsa_windows_bwd: d_windows (same layout as out) -> dx bf16 [batch, heads, seq, d]
+ * contiguous (overlap-add in gather form; the gradient of pos is the sum of d_windows over batch and
+ * windows, left to the caller). */
+int nsa_windows_fwd(const void* x, const int64_t* x_stride, const void* pos, int32_t batch, int32_t heads, int32_t seq,
+                    int32_t dim_head, int32_t block, int32_t stride, void* out, void* stream);
+int nsa_windows_bwd(const void* d_windows, int32_t batch, int32_t heads, int32_t seq, int32_t dim_head, int32_t block,
+                    int32_t stride, void* dx, void* stream);
+
 /* Single-token decode attention over cached keys / values.  Replaces the three attention
  * computations of SparseAttention.forward_inference (NSA.py:396-420 compressed, :446-515 selected
  * blocks + own block, :519-530 sliding window).

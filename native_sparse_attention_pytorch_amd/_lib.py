@@ -80,6 +80,9 @@ def lib():
         i2 = C.POINTER(C.c_int64)
         L.nsa_decode_prep.argtypes = [vp, i2, vp, i2, vp, i2, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, C.c_int32, vp, vp, i2, vp, i2, vp]
         L.nsa_decode_combine.restype = L.nsa_decode_prep.restype = C.c_int
+        L.nsa_windows_fwd.argtypes = [vp, i3, vp] + [C.c_int32] * 6 + [vp, vp]
+        L.nsa_windows_bwd.argtypes = [vp] + [C.c_int32] * 6 + [vp, vp]
+        L.nsa_windows_fwd.restype = L.nsa_windows_bwd.restype = C.c_int
         for name in ("nsa_dense_workspace_bytes", "nsa_dense_fwd", "nsa_dense_bwd", "nsa_topk", "nsa_gate_fwd", "nsa_gate_bwd"):
             getattr(L, name).restype = C.c_int
         for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):

@@ -614,3 +614,68 @@ def decode_prep(q: Tensor, k: Tensor, v: Tensor, freqs: Tensor, pos: int, k_row:
     _lib.check(_lib.lib().nsa_decode_prep(_ptr(q), s2(q), _ptr(k), s2(k), _ptr(v), s2(v), b, hq, hk, d, _ptr(freqs), int(pos), _ptr(rq),
                                           _ptr(k_row), s2(k_row), _ptr(v_row), s2(v_row), _stream()), "nsa_decode_prep")
     return rq
+
+
+# ---------------------------------------------------------------------- compression windows
+
+@torch.library.custom_op("nsa_amd::windows_fwd", mutates_args=())
+def windows_fwd(x: Tensor, pos: Optional[Tensor], block: int, stride: int) -> Tensor:
+    x = _prep(x)
+    b, h, n, d = x.shape
+    w = n // stride
+    out = torch.empty((b, h, w, block, d), dtype=_BF16, device=x.device)
+    if pos is not None:
+        pos = pos.to(_BF16).contiguous()
+        if pos.shape != (h, block, d):
+            raise RuntimeError("window positions must be 'h block d'")
+    if w > 0:
+        _lib.check(_lib.lib().nsa_windows_fwd(_ptr(x), _s3(x), _ptr(pos), b, h, n, d, int(block), int(stride), _ptr(out), _stream()), "nsa_windows_fwd")
+    return out
+
+
+@windows_fwd.register_fake
+def _(x, pos, block, stride):
+    b, h, n, d = x.shape
+    return x.new_empty((b, h, n // stride, block, d))
+
+
+@torch.library.custom_op("nsa_amd::windows_bwd", mutates_args=())
+def windows_bwd(dwin: Tensor, n: int, stride: int) -> Tensor:
+    dwin = dwin.contiguous()
+    if dwin.dtype != _BF16:
+        raise RuntimeError("window gradients must be bfloat16")
+    b, h, w, block, d = dwin.shape
+    dx = torch.empty((b, h, n, d), dtype=_BF16, device=dwin.device)
+    if w == 0:
+        return dx.zero_()
+    _lib.check(_lib.lib().nsa_windows_bwd(_ptr(dwin), b, h, n, d, block, int(stride), _ptr(dx), _stream()), "nsa_windows_bwd")
+    return dx
+
+
+@windows_bwd.register_fake
+def _(dwin, n, stride):
+    b, h, w, block, d = dwin.shape
+    return dwin.new_empty((b, h, n, d))
+
+
+def _windows_setup(ctx, inputs, output):
+    x, pos, block, stride = inputs
+    ctx.n, ctx.stride, ctx.has_pos = x.shape[2], stride, pos is not None
+    ctx.pos_dtype = pos.dtype if pos is not None else None
+
+
+def _windows_backward(ctx, dwin):
+    dwin = dwin if dwin.dtype == _BF16 else dwin.to(_BF16)
+    dx = windows_bwd(dwin, ctx.n, ctx.stride)
+    dpos = dwin.sum(dim=(0, 2), dtype=torch.float32).to(ctx.pos_dtype) if ctx.has_pos else None
+    return dx, dpos, None, None
+
+
+windows_fwd.register_autograd(_windows_backward, setup_context=_windows_setup)
+
+
+def compress_windows(x: Tensor, pos: Tensor | None, block: int, stride: int) -> Tensor:
+    """'b h n d' -> 'b h w block d' with w = n // stride: window w = tokens (w+1)*stride - block ..
+    (w+1)*stride - 1, zeros left of token 0, plus the intra-window positions 'h block d'
+    (NSA.py:270-275, 589-603)."""
+    return windows_fwd(x, pos, int(block), int(stride))

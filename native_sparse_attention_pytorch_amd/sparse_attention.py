@@ -159,15 +159,6 @@ class SparseAttention(nn.Module):
         b, n, hd = t.shape
         return t.view(b, n, hd // self.dim_head, self.dim_head).permute(0, 2, 1, 3)
 
-    def _compress_windows(self, t):
-        """'b h n d' (n divisible by the stride) -> 'b h w cbs d'; window w = tokens
-        [(w+1)*stride - cbs, (w+1)*stride), zeros left of token 0 (NSA.py:270-275)."""
-        cbs, st = self.compress_block_size, self.compress_block_sliding_stride
-        b, h, L, d = t.shape
-        if L == 0:
-            return t.reshape(b, h, 0, cbs, d)
-        return F.pad(t, (0, 0, cbs - st, 0)).unfold(2, cbs, st).permute(0, 1, 2, 4, 3)
-
     @torch.no_grad()
     def forward_inference(self, inp, cache, return_cache=True):
         """One decode step (NSA.py:338-547): `inp` 'b 1 dim' is the token at position t = cached
@@ -263,10 +254,9 @@ class SparseAttention(nn.Module):
 
         # compressed keys / values from the un-rotated k, v
         L = (n // st) * st
-        kw, vw = self._compress_windows(k[..., :L, :]), self._compress_windows(v[..., :L, :])
-        if kw.numel() > 0:
-            kw = kw + self.k_intrablock_positions[None, :, None]
-            vw = vw + self.v_intrablock_positions[None, :, None]
+        # window gather + intra-window positions in one HIP kernel per tensor (NSA.py:589-603)
+        kw = ops.compress_windows(k.to(bf16), self.k_intrablock_positions, cbs, st).to(k.dtype)
+        vw = ops.compress_windows(v.to(bf16), self.v_intrablock_positions, cbs, st).to(v.dtype)
         ck0, cv0 = self.k_compress(kw), self.v_compress(vw)
         mem_k, mem_v = self.compress_mem_kv[0].to(ck0.dtype), self.compress_mem_kv[1].to(cv0.dtype)
         ck = torch.cat((mem_k[None].expand(b, -1, -1, -1), ck0), dim=-2)

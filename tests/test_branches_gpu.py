@@ -197,3 +197,32 @@ def test_rotary_matches_oracle(b, h, n, d, offset, view):
     assert out.is_contiguous()
     assert_close(out, ref, 1.6e-2 * ref.abs().max().item(), 1e-2, "rotary out")
     _grad_close(xg.grad, xr.grad, "rotary dx")
+
+
+@pytest.mark.parametrize("b,h,n,d,cbs,st", [(2, 2, 100, 64, 16, 8), (1, 4, 333, 128, 32, 16), (2, 3, 64, 64, 8, 8), (1, 2, 50, 64, 24, 4), (1, 1, 5, 64, 8, 8)])
+def test_compress_windows_match_oracle(b, h, n, d, cbs, st):
+    """Window gather + position add against the oracle's pad/unfold restatement (itself pinned by a
+    brute-force loop), forward and backward (overlap-add), on the strided view the projection gives."""
+    from native_sparse_attention_pytorch_amd.ops import compress_windows
+    g = torch.Generator().manual_seed(n + cbs)
+    base = _rand((b, n, h * d), g)
+    x = base.view(b, n, h, d).permute(0, 2, 1, 3)
+    pos = _rand((h, cbs, d), g, 0.3)
+    L = (n // st) * st
+    xr, pr = x.float().requires_grad_(), pos.float().requires_grad_()
+    want = O.compress_windows(xr[..., :L, :], cbs, st)
+    if want.numel() > 0:
+        want = want + pr[None, :, None]
+    xg, pg = x.to(DEV).requires_grad_(), pos.to(DEV).requires_grad_()
+    got = compress_windows(xg, pg, cbs, st)
+    torch.cuda.synchronize()
+    assert got.shape == want.shape
+    if want.numel() == 0:
+        return
+    do = _rand(tuple(want.shape), g)
+    (want * do.float()).sum().backward()
+    (got.float() * do.to(DEV).float()).sum().backward()
+    torch.cuda.synchronize()
+    assert_close(got, want, 1.6e-2 * want.abs().max().item(), 1e-2, "windows")
+    _grad_close(xg.grad, xr.grad, "d tokens")
+    _grad_close(pg.grad, pr.grad, "d positions")
