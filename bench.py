@@ -31,8 +31,8 @@ CFG = dict(batch=1, seq=32768, heads=32, kv_heads=8, dim_head=128, block=64, num
 
 # HBM bytes per launch on this workload, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
 # scaled by streaming kernels of known size (profiles/select_fwd_bwd_seq32k_hbm_traffic.txt)
-MEASURED_TRAFFIC_BYTES = {"fwd_block_walk": 7.383e9, "fwd_merge": 4.627e9, "bwd_dq_merge": 4.546e9,
-                          "bwd_dkv_walk": 13.688e9, "bwd_dkv_reduce": 0.547e9, "bwd_delta": 0.541e9}
+MEASURED_TRAFFIC_BYTES = {"fwd_block_walk": 7.389e9, "fwd_merge": 4.627e9, "bwd_dq_merge": 4.546e9,
+                          "bwd_dkv_walk": 13.697e9, "bwd_dkv_reduce": 0.547e9, "bwd_delta": 0.541e9}
 
 
 def selection(b, h, n, B, S, seed, device):
@@ -97,12 +97,17 @@ def cpu_baseline(cfg, q, k, v, do, idx, msk, nq=8192):
                        f"host has {os.cpu_count()} logical CPUs"), out.detach()
 
 
+class _Skip(Exception):
+    """Raised inside an optional leg that --headline-only turns off."""
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--headline-only", action="store_true", help="only the headline workload (for profiler runs): no compressed-branch, module or decode legs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
@@ -191,6 +196,8 @@ def main():
     # the other half of BASELINE configs[3]: compressed attention with fused importance logits +
     # top-k over 2048 compressed keys (+1 memory slot), forward and backward, reported beside the headline
     try:
+        if args.headline_only:
+            raise _Skip()
         g2 = torch.Generator(device=dev).manual_seed(1)
         nc = n // 16
         ck = (torch.randn(b, hk, nc + 1, d, generator=g2, device=dev) * d ** -0.5).to(torch.bfloat16).requires_grad_()
@@ -212,6 +219,8 @@ def main():
         best = min(tms[1:], key=sum)
         res["compressed_branch"] = dict(fwd_with_importance_ms=round(best[0], 4), topk_ms=round(best[1], 4), bwd_ms=round(best[2], 4),
                                         attended_pairs=p_cmp, fwd_bwd_tflops=round(14 * d * p_cmp / (sum(best) * 1e-3) / 1e12, 2))
+    except _Skip:
+        pass
     except Exception as ex:  # the headline must still be printed
         res["compressed_branch"] = dict(error=repr(ex))
 
@@ -219,6 +228,8 @@ def main():
     # module (BASELINE configs[2]: b4 n4096 dim1024, forward + backward) and one decode step of a
     # configs[3]-sized layer over a 32k-token cache
     try:
+        if args.headline_only:
+            raise _Skip()
         from native_sparse_attention_pytorch_amd import SparseAttention
         torch.manual_seed(0)
         mod = SparseAttention(dim=1024, dim_head=64, heads=16, kv_heads=4, sliding_window_size=512, compress_block_size=32,
@@ -235,9 +246,13 @@ def main():
         tm = (time.perf_counter() - t0) / 5
         res["module_config3"] = dict(ms_per_step=round(tm * 1e3, 3), tokens_per_s=round(4 * 4096 / tm, 1))
         del mod, xm, dom
+    except _Skip:
+        pass
     except Exception as ex:
         res["module_config3"] = dict(error=repr(ex))
     try:
+        if args.headline_only:
+            raise _Skip()
         from native_sparse_attention_pytorch_amd import SparseAttention
         torch.manual_seed(0)
         bd, ctx = 32, 32768
@@ -261,6 +276,8 @@ def main():
         td = (time.perf_counter() - t0) / 100
         res["decode_layer_32k"] = dict(batch=bd, us_per_step=round(td * 1e6, 1), tokens_per_s=round(bd / td, 1))
         del mod, cache
+    except _Skip:
+        pass
     except Exception as ex:
         res["decode_layer_32k"] = dict(error=repr(ex))
 
