@@ -155,7 +155,7 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     q_heads, kv_heads, sel_heads = fq.shape[1], fk.shape[1], selected_block_indices.shape[1]
     assert q_heads % kv_heads == 0
     assert sel_heads in (q_heads, kv_heads)
-    assert block_size >= 16, 'fine selection block size must be 16 or greater for now'
+    assert block_size in (8, 16, 32, 64), 'the HIP kernels are compiled for selection blocks of 8, 16, 32 or 64 keys'
     if return_sliding_window_out:
         raise NotImplementedError("the fused sliding-window output is experimental in the reference "
                                   "(test_triton_nsa.py:144) and is served by sliding_attend here")

@@ -42,6 +42,8 @@ CASES = [
     (1, 4, 4, 300, 64, 32, 5),       # G=1, ragged
     (1, 16, 2, 1024, 64, 64, 16),    # G=8, config-2-like
     (1, 8, 2, 1000, 128, 32, 7),     # ragged, d=128, B=32
+    (2, 8, 4, 77, 64, 8, 3),         # 8-key blocks (below the reference Triton path's minimum), ragged
+    (1, 4, 1, 250, 128, 8, 6),       # 8-key blocks, G=4, d=128
 ]
 
 
