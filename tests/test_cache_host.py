@@ -1,0 +1,58 @@
+"""Host logic of the growing decode caches (no GPU): a cache tensor is the filled prefix of a
+buffer with spare rows; appending takes a spare row in place, and any tensor that is not the
+live prefix of such a buffer (a prefill cache, an older tuple at a branch point, a full buffer)
+is copied into a new buffer first, so tensors handed out earlier never change."""
+import torch
+
+from native_sparse_attention_pytorch_amd.sparse_attention import _append_rows
+
+
+def test_first_append_copies_then_appends_in_place():
+    t = torch.randn(2, 3, 5, 8).to(torch.bfloat16)              # e.g. the cache the parallel forward returned
+    grown, row = _append_rows(t)
+    assert grown.shape == (2, 3, 6, 8) and row.shape == (2, 3, 1, 8)
+    assert torch.equal(grown[:, :, :5], t) and grown._base is not None and grown._base.shape[2] >= 12
+    row.fill_(1.0)
+    base = grown._base
+    grown2, row2 = _append_rows(grown)
+    assert grown2._base is base, "second append must reuse the buffer"
+    assert grown2.data_ptr() == grown.data_ptr() and torch.equal(grown2[:, :, :6], grown)
+    assert row2.data_ptr() == base[:, :, 6:7].data_ptr()
+
+
+def test_branching_from_an_older_cache_copies():
+    t = torch.zeros(1, 1, 4, 8, dtype=torch.bfloat16)
+    a, ra = _append_rows(t)
+    ra.fill_(1.0)
+    b, rb = _append_rows(a)          # advances the shared buffer to 6 rows
+    rb.fill_(2.0)
+    c, rc = _append_rows(a)          # `a` is no longer the live prefix: must not overwrite b's row
+    rc.fill_(3.0)
+    assert c._base is not b._base
+    assert float(b[0, 0, 5, 0]) == 2.0 and float(c[0, 0, 5, 0]) == 3.0
+    assert torch.equal(c[:, :, :5], a) and torch.equal(b[:, :, :5], a)
+
+
+def test_growth_when_capacity_is_exhausted_and_dtype_policy():
+    t = torch.randn(1, 2, 3, 8)                                   # fp32 cache from an fp32 module: converted once
+    cur, _ = _append_rows(t, min_capacity=4)
+    assert cur.dtype == torch.bfloat16
+    bases = {id(cur._base)}
+    for _ in range(40):
+        cur, row = _append_rows(cur, min_capacity=4)
+        row.zero_()
+        bases.add(id(cur._base))
+    assert cur.shape[2] == 44
+    assert 2 <= len(bases) <= 6, "doubling growth: a handful of reallocations for 40 appends"
+    keep, _ = _append_rows(torch.randn(1, 2, 3, 8), dtype=torch.float32, min_capacity=16)
+    assert keep.dtype == torch.float32 and keep._base.shape[2] == 16
+
+
+def test_empty_cache_and_views_that_do_not_start_at_the_buffer():
+    e = torch.zeros(2, 2, 0, 8, dtype=torch.bfloat16)
+    g, row = _append_rows(e)
+    assert g.shape[2] == 1
+    g2, _ = _append_rows(g)
+    tail = g2[:, :, 1:]              # a suffix view (what the running window keeps after a compression step)
+    h, _ = _append_rows(tail)
+    assert h._base is not g2._base and h.shape[2] == 2
