@@ -60,20 +60,38 @@ __global__ __launch_bounds__(256) void sel_scan_kernel(const SelPlan P, char* iw
   int* cnt = reinterpret_cast<int*>(iws + P.off_cnt) + (size_t)bh * P.nch * P.W;
   for (int j = tid; j < P.W; j += 256) {
     int run = 0;
-    for (int c = 0; c < P.nch; ++c) {
-      const int t = cnt[(size_t)c * P.W + j];
-      cnt[(size_t)c * P.W + j] = run;
-      run += t;
+    // chunks in batches of 16 whose loads are independent (one memory round trip per batch, not per chunk)
+    for (int c0 = 0; c0 < P.nch; c0 += 16) {
+      int t[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) t[u] = (c0 + u < P.nch) ? cnt[(size_t)(c0 + u) * P.W + j] : 0;
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        if (c0 + u < P.nch) cnt[(size_t)(c0 + u) * P.W + j] = run;
+        run += t[u];
+      }
     }
     tot[j] = run;
   }
   __syncthreads();
+  // exclusive scan of tot[] over the blocks: per-thread serial over a contiguous slice, then the slice sums
+  __shared__ int slice[256];
+  const int per = (P.W + 255) / 256;
+  const int lo = min(P.W, tid * per), hi = min(P.W, lo + per);
+  int sum = 0;
+  for (int j = lo; j < hi; ++j) sum += tot[j];
+  slice[tid] = sum;
+  __syncthreads();
   if (tid == 0) {
-    int* blk = reinterpret_cast<int*>(iws + P.off_blk) + (size_t)bh * (P.W + 1);
     int acc = 0;
-    for (int j = 0; j < P.W; ++j) { blk[j] = acc; acc += tot[j]; }
-    blk[P.W] = acc;
+    for (int k = 0; k < 256; ++k) { const int v = slice[k]; slice[k] = acc; acc += v; }
   }
+  __syncthreads();
+  int* blk = reinterpret_cast<int*>(iws + P.off_blk) + (size_t)bh * (P.W + 1);
+  int acc = slice[tid];
+  for (int j = lo; j < hi; ++j) { blk[j] = acc; acc += tot[j]; }
+  if (hi == P.W && lo < hi) blk[P.W] = acc;
+  if (P.W == 0 && tid == 0) blk[0] = 0;
 }
 
 // pairs of cell (phase p, block j) of table t: own queries (if the block lies in the phase and
