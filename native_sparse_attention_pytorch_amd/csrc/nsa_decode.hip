@@ -198,26 +198,31 @@ __global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_
   }
 }
 
-// one work-group per query head, one thread per feature: streaming merge of the head's partials
+// Feature `f` of head (b, head) of one branch: log-sum-exp merge of the split-K partials.
+template <int D>
+__device__ __forceinline__ float merge_head_partials(const DecodePlan& P, const float* __restrict__ part, int b, int head, int f) {
+  const int u = (P.units == P.hk) ? head / P.g : head, gi = (P.units == P.hk) ? head % P.g : 0;
+  const float* base = part + (long)(b * P.units + u) * P.nparts * P.rec;
+  const int om = P.gc * D + gi, ol = om + P.gc;
+  float M = -INFINITY;
+  for (int p = 0; p < P.nparts; ++p) M = fmaxf(M, base[(long)p * P.rec + om]);
+  if (!(M > -INFINITY)) return 0.f;                    // no wave saw a key
+  float acc = 0.f, L = 0.f;
+  for (int p = 0; p < P.nparts; ++p) {
+    const float* rec = base + (long)p * P.rec;
+    const float w = fast_exp2(rec[om] - M);            // exp2(-inf) = 0 for waves that saw no key
+    L += w * rec[ol];
+    acc += w * rec[gi * D + f];
+  }
+  return L > 0.f ? acc / L : 0.f;
+}
+
+// one work-group per query head, one thread per feature
 template <int D>
 __global__ __launch_bounds__(D) void decode_merge_kernel(const DecodePlan P, const float* __restrict__ part, __bf16* __restrict__ out) {
   const int hq = P.hk * P.g;
   const int bh = blockIdx.x, b = bh / hq, head = bh % hq;
-  const int u = (P.units == P.hk) ? head / P.g : head, gi = (P.units == P.hk) ? head % P.g : 0;
-  const float* base = part + (long)(b * P.units + u) * P.nparts * P.rec;
-  float M = -INFINITY;
-  const int om = P.gc * D + gi, ol = om + P.gc;
-  for (int p = 0; p < P.nparts; ++p) M = fmaxf(M, base[(long)p * P.rec + om]);
-  float acc = 0.f, L = 0.f;
-  if (M > -INFINITY) {
-    for (int p = 0; p < P.nparts; ++p) {
-      const float* rec = base + (long)p * P.rec;
-      const float w = fast_exp2(rec[om] - M);          // exp2(-inf) = 0 for waves that saw no key
-      L += w * rec[ol];
-      acc += w * rec[gi * D + threadIdx.x];
-    }
-  }
-  out[(long)bh * D + threadIdx.x] = (__bf16)(L > 0.f ? acc / L : 0.f);
+  out[(long)bh * D + threadIdx.x] = (__bf16)merge_head_partials<D>(P, part, b, head, threadIdx.x);
 }
 
 // Merge of the three branches' partials, sigmoid strategy gate and head merge in one pass
@@ -236,23 +241,8 @@ __global__ __launch_bounds__(D) void decode_combine_kernel(const CombineArgs A, 
 #pragma unroll
   for (int s = 0; s < 3; ++s) {
     if (A.part[s] == nullptr) continue;
-    const DecodePlan& P = A.P[s];
-    const int u = (P.units == P.hk) ? head / P.g : head, gi = (P.units == P.hk) ? head % P.g : 0;
-    const float* base = A.part[s] + (long)(b * P.units + u) * P.nparts * P.rec;
-    const int om = P.gc * D + gi, ol = om + P.gc;
-    float M = -INFINITY;
-    for (int p = 0; p < P.nparts; ++p) M = fmaxf(M, base[(long)p * P.rec + om]);
-    float acc = 0.f, L = 0.f;
-    if (M > -INFINITY) {
-      for (int p = 0; p < P.nparts; ++p) {
-        const float* rec = base + (long)p * P.rec;
-        const float w = fast_exp2(rec[om] - M);
-        L += w * rec[ol];
-        acc += w * rec[gi * D + threadIdx.x];
-      }
-    }
     // branch outputs are rounded to bf16 as when each is merged on its own
-    const float o = (float)(__bf16)(L > 0.f ? acc / L : 0.f);
+    const float o = (float)(__bf16)merge_head_partials<D>(A.P[s], A.part[s], b, head, threadIdx.x);
     const float gl = (float)gate_logits[((long)b * hq + head) * 3 + s];
     res += o / (1.f + __expf(-gl));
   }
