@@ -5,7 +5,7 @@ native_sparse_attention_pytorch/compress_networks.py:19-241, so that checkpoints
 
 All of them are dense projections: they run as (batched) hipBLASLt GEMMs.  The per-head
 networks (compress_networks.py:73-138) are written as one batched GEMM over the head axis
-(`torch.baddbmm` on 'h (b w) i' x 'h i o') instead of a general einsum, which keeps a single
+(`torch.bmm` on 'h (b w) i' x 'h i o') instead of a general einsum, which keeps a single
 strided-batched launch per layer whatever the head count.
 """
 from __future__ import annotations
@@ -29,10 +29,9 @@ class HeadwiseLinear(nn.Module):
     def forward(self, x):                                   # 'b h w i -> b h w o'
         b, h, w, i = x.shape
         xh = x.permute(1, 0, 2, 3).reshape(h, b * w, i)
+        y = torch.bmm(xh, self.weight.to(xh.dtype))
         if self.bias is not None:
-            y = torch.baddbmm(self.bias[0].to(xh.dtype), xh, self.weight.to(xh.dtype))
-        else:
-            y = torch.bmm(xh, self.weight.to(xh.dtype))
+            y = y + self.bias[0].to(xh.dtype)
         return y.reshape(h, b, w, self.weight.shape[-1]).permute(1, 0, 2, 3)
 
 
