@@ -68,13 +68,19 @@ __device__ __forceinline__ void make_ident(int lane, bf16x8& lo, bf16x8& hi) {
 
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short shortx4;
 
-// Transposed MFMA operand from a row-major bf16 tile X in LDS (row stride RS elements, RS*2
-// bytes = 32 mod 128 keeps the reads conflict-free): returns, for lane (m = lane % 32,
+// Transposed MFMA operand from a row-major bf16 tile X in LDS (row stride RS elements): returns, for lane (m = lane % 32,
 // h = lane / 32), the 8 values X[row0 + 8*(e/4) + 4h + e%4][col0 + m], e = 0..7 - i.e. an
 // A/B operand whose lane index runs over 32 columns of X and whose k index runs over 16 rows
 // of X in the same order in which a 32x32 MFMA result holds its rows (registers 8u .. 8u+7).
 // Uses the gfx950 LDS transpose load: in every group of 16 lanes, lane ll receives element
 // ll % 4 of the four 8-byte rows addressed by lanes 4e + ll / 4 (e = 0..3) of its group.
+// Bank conflicts (32 banks of 4 bytes; a 16-lane group reads 4 consecutive rows x 32 bytes): free
+// when the row stride is 8 banks mod 32 (RS*2 bytes = 32 mod 128, i.e. RS = D + 16), two-way at
+// RS = D + 8.  The 16-byte row reads of lds_row_operand are served 8 rows per clock and want 4
+// banks per row instead (RS = D + 8); a tile read both ways cannot have both with a plain stride,
+// and an XOR swizzle that gives both was measured slower in the backward kernels (its chunk index
+// no longer folds into the instructions' immediate offsets: more address registers in kernels that
+// have none to spare).
 __device__ __forceinline__ bf16x8 lds_transposed_operand(const __bf16* X, int RS, int row0, int col0, int lane) {
   const int ll = lane & 15, e = ll >> 2, qq = ll & 3, mh = (lane >> 4) & 1, h = lane >> 5;
   const __bf16* p0 = X + (row0 + 4 * h + e) * RS + col0 + 16 * mh + 4 * qq;

@@ -85,9 +85,9 @@ __global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_
                                                                           const __bf16* __restrict__ mem_k, const __bf16* __restrict__ mem_v,
                                                                           const void* __restrict__ idx, const unsigned char* __restrict__ fmask,
                                                                           float* __restrict__ part, float* __restrict__ logits) {
-  constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
+  constexpr int KS = D / 16, DT = D / 32, RS = D + 8, RSV = D + 16;   // row reads want 4 banks per row, transpose loads 8
   constexpr int LPR = D / 8, RPI = 64 / LPR, NI = 32 / RPI;      // lanes per row, rows per load instruction, instructions per tile
-  __shared__ __align__(16) __bf16 kv_s[kDecodeWaves][2][32 * RS];
+  __shared__ __align__(16) __bf16 kv_s[kDecodeWaves][2][32 * RSV];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_ = lane & 31, h = lane >> 5;
   const int lr = lane / LPR, lc = lane % LPR;
   __bf16* k_s = kv_s[wave][0];
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_
 #pragma unroll
     for (int r = 0; r < NI; ++r) {
       *reinterpret_cast<bf16x8*>(k_s + (RPI * r + lr) * RS + 8 * lc) = kr[r];
-      *reinterpret_cast<bf16x8*>(v_s + (RPI * r + lr) * RS + 8 * lc) = vr[r];
+      *reinterpret_cast<bf16x8*>(v_s + (RPI * r + lr) * RSV + 8 * lc) = vr[r];
     }
     const int tn = next_tile(t + nw, Tn);
     if (tn < P.tiles) issue(Tn);
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_
       for (int i = 0; i < 16; ++i) Oa[dt][i] *= alpha;
 #pragma unroll
       for (int u2 = 0; u2 < 2; ++u2)
-        Oa[dt] = mfma32(lds_transposed_operand(v_s, RS, 16 * u2, 32 * dt, lane), pack8(Sa, 8 * u2), Oa[dt]);
+        Oa[dt] = mfma32(lds_transposed_operand(v_s, RSV, 16 * u2, 32 * dt, lane), pack8(Sa, 8 * u2), Oa[dt]);
     }
     t = tn;
     T = Tn;

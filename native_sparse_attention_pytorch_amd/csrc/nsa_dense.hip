@@ -80,8 +80,9 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
                                                         const __bf16* __restrict__ v, __bf16* __restrict__ out, float* __restrict__ lse,
                                                         float* __restrict__ pooled) {
   constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
+  constexpr int RSV = D + 16;       // V is only read through the transpose load: 8 banks per row keep it conflict-free
   __shared__ __align__(16) __bf16 k_s[kBK * RS];
-  __shared__ __align__(16) __bf16 v_s[kBK * RS];
+  __shared__ __align__(16) __bf16 v_s[kBK * RSV];
   constexpr bool POOL = NPF > 0;
   constexpr int NBT = POOL ? kBK / (POOL ? NPF : 1) : 1;        // fine blocks per key tile
   __shared__ float pool_s[POOL ? 4 * 32 * NBT : 1];   // per wave: [rows or queries of the tile][fine blocks of the key tile]
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
 
   for (; t <= walk.t_hi; t = walk.next(t)) {
     kr.commit(k_s, RS, tid);
-    vr.commit(v_s, RS, tid);
+    vr.commit(v_s, RSV, tid);
     __syncthreads();
     const int tn = walk.next(t);
     if (tn <= walk.t_hi) load_tile(tn);
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
           const bf16x8 Pf = pack8(Sa[kt], 8 * u2);
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt)
-            Oa[dt] = mfma32(lds_transposed_operand(v_s, RS, 32 * kt + 16 * u2, 32 * dt, lane), Pf, Oa[dt]);
+            Oa[dt] = mfma32(lds_transposed_operand(v_s, RSV, 32 * kt + 16 * u2, 32 * dt, lane), Pf, Oa[dt]);
         }
     }
     __syncthreads();

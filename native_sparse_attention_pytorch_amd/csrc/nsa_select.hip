@@ -748,14 +748,15 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
                                                               const float* __restrict__ lse, const float* __restrict__ delta,
                                                               const char* __restrict__ iws, char* __restrict__ bws) {
   constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
-  constexpr int RST = 32 + 8;                  // row stride of the [key][row] dS tile
+  constexpr int RST = 32 + 16;                 // row stride of the [key][row] dS tile (transpose loads only: 8 banks mod 32 per row)
+  constexpr int RSK = D + 16;                  // row stride of the K block copy (transpose loads only)
   constexpr int DTW = DT / KT;                 // feature tiles of dQ per wave
   __shared__ __align__(16) float lse_s[32];
   __shared__ __align__(16) float del_s[32];
   __shared__ __align__(16) int lim_s[32];
   __shared__ __align__(16) __bf16 xq_s[32 * RS];
   __shared__ __align__(16) __bf16 xg_s[32 * RS];
-  __shared__ __align__(16) __bf16 kb_s[FUSE_DQ ? 32 * KT * RS : 8];     // the K block, row-major
+  __shared__ __align__(16) __bf16 kb_s[FUSE_DQ ? 32 * KT * RSK : 8];    // the K block, row-major
   __shared__ __align__(16) __bf16 ds_s[FUSE_DQ ? 32 * KT * RST : 8];    // dS^T: [key][row]
   __shared__ __align__(16) __bf16 dq_s[FUSE_DQ ? 32 * RS : 8];          // finished dQ tile, row-major
   __shared__ size_t row_s[32];
@@ -783,7 +784,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
     }
     if (FUSE_DQ) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<bf16x8*>(kb_s + kl * RS + 16 * ks + 8 * h) = Kf[ks];
+      for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<bf16x8*>(kb_s + kl * RSK + 16 * ks + 8 * h) = Kf[ks];
     }
   }
   floatx16 dKa[DT], dVa[DT];
@@ -896,7 +897,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
         const bf16x8 Sf = lds_transposed_operand(ds_s, RST, k0, 0, lane);          // lane <-> row, k <-> keys k0 ..
 #pragma unroll
         for (int w = 0; w < DTW; ++w)
-          Qa[w] = mfma32(lds_transposed_operand(kb_s, RS, k0, 32 * (DTW * kt + w), lane), Sf, Qa[w]);
+          Qa[w] = mfma32(lds_transposed_operand(kb_s, RSK, k0, 32 * (DTW * kt + w), lane), Sf, Qa[w]);
       }
       // Qa[w][4a + bb] = dQ[row n_][feature 32(DTW kt + w) + 8a + 4h + bb]
 #pragma unroll
