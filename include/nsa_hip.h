@@ -187,6 +187,15 @@ int nsa_decode_attend(const nsa_decode_desc* desc, const void* q, const void* k,
                       const void* mem_v, const void* idx, const uint8_t* fmask, void* ws, size_t ws_bytes, void* out,
                       float* logits, void* stream);
 
+/* Decode step: block selection from the compressed branch's logits.  Replaces the reduce over the
+ * compressed keys of a block and over the heads of a group, the padded softmax, topk and the mask of
+ * NSA.py:448-476, 502.  logits: fp32 [batch, heads, num_compressed] as written by nsa_decode_attend;
+ * the first (num_compressed / per_block) * per_block columns are used.  share != 0: one selection per
+ * kv head (mean over its group heads), rows = batch * kv_heads; otherwise per head, rows = batch * heads.
+ * Outputs [rows, k] as for nsa_topk. */
+int nsa_decode_topk(const float* logits, int32_t batch, int32_t kv_heads, int32_t group, int32_t num_compressed,
+                    int32_t per_block, int32_t share, int32_t k, int32_t* idx, float* vals, uint8_t* fmask, void* stream);
+
 /* Decode step, after three nsa_decode_attend calls with out == NULL (their partials left in the
  * three workspaces): merges each branch, applies the sigmoid strategy gate and writes the merged
  * heads.  Replaces to_strategy_combine's sigmoid + rearrange, the stack / einsum and merge_heads of

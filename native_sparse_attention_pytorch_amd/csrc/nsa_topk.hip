@@ -31,8 +31,12 @@ __device__ __forceinline__ float wave_max(float v) {
 // lowest lane holds the lowest index, and inside a lane the scan keeps the lower one: ties go to the
 // lower block index), and a re-scan in the winning lane.  Result s stays in lane s until the end,
 // so the outputs leave in one coalesced store each.
+// Pooling of raw decode logits in front of the top-k (NSA.py:448-476): row (b, u) of the top-k is the mean of
+// logits[b, u*pg + g, j*npf + c] over g < pg heads and c < npf compressed keys (row stride nc).
+struct PoolArgs { int pg, npf, nc, units; };
+
 template <int VPL>
-__global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in, long rows, int nb, int k, int softmax, int vec4,
+__global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in, long rows, int nb, int k, int softmax, int vec4, PoolArgs pool,
                                                    int* __restrict__ idx, float* __restrict__ vals, uint8_t* __restrict__ fmask) {
   const int lane = threadIdx.x & 63;
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -40,8 +44,26 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in,
   const float* src = in + row * nb;
   float x[VPL];
   bool loaded = false;
+  if (pool.pg > 0) {
+    const long b = row / pool.units, u = row % pool.units;
+    const float* base = in + (b * pool.units * pool.pg + u * pool.pg) * (long)pool.nc;
+    const float norm = 1.0f / (float)(pool.pg * pool.npf);
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+      const int j = lane * VPL + r;
+      float acc = -INFINITY;
+      if (j < nb) {
+        acc = 0.f;
+        for (int g = 0; g < pool.pg; ++g)
+          for (int c = 0; c < pool.npf; ++c) acc += base[(long)g * pool.nc + (long)j * pool.npf + c];
+        acc *= norm;
+      }
+      x[r] = acc;
+    }
+    loaded = true;
+  }
   if constexpr (VPL % 4 == 0) {
-    if (vec4) {                                          // rows are 16-byte aligned and nb % 4 == 0
+    if (vec4 && !loaded) {                               // rows are 16-byte aligned and nb % 4 == 0
 #pragma unroll
       for (int r4 = 0; r4 < VPL / 4; ++r4) {
         const int j = lane * VPL + 4 * r4;
@@ -121,13 +143,37 @@ extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   const int vpl = (nb + 63) / 64;
   const int vec4 = (nb % 4 == 0) && ((reinterpret_cast<uintptr_t>(scores) & 15) == 0);
-#define NSA_TOPK(V) hipLaunchKernelGGL((topk_kernel<V>), grid, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, idx, vals, fmask)
-  if (vpl <= 1) NSA_TOPK(1);
-  else if (vpl <= 2) NSA_TOPK(2);
-  else if (vpl <= 4) NSA_TOPK(4);
-  else if (vpl <= 8) NSA_TOPK(8);
-  else if (vpl <= 16) NSA_TOPK(16);
-  else NSA_TOPK(32);
+  const PoolArgs pool{0, 1, 0, 1};
+#define NSA_TOPK(V) hipLaunchKernelGGL((topk_kernel<V>), grid, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, pool, idx, vals, fmask)
+#define NSA_TOPK_DISPATCH()            \
+  if (vpl <= 1) NSA_TOPK(1);           \
+  else if (vpl <= 2) NSA_TOPK(2);      \
+  else if (vpl <= 4) NSA_TOPK(4);      \
+  else if (vpl <= 8) NSA_TOPK(8);      \
+  else if (vpl <= 16) NSA_TOPK(16);    \
+  else NSA_TOPK(32)
+  NSA_TOPK_DISPATCH();
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
+
+extern "C" int nsa_decode_topk(const float* logits, int32_t batch, int32_t kv_heads, int32_t group, int32_t num_compressed,
+                               int32_t per_block, int32_t share, int32_t k, int32_t* idx, float* vals, uint8_t* fmask, void* stream) {
+  using namespace nsa;
+  if (!logits || !idx || !vals || !fmask || batch <= 0 || kv_heads <= 0 || group <= 0 || per_block <= 0 || num_compressed <= 0) return NSA_E_ARG;
+  const int nb = num_compressed / per_block;
+  if (k <= 0 || k > nb) return NSA_E_ARG;
+  if (nb > 64 * 32 || k > 64) return NSA_E_UNSUPPORTED;
+  const int units = share ? kv_heads : kv_heads * group;
+  const long rows = (long)batch * units;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  const int vpl = (nb + 63) / 64;
+  const int vec4 = 0, apply_softmax = 1;
+  const float* scores = logits;
+  const PoolArgs pool{share ? group : 1, per_block, num_compressed, units};
+  NSA_TOPK_DISPATCH();
+#undef NSA_TOPK_DISPATCH
 #undef NSA_TOPK
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;

@@ -679,3 +679,22 @@ def compress_windows(x: Tensor, pos: Tensor | None, block: int, stride: int) -> 
     (w+1)*stride - 1, zeros left of token 0, plus the intra-window positions 'h block d'
     (NSA.py:270-275, 589-603)."""
     return windows_fwd(x, pos, int(block), int(stride))
+
+
+@torch.no_grad()
+def decode_importance_topk(logits: Tensor, kv_heads: int, per_block: int, share: bool, num_selected: int):
+    """Decode step: logits 'b hq nc' (from decode_range_attend) -> pooled over the `per_block`
+    compressed keys of a selection block and, if `share`, over the heads of a kv group; padded
+    softmax, top-k, mask (NSA.py:448-476, 502).  Returns (values, indices, mask) shaped
+    'b hk 1 k' or 'b hq 1 k'."""
+    if logits.dtype != torch.float32 or not logits.is_cuda or not logits.is_contiguous():
+        raise RuntimeError("decode logits must be contiguous fp32 device tensors")
+    b, hq, nc = logits.shape
+    units = kv_heads if share else hq
+    shp = (b, units, 1, int(num_selected))
+    idx = torch.empty(shp, dtype=torch.int32, device=logits.device)
+    vals = torch.empty(shp, dtype=torch.float32, device=logits.device)
+    fm = torch.empty(shp, dtype=torch.uint8, device=logits.device)
+    _lib.check(_lib.lib().nsa_decode_topk(_ptr(logits), b, int(kv_heads), hq // kv_heads, nc, int(per_block), int(bool(share)),
+                                          int(num_selected), _ptr(idx), _ptr(vals), _ptr(fm), _stream()), "nsa_decode_topk")
+    return vals, idx, fm.view(torch.bool)

@@ -213,9 +213,8 @@ class SparseAttention(nn.Module):
         nb = nc // npf
         num_sel = min(self.num_selected_blocks, nb)
         if num_sel > 0:
-            imp = logits[..., :nb * npf].reshape(b, self.kv_heads, G, 1, nb, npf).mean(dim=-1)
-            imp = imp.mean(dim=2) if self.query_heads_share_selected_kv else imp.reshape(b, self.heads, 1, nb)
-            _, idx, fmask = ops.importance_topk(imp.contiguous(), num_sel)
+            # pooling over the block's compressed keys and the group's heads, padded softmax and top-k in one kernel
+            _, idx, fmask = ops.decode_importance_topk(logits, self.kv_heads, npf, self.query_heads_share_selected_kv, num_sel)
         else:
             idx = torch.zeros((b, self.kv_heads, 1, 0), dtype=torch.int32, device=inp.device)
             fmask = idx.bool()

@@ -192,21 +192,21 @@ def test_module_decode_matches_oracle_decode(ci, prefill):
         y, cache = mod(x[:, :prefill].to(DEV), return_cache=True)
         _, rcache = ref(x[:, :prefill].float(), return_cache=True)
     captured = {}
-    orig = ops.importance_topk
-    def spy(imp, k_):
-        r = orig(imp, k_)
+    orig = ops.decode_importance_topk
+    def spy(*a):
+        r = orig(*a)
         captured["sel"] = (r[1].cpu().long(), r[2].cpu())
         return r
     agree = total = 0
     worst = 0.0
     for i in range(prefill, n):
         captured.clear()
-        ops.importance_topk = spy
+        ops.decode_importance_topk = spy
         try:
             out, cache = mod(x[:, i:i + 1].to(DEV), cache=cache, return_cache=True)
             torch.cuda.synchronize()
         finally:
-            ops.importance_topk = orig
+            ops.decode_importance_topk = orig
         with torch.no_grad():
             own, _ = ref(x[:, i:i + 1].float(), cache=rcache, return_cache=True)           # the oracle's own selection
             want, rcache2 = ref(x[:, i:i + 1].float(), cache=rcache, return_cache=True, selection_override=captured.get("sel"))
@@ -282,3 +282,25 @@ def test_transformer_greedy_sampling_with_and_without_cache():
     c2 = model.sample(prompt, 64, temperature=0., use_cache_kv=True)
     assert a.shape == (1, 63) and torch.equal(c, c2)
     assert torch.equal(a[:, :8], c[:, :8]), (a, c)
+
+
+@pytest.mark.parametrize("b,hq,hk,nc,npf,share,k", [(2, 8, 2, 37, 4, True, 3), (1, 4, 4, 512, 1, True, 16), (3, 8, 2, 130, 2, False, 5), (1, 16, 1, 2048, 4, True, 16)])
+def test_decode_importance_topk_matches_oracle(b, hq, hk, nc, npf, share, k):
+    """Fused pooling + padded softmax + top-k of the decode step against the oracle's functions on
+    the same logits: indices equal where the probabilities are distinct, values to 1e-5."""
+    from native_sparse_attention_pytorch_amd.ops import decode_importance_topk
+    g = torch.Generator().manual_seed(nc + k)
+    logits = torch.randn(b, hq, nc, generator=g) * 3
+    nb = nc // npf
+    pooled = logits[..., :nb * npf].reshape(b, hk, hq // hk, nb, npf).mean(dim=-1)
+    pooled = pooled.mean(dim=2, keepdim=True) if share else pooled.reshape(b, hq, 1, nb)
+    probs = O.importance_softmax(pooled)
+    want_v, want_i = O.topk_lower_index_first(probs, k)
+    vals, idx, fm = decode_importance_topk(logits.to(DEV), hk, npf, share, k)
+    torch.cuda.synchronize()
+    assert idx.shape == want_i.shape
+    assert_close(vals, want_v, 1e-5, 1e-4, "selected probabilities")
+    gap = (want_v[..., :-1] - want_v[..., 1:]).min().item()
+    if gap > 1e-6:
+        assert torch.equal(idx.cpu().long(), want_i)
+    assert torch.equal(fm.cpu(), want_v > 1e-10) or (want_v - 1e-10).abs().min() < 1e-12
