@@ -210,11 +210,14 @@ int nsa_decode_combine(const nsa_decode_desc* compressed, const void* ws_compres
  * position pos, writes the rotated keys into row pos of the key cache and the values into row pos
  * of the value cache.  Replaces rotate_queries_or_keys x2 and the two cache concatenations of
  * NSA.py:384-393.  q, k, v: bf16 [batch, heads|kv_heads, d] with element strides {batch, head};
- * k_row / v_row: address of row pos of head 0 of batch 0 in the caches, strides {batch, head}. */
+ * k_row / v_row: address of row pos of head 0 of batch 0 in the caches, strides {batch, head}.
+ * k_run_row / v_run_row (optional, both or neither): where the un-rotated key / value rows of the open
+ * compression window go (NSA.py:377-380), same addressing. */
 int nsa_decode_prep(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v,
                     const int64_t* v_stride, int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head,
                     const float* freqs, int32_t pos, void* rq, void* k_row, const int64_t* k_row_stride, void* v_row,
-                    const int64_t* v_row_stride, void* stream);
+                    const int64_t* v_row_stride, void* k_run_row, const int64_t* k_run_stride, void* v_run_row,
+                    const int64_t* v_run_stride, void* stream);
 
 /* Same as nsa_select_fwd / nsa_select_bwd, additionally recording the caller's hipEvent_t
  * handles (created with timing enabled) between the kernels of the call, so that a benchmark

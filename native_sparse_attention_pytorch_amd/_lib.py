@@ -78,7 +78,7 @@ def lib():
         dd = C.POINTER(DecodeDesc)
         L.nsa_decode_combine.argtypes = [dd, vp, dd, vp, dd, vp, vp, vp, vp]
         i2 = C.POINTER(C.c_int64)
-        L.nsa_decode_prep.argtypes = [vp, i2, vp, i2, vp, i2, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, C.c_int32, vp, vp, i2, vp, i2, vp]
+        L.nsa_decode_prep.argtypes = [vp, i2, vp, i2, vp, i2, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, C.c_int32, vp, vp, i2, vp, i2, vp, i2, vp, i2, vp]
         L.nsa_decode_combine.restype = L.nsa_decode_prep.restype = C.c_int
         L.nsa_decode_topk.argtypes = [vp] + [C.c_int32] * 7 + [vp, vp, vp, vp]
         L.nsa_decode_topk.restype = C.c_int

@@ -40,7 +40,8 @@ template <int D>
 __global__ __launch_bounds__(256) void decode_prep_kernel(const __bf16* __restrict__ q, long q0, long q1, const __bf16* __restrict__ k, long k0, long k1,
                                                           const __bf16* __restrict__ v, long v0, long v1, int b, int hq, int hk,
                                                           const float* __restrict__ freqs, int pos, __bf16* __restrict__ rq,
-                                                          __bf16* __restrict__ krow, long kr0, long kr1, __bf16* __restrict__ vrow, long vr0, long vr1) {
+                                                          __bf16* __restrict__ krow, long kr0, long kr1, __bf16* __restrict__ vrow, long vr0, long vr1,
+                                                          __bf16* __restrict__ krun, long ku0, long ku1, __bf16* __restrict__ vrun, long vu0, long vu1) {
   constexpr int LPR = D / 8, RPB = 256 / LPR;
   const int per = hq + 2 * hk;
   const long row = (long)blockIdx.x * RPB + threadIdx.x / LPR;
@@ -54,6 +55,11 @@ __global__ __launch_bounds__(256) void decode_prep_kernel(const __bf16* __restri
   else if (r < hq + hk) { src = k + bb * k0 + (r - hq) * k1; dst = krow + bb * kr0 + (r - hq) * kr1; }
   else { src = v + bb * v0 + (r - hq - hk) * v1; dst = vrow + bb * vr0 + (r - hq - hk) * vr1; rot = false; }
   const bf16x8 x = load8(src + 8 * c);
+  // the un-rotated key / value also go into the open compression window (NSA.py:377-380)
+  if (krun != nullptr && r >= hq) {
+    __bf16* run = r < hq + hk ? krun + bb * ku0 + (r - hq) * ku1 : vrun + bb * vu0 + (r - hq - hk) * vu1;
+    *reinterpret_cast<bf16x8*>(run + 8 * c) = x;
+  }
   bf16x8 o = x;
   if (rot) {
     const float p = (float)pos;
@@ -74,7 +80,8 @@ __global__ __launch_bounds__(256) void decode_prep_kernel(const __bf16* __restri
 extern "C" int nsa_decode_prep(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v,
                                const int64_t* v_stride, int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head,
                                const float* freqs, int32_t pos, void* rq, void* k_row, const int64_t* k_row_stride, void* v_row,
-                               const int64_t* v_row_stride, void* stream) {
+                               const int64_t* v_row_stride, void* k_run_row, const int64_t* k_run_stride, void* v_run_row,
+                               const int64_t* v_run_stride, void* stream) {
   using namespace nsa;
   if (!q || !k || !v || !q_stride || !k_stride || !v_stride || !freqs || !rq || !k_row || !v_row || !k_row_stride || !v_row_stride)
     return NSA_E_ARG;
@@ -82,18 +89,26 @@ extern "C" int nsa_decode_prep(const void* q, const int64_t* q_stride, const voi
   if ((q_stride[0] | q_stride[1] | k_stride[0] | k_stride[1] | v_stride[0] | v_stride[1] | k_row_stride[0] | k_row_stride[1] |
        v_row_stride[0] | v_row_stride[1]) & 7)
     return NSA_E_ARG;
+  long ku[2] = {0, 0}, vu[2] = {0, 0};
+  if (k_run_row || v_run_row) {
+    if (!k_run_row || !v_run_row || !k_run_stride || !v_run_stride) return NSA_E_ARG;
+    if ((k_run_stride[0] | k_run_stride[1] | v_run_stride[0] | v_run_stride[1]) & 7) return NSA_E_ARG;
+    ku[0] = k_run_stride[0]; ku[1] = k_run_stride[1]; vu[0] = v_run_stride[0]; vu[1] = v_run_stride[1];
+  }
   const long rows = (long)batch * (heads + 2 * kv_heads);
   hipStream_t st = (hipStream_t)stream;
   if (dim_head == 64) {
     hipLaunchKernelGGL((decode_prep_kernel<64>), dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, (const __bf16*)q, (long)q_stride[0],
                        (long)q_stride[1], (const __bf16*)k, (long)k_stride[0], (long)k_stride[1], (const __bf16*)v, (long)v_stride[0],
                        (long)v_stride[1], batch, heads, kv_heads, freqs, pos, (__bf16*)rq, (__bf16*)k_row, (long)k_row_stride[0],
-                       (long)k_row_stride[1], (__bf16*)v_row, (long)v_row_stride[0], (long)v_row_stride[1]);
+                       (long)k_row_stride[1], (__bf16*)v_row, (long)v_row_stride[0], (long)v_row_stride[1], (__bf16*)k_run_row, ku[0], ku[1],
+                       (__bf16*)v_run_row, vu[0], vu[1]);
   } else if (dim_head == 128) {
     hipLaunchKernelGGL((decode_prep_kernel<128>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const __bf16*)q, (long)q_stride[0],
                        (long)q_stride[1], (const __bf16*)k, (long)k_stride[0], (long)k_stride[1], (const __bf16*)v, (long)v_stride[0],
                        (long)v_stride[1], batch, heads, kv_heads, freqs, pos, (__bf16*)rq, (__bf16*)k_row, (long)k_row_stride[0],
-                       (long)k_row_stride[1], (__bf16*)v_row, (long)v_row_stride[0], (long)v_row_stride[1]);
+                       (long)k_row_stride[1], (__bf16*)v_row, (long)v_row_stride[0], (long)v_row_stride[1], (__bf16*)k_run_row, ku[0], ku[1],
+                       (__bf16*)v_run_row, vu[0], vu[1]);
   } else {
     return NSA_E_UNSUPPORTED;
   }

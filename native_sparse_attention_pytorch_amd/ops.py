@@ -596,23 +596,28 @@ def decode_combine(gate_logits: Tensor, compressed, selected, sliding) -> Tensor
 
 
 @torch.no_grad()
-def decode_prep(q: Tensor, k: Tensor, v: Tensor, freqs: Tensor, pos: int, k_row: Tensor, v_row: Tensor) -> Tensor:
+def decode_prep(q: Tensor, k: Tensor, v: Tensor, freqs: Tensor, pos: int, k_row: Tensor, v_row: Tensor,
+                k_run_row: Tensor | None = None, v_run_row: Tensor | None = None) -> Tensor:
     """New token's q 'b hq 1 d', k, v 'b hk 1 d' (bf16 views are fine): returns the rotated
     queries and writes the rotated keys / the values into the cache rows k_row, v_row 'b hk 1 d'
-    (NSA.py:384-393)."""
+    (NSA.py:384-393) and, when given, the un-rotated keys / values into k_run_row, v_run_row (the
+    open compression window, NSA.py:377-380)."""
     q, k, v = _prep(q), _prep(k), _prep(v)
     b, hq, _, d = q.shape
     hk = k.shape[1]
-    for t in (k_row, v_row):
-        if t.dtype != _BF16 or t.shape != (b, hk, 1, d) or not _rows_ok(t):
+    for t in (k_row, v_row, k_run_row, v_run_row):
+        if t is not None and (t.dtype != _BF16 or t.shape != (b, hk, 1, d) or not _rows_ok(t)):
             raise RuntimeError("decode_prep: cache rows must be bf16 'b hk 1 d' views with 16-byte aligned rows")
     freqs = freqs.detach()
     if freqs.dtype != torch.float32 or not freqs.is_contiguous():
         freqs = freqs.to(torch.float32).contiguous()
     rq = torch.empty((b, hq, 1, d), dtype=_BF16, device=q.device)
     s2 = lambda t: (C.c_int64 * 2)(t.stride(0), t.stride(1))
+    run = k_run_row is not None and v_run_row is not None
     _lib.check(_lib.lib().nsa_decode_prep(_ptr(q), s2(q), _ptr(k), s2(k), _ptr(v), s2(v), b, hq, hk, d, _ptr(freqs), int(pos), _ptr(rq),
-                                          _ptr(k_row), s2(k_row), _ptr(v_row), s2(v_row), _stream()), "nsa_decode_prep")
+                                          _ptr(k_row), s2(k_row), _ptr(v_row), s2(v_row),
+                                          _ptr(k_run_row) if run else None, s2(k_run_row) if run else None,
+                                          _ptr(v_run_row) if run else None, s2(v_run_row) if run else None, _stream()), "nsa_decode_prep")
     return rq
 
 

@@ -180,13 +180,16 @@ class SparseAttention(nn.Module):
         # raw tokens of the open compression window (not rotated, NSA.py:377-380)
         run_k, rk_row = _append_rows(run_k, dtype=run_k.dtype, min_capacity=cbs)
         run_v, rv_row = _append_rows(run_v, dtype=run_v.dtype, min_capacity=cbs)
-        rk_row.copy_(k)
-        rv_row.copy_(v)
+        fused_run = run_k.dtype == bf16 and run_v.dtype == bf16
+        if not fused_run:
+            rk_row.copy_(k)
+            rv_row.copy_(v)
 
-        # the rotated key and the value go into row t of the caches (NSA.py:384-393)
+        # the rotated key and the value go into row t of the caches (NSA.py:384-393); the same kernel
+        # rotates the queries and (bf16 windows) fills the rows of the open compression window
         keys, k_row = _append_rows(cache_k)
         vals, v_row = _append_rows(cache_v)
-        rq16 = ops.decode_prep(q16, k16, v16, freqs, t, k_row, v_row)
+        rq16 = ops.decode_prep(q16, k16, v16, freqs, t, k_row, v_row, rk_row if fused_run else None, rv_row if fused_run else None)
 
         # 1. compressed branch: every cached compressed key, no mask (NSA.py:396-420)
         nc = cache_ck.shape[-2]
