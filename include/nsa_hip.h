@@ -206,6 +206,31 @@ int nsa_decode_combine(const nsa_decode_desc* compressed, const void* ws_compres
                        const void* ws_selected, const nsa_decode_desc* sliding, const void* ws_sliding,
                        const void* gate_logits, void* out, void* stream);
 
+/* The attention part of one decode step (NSA.py:377-545 without the projections and the compression of
+ * a completed window) as one host call: nsa_decode_prep, the compressed branch, nsa_decode_topk, the
+ * selected-block branch, the sliding branch and nsa_decode_combine, with all intermediates in `ws`.
+ * pos = rows already in the key / value caches (the new token's position); the caches must have row
+ * pos free.  num_sel is the configured number of blocks; min(num_sel, num_compressed / per_block) are
+ * selected, their indices (int32) and mask (uint8), [batch, kv_heads or heads, k], are left in the
+ * workspace at the offsets nsa_decode_step_workspace_bytes reports.  q, k, v: the new token's
+ * projections, bf16 [batch, heads | kv_heads, d], element strides {batch, head}; gate_logits: bf16
+ * [batch, 3 * heads]; out: bf16 [batch, heads * d]. */
+typedef struct nsa_decode_step_desc {
+  int32_t batch, heads, kv_heads, dim_head;
+  int32_t pos, num_compressed, num_mem, per_block, block, num_sel, share, window;
+  float scale;
+  int64_t q_stride[2], k_stride[2], v_stride[2];
+  int64_t kc_stride[3], vc_stride[3];     /* key / value caches [batch, kv_heads, capacity, d] */
+  int64_t ck_stride[3], cv_stride[3];     /* compressed key / value caches */
+  int64_t krun_stride[2], vrun_stride[2]; /* rows of the open compression window (if passed) */
+} nsa_decode_step_desc;
+int nsa_decode_step_workspace_bytes(const nsa_decode_step_desc* desc, size_t* bytes, size_t* idx_offset, size_t* fmask_offset,
+                                    int32_t* num_selected);
+int nsa_decode_step(const nsa_decode_step_desc* desc, const void* q, const void* k, const void* v, const float* freqs,
+                    void* k_cache, void* v_cache, const void* ck_cache, const void* cv_cache, const void* mem_k,
+                    const void* mem_v, void* k_run_row, void* v_run_row, const void* gate_logits, void* ws, size_t ws_bytes,
+                    void* out, void* stream);
+
 /* Decode step: rotates the new token's queries (-> rq, bf16 [batch, heads, d] contiguous) and keys to
  * position pos, writes the rotated keys into row pos of the key cache and the values into row pos
  * of the value cache.  Replaces rotate_queries_or_keys x2 and the two cache concatenations of

@@ -41,6 +41,17 @@ class DecodeDesc(C.Structure):
     ]
 
 
+class DecodeStepDesc(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("heads", C.c_int32), ("kv_heads", C.c_int32), ("dim_head", C.c_int32),
+        ("pos", C.c_int32), ("num_compressed", C.c_int32), ("num_mem", C.c_int32), ("per_block", C.c_int32),
+        ("block", C.c_int32), ("num_sel", C.c_int32), ("share", C.c_int32), ("window", C.c_int32), ("scale", C.c_float),
+        ("q_stride", C.c_int64 * 2), ("k_stride", C.c_int64 * 2), ("v_stride", C.c_int64 * 2),
+        ("kc_stride", C.c_int64 * 3), ("vc_stride", C.c_int64 * 3), ("ck_stride", C.c_int64 * 3), ("cv_stride", C.c_int64 * 3),
+        ("krun_stride", C.c_int64 * 2), ("vrun_stride", C.c_int64 * 2),
+    ]
+
+
 _ERR = {-1: "invalid argument", -2: "shape not supported by the compiled kernels", -3: "workspace too small"}
 
 
@@ -82,6 +93,10 @@ def lib():
         L.nsa_decode_combine.restype = L.nsa_decode_prep.restype = C.c_int
         L.nsa_decode_topk.argtypes = [vp] + [C.c_int32] * 7 + [vp, vp, vp, vp]
         L.nsa_decode_topk.restype = C.c_int
+        ds = C.POINTER(DecodeStepDesc)
+        L.nsa_decode_step_workspace_bytes.argtypes = [ds, C.POINTER(sz), C.POINTER(sz), C.POINTER(sz), C.POINTER(C.c_int32)]
+        L.nsa_decode_step.argtypes = [ds] + [vp] * 14 + [sz, vp, vp]
+        L.nsa_decode_step_workspace_bytes.restype = L.nsa_decode_step.restype = C.c_int
         L.nsa_windows_fwd.argtypes = [vp, i3, vp] + [C.c_int32] * 6 + [vp, vp]
         L.nsa_windows_bwd.argtypes = [vp] + [C.c_int32] * 6 + [vp, vp]
         L.nsa_windows_fwd.restype = L.nsa_windows_bwd.restype = C.c_int

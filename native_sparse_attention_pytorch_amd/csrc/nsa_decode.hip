@@ -356,3 +356,123 @@ extern "C" int nsa_decode_combine(const nsa_decode_desc* compressed, const void*
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
 }
+
+// ---------------------------------------------------------------------------- whole step
+// The attention part of one decode step as a single host call: prep, compressed branch, block
+// selection, selected-block branch, sliding branch, merge + gate.  The launches are the same as
+// through the separate entry points; what goes away is the host-side work between them, which
+// at small batch is most of a step's time.
+
+namespace nsa {
+
+struct StepLayout {
+  nsa_decode_desc c, f, s;
+  int nb, k;                       // selection blocks available / selected this step
+  int sel_units;                   // rows of idx per batch element
+  size_t off_rq, off_wsc, off_wsf, off_wss, off_logits, off_idx, off_vals, off_fm, total;
+  size_t wsc, wsf, wss;
+};
+
+static size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static int make_step_layout(const nsa_decode_step_desc* d, StepLayout& L) {
+  if (!d) return NSA_E_ARG;
+  if (d->batch <= 0 || d->heads <= 0 || d->kv_heads <= 0 || d->heads % d->kv_heads) return NSA_E_ARG;
+  if (d->pos < 0 || d->num_compressed < 0 || d->num_mem < 0 || d->per_block <= 0 || d->block <= 0 || d->num_sel < 0 || d->window < 0)
+    return NSA_E_ARG;
+  const int g = d->heads / d->kv_heads, kv_len = d->pos + 1;
+  auto common = [&](nsa_decode_desc& x) {
+    x = nsa_decode_desc{};
+    x.batch = d->batch; x.kv_heads = d->kv_heads; x.group = g; x.dim_head = d->dim_head; x.scale = d->scale;
+  };
+  // compressed branch reads the un-rotated projection, the other two the rotated queries in the workspace
+  common(L.c);
+  L.c.mode = 0; L.c.start = 0; L.c.count = d->num_compressed; L.c.num_mem = d->num_compressed > 0 ? d->num_mem : 0;
+  L.c.q_stride[0] = d->q_stride[0]; L.c.q_stride[1] = d->q_stride[1];
+  for (int i = 0; i < 3; ++i) { L.c.k_stride[i] = d->ck_stride[i]; L.c.v_stride[i] = d->cv_stride[i]; }
+  L.nb = d->num_compressed / d->per_block;
+  L.k = d->num_sel < L.nb ? d->num_sel : L.nb;
+  L.sel_units = d->share ? d->kv_heads : d->heads;
+  common(L.f);
+  L.f.mode = 1; L.f.block = d->block; L.f.num_sel = L.k; L.f.kv_len = kv_len; L.f.per_head_sel = (!d->share && g > 1) ? 1 : 0;
+  L.f.idx_is_int64 = 0;
+  common(L.s);
+  L.s.mode = 0;
+  const int w = kv_len < d->window + 1 ? kv_len : d->window + 1;
+  L.s.start = kv_len - w; L.s.count = w; L.s.num_mem = 0;
+  for (nsa_decode_desc* x : {&L.f, &L.s}) {
+    x->q_stride[0] = (int64_t)d->heads * d->dim_head; x->q_stride[1] = d->dim_head;
+    for (int i = 0; i < 3; ++i) { x->k_stride[i] = d->kc_stride[i]; x->v_stride[i] = d->vc_stride[i]; }
+  }
+  if (d->num_compressed > 0)
+    if (int e = nsa_decode_workspace_bytes(&L.c, &L.wsc)) return e;
+  if (d->num_compressed <= 0) L.wsc = 0;
+  if (int e = nsa_decode_workspace_bytes(&L.f, &L.wsf)) return e;
+  if (int e = nsa_decode_workspace_bytes(&L.s, &L.wss)) return e;
+  size_t o = 0;
+  L.off_rq = o;     o = up256(o + (size_t)d->batch * d->heads * d->dim_head * 2);
+  L.off_wsc = o;    o = up256(o + L.wsc);
+  L.off_wsf = o;    o = up256(o + L.wsf);
+  L.off_wss = o;    o = up256(o + L.wss);
+  L.off_logits = o; o = up256(o + (size_t)d->batch * d->heads * (d->num_compressed > 0 ? d->num_compressed : 1) * 4);
+  const size_t sel = (size_t)d->batch * L.sel_units * (L.k > 0 ? L.k : 1);
+  L.off_idx = o;    o = up256(o + sel * 4);
+  L.off_vals = o;   o = up256(o + sel * 4);
+  L.off_fm = o;     o = up256(o + sel);
+  L.total = o;
+  return 0;
+}
+
+}  // namespace nsa
+
+extern "C" int nsa_decode_step_workspace_bytes(const nsa_decode_step_desc* desc, size_t* bytes, size_t* idx_offset, size_t* fmask_offset,
+                                               int32_t* num_selected) {
+  nsa::StepLayout L;
+  if (int e = nsa::make_step_layout(desc, L)) return e;
+  if (!bytes) return NSA_E_ARG;
+  *bytes = L.total;
+  if (idx_offset) *idx_offset = L.off_idx;
+  if (fmask_offset) *fmask_offset = L.off_fm;
+  if (num_selected) *num_selected = L.k;
+  return 0;
+}
+
+extern "C" int nsa_decode_step(const nsa_decode_step_desc* d, const void* q, const void* k, const void* v, const float* freqs,
+                               void* k_cache, void* v_cache, const void* ck_cache, const void* cv_cache, const void* mem_k,
+                               const void* mem_v, void* k_run_row, void* v_run_row, const void* gate_logits, void* ws, size_t ws_bytes,
+                               void* out, void* stream) {
+  using namespace nsa;
+  StepLayout L;
+  if (int e = make_step_layout(d, L)) return e;
+  if (!q || !k || !v || !freqs || !k_cache || !v_cache || !gate_logits || !ws || !out) return NSA_E_ARG;
+  if (ws_bytes < L.total) return NSA_E_WORKSPACE;
+  if (d->num_compressed > 0 && (!ck_cache || !cv_cache)) return NSA_E_ARG;
+  char* w = (char*)ws;
+  void* rq = w + L.off_rq;
+  // row `pos` of the caches
+  const int64_t krs[2] = {d->kc_stride[0], d->kc_stride[1]}, vrs[2] = {d->vc_stride[0], d->vc_stride[1]};
+  __bf16* k_row = (__bf16*)k_cache + (int64_t)d->pos * d->kc_stride[2];
+  __bf16* v_row = (__bf16*)v_cache + (int64_t)d->pos * d->vc_stride[2];
+  if (int e = nsa_decode_prep(q, d->q_stride, k, d->k_stride, v, d->v_stride, d->batch, d->heads, d->kv_heads, d->dim_head, freqs, d->pos, rq,
+                              k_row, krs, v_row, vrs, k_run_row, k_run_row ? d->krun_stride : nullptr, v_run_row,
+                              v_run_row ? d->vrun_stride : nullptr, stream))
+    return e;
+  const bool has_c = d->num_compressed > 0;
+  float* logits = (float*)(w + L.off_logits);
+  if (has_c)
+    if (int e = nsa_decode_attend(&L.c, q, ck_cache, cv_cache, mem_k, mem_v, nullptr, nullptr, w + L.off_wsc, L.wsc, nullptr, logits, stream))
+      return e;
+  int32_t* idx = (int32_t*)(w + L.off_idx);
+  uint8_t* fm = (uint8_t*)(w + L.off_fm);
+  if (L.k > 0)
+    if (int e = nsa_decode_topk(logits, d->batch, d->kv_heads, d->heads / d->kv_heads, d->num_compressed, d->per_block, d->share, L.k, idx,
+                                (float*)(w + L.off_vals), fm, stream))
+      return e;
+  if (int e = nsa_decode_attend(&L.f, rq, k_cache, v_cache, nullptr, nullptr, L.k > 0 ? idx : nullptr, L.k > 0 ? fm : nullptr, w + L.off_wsf,
+                                L.wsf, nullptr, nullptr, stream))
+    return e;
+  if (int e = nsa_decode_attend(&L.s, rq, k_cache, v_cache, nullptr, nullptr, nullptr, nullptr, w + L.off_wss, L.wss, nullptr, nullptr, stream))
+    return e;
+  return nsa_decode_combine(has_c ? &L.c : nullptr, has_c ? w + L.off_wsc : nullptr, &L.f, w + L.off_wsf, &L.s, w + L.off_wss, gate_logits, out,
+                            stream);
+}

@@ -703,3 +703,67 @@ def decode_importance_topk(logits: Tensor, kv_heads: int, per_block: int, share:
     _lib.check(_lib.lib().nsa_decode_topk(_ptr(logits), b, int(kv_heads), hq // kv_heads, nc, int(per_block), int(bool(share)),
                                           int(num_selected), _ptr(idx), _ptr(vals), _ptr(fm), _stream()), "nsa_decode_topk")
     return vals, idx, fm.view(torch.bool)
+
+
+@torch.no_grad()
+def decode_step(q: Tensor, k: Tensor, v: Tensor, freqs: Tensor, pos: int, keys: Tensor, vals: Tensor, ck: Tensor | None, cv: Tensor | None,
+                mem_k: Tensor | None, mem_v: Tensor | None, k_run_row: Tensor | None, v_run_row: Tensor | None, gate_logits: Tensor,
+                *, per_block: int, block: int, num_sel: int, share: bool, window: int):
+    """The attention part of one decode step in a single library call (see nsa_decode_step in
+    include/nsa_hip.h).  q 'b hq 1 d', k, v 'b hk 1 d': the new token's projections; keys, vals: the
+    caches with row `pos` free ('b hk >=pos+1 d' views from the start of their buffers); ck, cv: the
+    compressed caches (None or empty before the first compressed key); mem_k, mem_v 'hk m d'.
+    Returns (merged 'b 1 (h d)', idx int32, fmask bool) with idx / fmask 'b hk|hq 1 k'."""
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    b, hq, _, d = q.shape
+    hk = k.shape[1]
+    nc = 0 if ck is None else ck.shape[2]
+    for t in (keys, vals) + ((ck, cv) if nc else ()):
+        if t.dtype != _BF16 or not t.is_cuda or not _rows_ok(t):
+            raise RuntimeError("decode_step: caches must be bf16 device tensors with unit feature stride and 16-byte aligned rows")
+    if keys.shape[2] < pos + 1 or vals.shape[2] < pos + 1:
+        raise RuntimeError("decode_step: the caches have no row for the new token")
+    dsc = _lib.DecodeStepDesc()
+    dsc.batch, dsc.heads, dsc.kv_heads, dsc.dim_head = b, hq, hk, d
+    dsc.pos, dsc.num_compressed, dsc.per_block, dsc.block = int(pos), nc, int(per_block), int(block)
+    dsc.num_sel, dsc.share, dsc.window, dsc.scale = int(num_sel), int(bool(share)), int(window), d ** -0.5
+    m = 0
+    if nc and mem_k is not None:
+        mem_k, mem_v = mem_k.to(_BF16).contiguous(), mem_v.to(_BF16).contiguous()
+        m = mem_k.shape[-2]
+    dsc.num_mem = m
+    for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v)):
+        getattr(dsc, name)[:] = (t.stride(0), t.stride(1))
+    dsc.kc_stride[:] = keys.stride()[:3]
+    dsc.vc_stride[:] = vals.stride()[:3]
+    if nc:
+        dsc.ck_stride[:] = ck.stride()[:3]
+        dsc.cv_stride[:] = cv.stride()[:3]
+    run = k_run_row is not None and v_run_row is not None
+    if run:
+        for t in (k_run_row, v_run_row):
+            if t.dtype != _BF16 or t.shape != (b, hk, 1, d) or not _rows_ok(t):
+                raise RuntimeError("decode_step: window rows must be bf16 'b hk 1 d' views")
+        dsc.krun_stride[:] = (k_run_row.stride(0), k_run_row.stride(1))
+        dsc.vrun_stride[:] = (v_run_row.stride(0), v_run_row.stride(1))
+    L = _lib.lib()
+    nbytes, ioff, foff, ksel = C.c_size_t(), C.c_size_t(), C.c_size_t(), C.c_int32()
+    _lib.check(L.nsa_decode_step_workspace_bytes(C.byref(dsc), C.byref(nbytes), C.byref(ioff), C.byref(foff), C.byref(ksel)),
+               "nsa_decode_step_workspace_bytes")
+    ws = torch.empty(nbytes.value, dtype=torch.uint8, device=q.device)
+    gl = gate_logits if gate_logits.dtype == _BF16 and gate_logits.is_contiguous() else gate_logits.to(_BF16).contiguous()
+    if gl.numel() != b * hq * 3:
+        raise RuntimeError("decode_step: gate logits must be 'b 1 (h 3)'")
+    freqs = freqs.detach()
+    if freqs.dtype != torch.float32 or not freqs.is_contiguous():
+        freqs = freqs.to(torch.float32).contiguous()
+    out = torch.empty((b, 1, hq * d), dtype=_BF16, device=q.device)
+    _lib.check(L.nsa_decode_step(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(freqs), _ptr(keys), _ptr(vals), _ptr(ck) if nc else None,
+                                 _ptr(cv) if nc else None, _ptr(mem_k) if m else None, _ptr(mem_v) if m else None,
+                                 _ptr(k_run_row) if run else None, _ptr(v_run_row) if run else None, _ptr(gl), _ptr(ws), nbytes, _ptr(out),
+                                 _stream()), "nsa_decode_step")
+    units = hk if share else hq
+    kk = ksel.value
+    idx = ws[ioff.value:ioff.value + b * units * kk * 4].view(torch.int32).view(b, units, 1, kk)
+    fm = ws[foff.value:foff.value + b * units * kk].view(torch.bool).view(b, units, 1, kk)
+    return out, idx, fm

@@ -177,28 +177,29 @@ class SparseAttention(nn.Module):
         q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
         q16, k16, v16 = q.to(bf16), k.to(bf16), v.to(bf16)
 
-        # raw tokens of the open compression window (not rotated, NSA.py:377-380)
+        # raw tokens of the open compression window (not rotated, NSA.py:377-380) and the caches' new row
         run_k, rk_row = _append_rows(run_k, dtype=run_k.dtype, min_capacity=cbs)
         run_v, rv_row = _append_rows(run_v, dtype=run_v.dtype, min_capacity=cbs)
         fused_run = run_k.dtype == bf16 and run_v.dtype == bf16
         if not fused_run:
             rk_row.copy_(k)
             rv_row.copy_(v)
+        keys, _ = _append_rows(cache_k)
+        vals, _ = _append_rows(cache_v)
 
-        # the rotated key and the value go into row t of the caches (NSA.py:384-393); the same kernel
-        # rotates the queries and (bf16 windows) fills the rows of the open compression window
-        keys, k_row = _append_rows(cache_k)
-        vals, v_row = _append_rows(cache_v)
-        rq16 = ops.decode_prep(q16, k16, v16, freqs, t, k_row, v_row, rk_row if fused_run else None, rv_row if fused_run else None)
-
-        # 1. compressed branch: every cached compressed key, no mask (NSA.py:396-420)
+        # one library call for the attention part of the step: rotation of q / k and the new cache rows
+        # (NSA.py:384-393), compressed branch over every cached compressed key (NSA.py:396-420), block
+        # selection from its logits (NSA.py:448-476), selected blocks + own block (NSA.py:446-515), last
+        # window + 1 keys (NSA.py:519-530), merge + sigmoid gate + head merge (NSA.py:534-545)
         nc = cache_ck.shape[-2]
-        logits = c_part = None
+        ck16 = cv16 = None
         if nc > 0:
             ck16 = cache_ck if cache_ck.dtype == bf16 else cache_ck.to(bf16)
             cv16 = cache_cv if cache_cv.dtype == bf16 else cache_cv.to(bf16)
-            c_part, logits = ops.decode_range_attend(q16, ck16, cv16, 0, nc, self.compress_mem_kv[0], self.compress_mem_kv[1],
-                                                     return_logits=True, merge=False)
+        merged, _, _ = ops.decode_step(q16, k16, v16, freqs, t, keys, vals, ck16, cv16, self.compress_mem_kv[0], self.compress_mem_kv[1],
+                                       rk_row if fused_run else None, rv_row if fused_run else None, self.to_strategy_combine[0](x),
+                                       per_block=B // st, block=B, num_sel=self.num_selected_blocks,
+                                       share=self.query_heads_share_selected_kv, window=self.sliding_window_size)
 
         # a compression window is complete: compress it, keep the overlap (NSA.py:422-441)
         ck, cv = cache_ck, cache_cv
@@ -211,24 +212,6 @@ class SparseAttention(nn.Module):
             ck_row.copy_(next_ck)
             cv_row.copy_(next_cv)
 
-        # 2. selection branch (NSA.py:446-515): top blocks by importance + own block up to t
-        npf = B // st
-        nb = nc // npf
-        num_sel = min(self.num_selected_blocks, nb)
-        if num_sel > 0:
-            # pooling over the block's compressed keys and the group's heads, padded softmax and top-k in one kernel
-            _, idx, fmask = ops.decode_importance_topk(logits, self.kv_heads, npf, self.query_heads_share_selected_kv, num_sel)
-        else:
-            idx = torch.zeros((b, self.kv_heads, 1, 0), dtype=torch.int32, device=inp.device)
-            fmask = idx.bool()
-        f_part = ops.decode_select_attend(rq16, keys, vals, t + 1, B, idx, fmask, merge=False)
-
-        # 3. sliding branch: the last window + 1 keys (NSA.py:519-530)
-        w = min(t + 1, self.sliding_window_size + 1)
-        s_part = ops.decode_range_attend(rq16, keys, vals, t + 1 - w, w, merge=False)
-
-        # merge of the split-K partials, sigmoid gate and head merge in one kernel (NSA.py:534-545)
-        merged = ops.decode_combine(self.to_strategy_combine[0](x), c_part, f_part, s_part)
         out = self.combine_heads(merged.to(x.dtype))
         if not return_cache:
             return out

@@ -192,21 +192,22 @@ def test_module_decode_matches_oracle_decode(ci, prefill):
         y, cache = mod(x[:, :prefill].to(DEV), return_cache=True)
         _, rcache = ref(x[:, :prefill].float(), return_cache=True)
     captured = {}
-    orig = ops.decode_importance_topk
-    def spy(*a):
-        r = orig(*a)
-        captured["sel"] = (r[1].cpu().long(), r[2].cpu())
+    orig = ops.decode_step
+    def spy(*a, **kw_):
+        r = orig(*a, **kw_)
+        if r[1].shape[-1] > 0:
+            captured["sel"] = (r[1].cpu().long(), r[2].cpu())
         return r
     agree = total = 0
     worst = 0.0
     for i in range(prefill, n):
         captured.clear()
-        ops.decode_importance_topk = spy
+        ops.decode_step = spy
         try:
             out, cache = mod(x[:, i:i + 1].to(DEV), cache=cache, return_cache=True)
             torch.cuda.synchronize()
         finally:
-            ops.decode_importance_topk = orig
+            ops.decode_step = orig
         with torch.no_grad():
             own, _ = ref(x[:, i:i + 1].float(), cache=rcache, return_cache=True)           # the oracle's own selection
             want, rcache2 = ref(x[:, i:i + 1].float(), cache=rcache, return_cache=True, selection_override=captured.get("sel"))
