@@ -119,3 +119,47 @@ def test_module_edge_shapes_run():
         x = torch.randn(2, n, 128, device=DEV, dtype=torch.bfloat16)
         y = m(x)
         assert y.shape == x.shape and torch.isfinite(y).all(), (causal, n, S)
+
+
+def test_fp32_module_runs_and_matches_oracle():
+    """A module left in fp32 (the reference's default dtype): parameters and activations stay fp32 for the
+    projections, the kernels compute in bf16; forward, backward and cached decoding must work and agree
+    with the oracle within the bf16 tolerances."""
+    from native_sparse_attention_pytorch_amd.sparse_attention import SparseAttention
+    kw = dict(dim=128, dim_head=64, heads=4, kv_heads=2, sliding_window_size=16, compress_block_size=8,
+              compress_block_sliding_stride=4, selection_block_size=16, num_selected_blocks=2, causal=True)
+    torch.manual_seed(21)
+    ref = O.SparseAttentionOracle(**kw)
+    with torch.no_grad():
+        ref.to_strategy_combine[0].weight.normal_(std=0.05)
+    mod = SparseAttention(**kw)
+    mod.load_state_dict(ref.state_dict(), strict=True)
+    mod = mod.to(DEV)                                   # fp32
+    x = torch.randn(2, 90, 128, generator=torch.Generator().manual_seed(5))
+    from native_sparse_attention_pytorch_amd import ops
+    captured = {}
+    orig = ops.importance_topk
+    def spy(imp, k):
+        r = orig(imp, k)
+        captured["sel"] = (r[1].cpu().long(), r[2].cpu())
+        return r
+    ops.importance_topk = spy
+    try:
+        xg = x.to(DEV).requires_grad_()
+        out = mod(xg)
+        out.sum().backward()
+    finally:
+        ops.importance_topk = orig
+    assert out.dtype == torch.float32 and xg.grad is not None and torch.isfinite(xg.grad).all()
+    want = ref(x, selection_override=captured["sel"])
+    assert_close(out, want, 3e-2 * want.abs().max().item(), 2e-2, "fp32 module out")
+    # prefill + decode with fp32 caches handed back by the parallel forward
+    with torch.no_grad():
+        y, cache = mod(x[:, :60].to(DEV), return_cache=True)
+        outs = [y]
+        for i in range(60, 90):
+            o, cache = mod(x[:, i:i + 1].to(DEV), cache=cache, return_cache=True)
+            outs.append(o)
+    seq = torch.cat(outs, dim=1)
+    bad = ((seq.float().cpu() - want).abs() > 4e-2 * want.abs().max()).any(dim=-1).float().mean().item()
+    assert bad < 0.05, f"{bad:.3f} of the tokens differ between prefill+decode and the oracle's parallel forward"
