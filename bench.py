@@ -281,6 +281,41 @@ def main():
     except Exception as ex:
         res["decode_layer_32k"] = dict(error=repr(ex))
 
+    # BASELINE configs[4]: end-to-end training step of the small NSA transformer on byte tokens
+    # (depth 6, dim 512, 8/4 heads, batch 8 x 1024 tokens; fp32 master weights, bf16 autocast, Adam)
+    try:
+        if args.headline_only:
+            raise _Skip()
+        from native_sparse_attention_pytorch_amd.transformer import Transformer
+        torch.manual_seed(0)
+        model = Transformer(num_tokens=256, dim=512, depth=6, dim_head=64, heads=8, kv_heads=4,
+                            sparse_attn_kwargs=dict(sliding_window_size=64, compress_block_size=16, compress_block_sliding_stride=8,
+                                                    selection_block_size=16, num_selected_blocks=4)).to(dev)
+        opt = torch.optim.Adam(model.parameters(), lr=1e-4)
+        ids = torch.randint(0, 256, (8, 1025), device=dev)
+
+        def train_step():
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                loss = model(ids, return_loss=True)
+            loss.backward()
+            opt.step()
+            opt.zero_grad()
+            return loss
+        for _ in range(3):
+            train_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            last = train_step()
+        torch.cuda.synchronize()
+        tt = (time.perf_counter() - t0) / 10
+        res["train_config5"] = dict(ms_per_step=round(tt * 1e3, 3), tokens_per_s=round(8 * 1024 / tt, 1), loss_after=round(last.item(), 4))
+        del model, opt
+    except _Skip:
+        pass
+    except Exception as ex:
+        res["train_config5"] = dict(error=repr(ex))
+
     if not args.no_cpu:
         torch.set_num_threads(min(16, os.cpu_count() or 1))
         base, ref = cpu_baseline(cfg, q, k, v, do, idx, msk)

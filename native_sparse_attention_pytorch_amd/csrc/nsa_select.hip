@@ -325,7 +325,7 @@ __device__ __forceinline__ void store_tile_rows(const floatx16 (&acc)[D / 32], f
   for (int t = 0; t < 32 / RPI; ++t) {
     const int rr = t * RPI + lane / CPR, c = lane % CPR;
     const bf16x8 v = *reinterpret_cast<const bf16x8*>(tile_s + rr * RS + 8 * c);
-    *reinterpret_cast<bf16x8*>(dst + row_s[rr] * D + 8 * c) = v;
+    __builtin_nontemporal_store(v, reinterpret_cast<bf16x8*>(dst + row_s[rr] * D + 8 * c));
   }
   __syncthreads();
 }
@@ -509,8 +509,8 @@ __global__ __launch_bounds__(256) void sel_fwd_combine_kernel(const SelPlan P, c
     for (unsigned long long m = live; m; m &= m - 1) {
       const int s = __builtin_ctzll(m);
       const size_t row = row0 + (size_t)s * P.g;
-      const float ls = lsepart[row];
-      const bf16x8 o = load8(opart + row * D + dd);
+      const float ls = __builtin_nontemporal_load(lsepart + row);
+      const bf16x8 o = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(opart + row * D + dd));
       const float mn = fmaxf(mx, ls);
       const float a = __expf(mx - mn), w = __expf(ls - mn);      // first slot: mx = -inf -> a = 0
       sum = sum * a + w;
@@ -714,7 +714,7 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
     for (unsigned long long m = live; m; m &= m - 1) {
       const int s = __builtin_ctzll(m);
-      const bf16x8 o = load8(dqpart + (row0 + (size_t)s * P.g) * D + dd);
+      const bf16x8 o = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(dqpart + (row0 + (size_t)s * P.g) * D + dd));
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] += (float)o[e];
     }
@@ -915,7 +915,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
       for (int t = 0; t < 32 / RPI; ++t) {
         const int rr = t * RPI + (int)threadIdx.x / CPR, c = threadIdx.x % CPR;
         const bf16x8 vv = *reinterpret_cast<const bf16x8*>(dq_s + rr * RS + 8 * c);
-        *reinterpret_cast<bf16x8*>(dqpart + row_s[rr] * D + 8 * c) = vv;
+        __builtin_nontemporal_store(vv, reinterpret_cast<bf16x8*>(dqpart + row_s[rr] * D + 8 * c));
       }
       __syncthreads();
     }
