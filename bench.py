@@ -255,27 +255,41 @@ def main():
             raise _Skip()
         from native_sparse_attention_pytorch_amd import SparseAttention
         torch.manual_seed(0)
-        bd, ctx = 32, 32768
+        ctx = 32768
         mod = SparseAttention(dim=hq * d, dim_head=d, heads=hq, kv_heads=hk, sliding_window_size=512, compress_block_size=32,
                               compress_block_sliding_stride=16, selection_block_size=B, num_selected_blocks=S + 1, causal=True).to(dev).bfloat16()
-        def filled(rows, cap):          # a cache tensor as the module hands it back: prefix of a buffer with spare rows
-            buf = torch.randn(bd, hk, cap, d, device=dev, dtype=torch.bfloat16)
-            buf._nsa_filled = rows
-            return buf[:, :, :rows]
-        cache = ((filled(ctx, ctx + 256), filled(ctx, ctx + 256)),
-                 ((filled(ctx // 16, ctx // 16 + 64), filled(ctx // 16, ctx // 16 + 64)),
-                  (torch.zeros(bd, hk, 16, d, device=dev, dtype=torch.bfloat16), torch.zeros(bd, hk, 16, d, device=dev, dtype=torch.bfloat16))))
-        xt = torch.randn(bd, 1, hq * d, device=dev, dtype=torch.bfloat16)
-        for _ in range(40):             # includes the first compression step (one-time library initialisation)
-            _, cache = mod(xt, cache=cache, return_cache=True)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(100):
-            _, cache = mod(xt, cache=cache, return_cache=True)
-        torch.cuda.synchronize()
-        td = (time.perf_counter() - t0) / 100
-        res["decode_layer_32k"] = dict(batch=bd, us_per_step=round(td * 1e6, 1), tokens_per_s=round(bd / td, 1))
-        del mod, cache
+        from native_sparse_attention_pytorch_amd.decode_session import DecodeSession
+        dec = {}
+        for bd in (1, 32):
+            def filled(rows, cap):          # a cache tensor as the module hands it back: prefix of a buffer with spare rows
+                buf = torch.randn(bd, hk, cap, d, device=dev, dtype=torch.bfloat16)
+                buf._nsa_filled = rows
+                return buf[:, :, :rows]
+            cache = ((filled(ctx, ctx + 256), filled(ctx, ctx + 256)),
+                     ((filled(ctx // 16, ctx // 16 + 64), filled(ctx // 16, ctx // 16 + 64)),
+                      (torch.zeros(bd, hk, 16, d, device=dev, dtype=torch.bfloat16), torch.zeros(bd, hk, 16, d, device=dev, dtype=torch.bfloat16))))
+            xt = torch.randn(bd, 1, hq * d, device=dev, dtype=torch.bfloat16)
+            # the same steps replayed from a captured HIP graph (fixed-capacity caches, lengths read on the device)
+            sess = DecodeSession(mod, cache, max_len=ctx + 256)
+            for _ in range(40):             # includes the first compression step (one-time library initialisation)
+                _, cache = mod(xt, cache=cache, return_cache=True)
+                sess.step(xt)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(100):
+                _, cache = mod(xt, cache=cache, return_cache=True)
+            torch.cuda.synchronize()
+            td = (time.perf_counter() - t0) / 100
+            t0 = time.perf_counter()
+            for _ in range(100):
+                sess.step(xt)
+            torch.cuda.synchronize()
+            tg = (time.perf_counter() - t0) / 100
+            dec[f"batch{bd}"] = dict(us_per_step=round(td * 1e6, 1), tokens_per_s=round(bd / td, 1),
+                                     graph_us_per_step=round(tg * 1e6, 1), graph_tokens_per_s=round(bd / tg, 1))
+            del sess, cache
+        res["decode_layer_32k"] = dec
+        del mod
     except _Skip:
         pass
     except Exception as ex:

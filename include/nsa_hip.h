@@ -231,6 +231,25 @@ int nsa_decode_step(const nsa_decode_step_desc* desc, const void* q, const void*
                     const void* mem_v, void* k_run_row, void* v_run_row, const void* gate_logits, void* ws, size_t ws_bytes,
                     void* out, void* stream);
 
+/* nsa_decode_step with the lengths read from device memory when the kernels run, so that the whole step can be
+ * recorded once into a HIP graph and replayed for every token (the host-side cost of a step is otherwise several
+ * times the kernels' run time at small batch).  No counterpart in the reference, whose decode step re-derives all
+ * shapes on the host (NSA.py:338-547).
+ * state: device int32[2] = {rows already in the key / value caches (the new token's position), compressed keys
+ * cached}.  `capacity` is a step descriptor whose pos and num_compressed give the LAST position the caches have a
+ * row for and the rows of the compressed caches: grids, the workspace and the selection's row stride are sized for
+ * them; min(num_sel, state[1] / per_block) blocks are selected.  k_run / v_run (optional, both or neither): rings of
+ * run_ring rows per (batch, kv head), element strides capacity->krun_stride / vrun_stride {batch, head} and
+ * krun_row_stride / vrun_row_stride; the un-rotated key / value of the new token go to row state[0] % run_ring.
+ * gate_logits: bf16, row b at gate_logits + b * gate_row_stride (0: rows are contiguous), gate_bias (optional, bf16
+ * [3 * heads]) is added to them - so the gate projection can be columns of the same GEMM as q, k, v.
+ * advance != 0: the call's last kernel adds 1 to state[0].  The call neither allocates nor synchronises. */
+int nsa_decode_step_dyn(const nsa_decode_step_desc* capacity, int32_t* state, const void* q, const void* k, const void* v,
+                        const float* freqs, void* k_cache, void* v_cache, const void* ck_cache, const void* cv_cache,
+                        const void* mem_k, const void* mem_v, void* k_run, void* v_run, int64_t krun_row_stride,
+                        int64_t vrun_row_stride, int32_t run_ring, const void* gate_logits, int64_t gate_row_stride,
+                        const void* gate_bias, void* ws, size_t ws_bytes, void* out, int32_t advance, void* stream);
+
 /* Decode step: rotates the new token's queries (-> rq, bf16 [batch, heads, d] contiguous) and keys to
  * position pos, writes the rotated keys into row pos of the key cache and the values into row pos
  * of the value cache.  Replaces rotate_queries_or_keys x2 and the two cache concatenations of

@@ -97,6 +97,8 @@ def lib():
         L.nsa_decode_step_workspace_bytes.argtypes = [ds, C.POINTER(sz), C.POINTER(sz), C.POINTER(sz), C.POINTER(C.c_int32)]
         L.nsa_decode_step.argtypes = [ds] + [vp] * 14 + [sz, vp, vp]
         L.nsa_decode_step_workspace_bytes.restype = L.nsa_decode_step.restype = C.c_int
+        L.nsa_decode_step_dyn.argtypes = [ds] + [vp] * 13 + [C.c_int64, C.c_int64, C.c_int32, vp, C.c_int64, vp, vp, sz, vp, C.c_int32, vp]
+        L.nsa_decode_step_dyn.restype = C.c_int
         L.nsa_windows_fwd.argtypes = [vp, i3, vp] + [C.c_int32] * 6 + [vp, vp]
         L.nsa_windows_bwd.argtypes = [vp] + [C.c_int32] * 6 + [vp, vp]
         L.nsa_windows_fwd.restype = L.nsa_windows_bwd.restype = C.c_int

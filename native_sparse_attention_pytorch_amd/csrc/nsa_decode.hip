@@ -28,7 +28,33 @@ struct DecodePlan {
   int idx64;
   float scale;
   long sq[2], sk[3], sv[3];
+  int sstride, lstride;              // row strides of the selection (idx / fmask) and of the logits output
+  // Lengths read at run time, for a step replayed from a captured graph: dyn[0] = rows in the key / value caches before
+  // this token, dyn[1] = compressed keys cached.  The fields above then hold capacities (the grid and the partial
+  // records are sized for them) and resolve() replaces them inside the kernel.
+  const int* dyn;
+  int dyn_kind;                      // 1 compressed range, 2 selected blocks, 3 sliding window
+  int window, per_block, smax;
 };
+
+__device__ __forceinline__ void resolve(DecodePlan& P) {
+  if (P.dyn == nullptr) return;
+  const int kv_len = P.dyn[0] + 1, nc = P.dyn[1];
+  if (P.dyn_kind == 1) {
+    P.count = nc;
+    if (nc == 0) P.mem = 0;                            // no compressed key yet: the branch contributes nothing (NSA.py:401)
+    P.tiles = ((P.mem + 31) >> 5) + ((nc + 31) >> 5);
+  } else if (P.dyn_kind == 2) {
+    P.kv_len = kv_len;
+    P.S = min(P.smax, nc / P.per_block);
+    P.tiles = (P.S + 1) * P.tps;
+  } else {
+    const int w = min(kv_len, P.window + 1);
+    P.start = kv_len - w;
+    P.count = w;
+    P.tiles = (w + 31) >> 5;
+  }
+}
 
 constexpr int kDecodeWaves = 2;      // waves per work-group; each stages its own K / V tile in LDS
 
@@ -63,7 +89,7 @@ __device__ __forceinline__ DecodeTile decode_tile(const DecodePlan& P, int D, in
     long blk;
     bool live = true;
     if (slot < P.S) {
-      const long e = (long)ug * P.S + slot;
+      const long e = (long)ug * P.sstride + slot;
       blk = P.idx64 ? reinterpret_cast<const long*>(idx)[e] : (long)reinterpret_cast<const int*>(idx)[e];
       live = fmask[e] != 0 && blk >= 0 && blk * P.B < P.kv_len;
       if (!live) blk = 0;
@@ -80,13 +106,15 @@ __device__ __forceinline__ DecodeTile decode_tile(const DecodePlan& P, int D, in
 }
 
 template <int D>
-__global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_eu(2))) void decode_attend_kernel(const DecodePlan P, const __bf16* __restrict__ q,
+__global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_eu(2))) void decode_attend_kernel(const DecodePlan P_launch, const __bf16* __restrict__ q,
                                                                           const __bf16* __restrict__ k, const __bf16* __restrict__ v,
                                                                           const __bf16* __restrict__ mem_k, const __bf16* __restrict__ mem_v,
                                                                           const void* __restrict__ idx, const unsigned char* __restrict__ fmask,
                                                                           float* __restrict__ part, float* __restrict__ logits) {
   constexpr int KS = D / 16, DT = D / 32, RS = D + 8, RSV = D + 16;   // row reads want 4 banks per row, transpose loads 8
   constexpr int LPR = D / 8, RPI = 64 / LPR, NI = 32 / RPI;      // lanes per row, rows per load instruction, instructions per tile
+  DecodePlan P = P_launch;
+  resolve(P);
   __shared__ __align__(16) __bf16 kv_s[kDecodeWaves][2][32 * RSV];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_ = lane & 31, h = lane >> 5;
   const int lr = lane / LPR, lc = lane % LPR;
@@ -153,7 +181,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_
     for (int i = 0; i < 16; ++i) {
       const int kl = 8 * (i >> 2) + 4 * h + (i & 3);
       if (logits != nullptr && T.lcol >= 0 && n_ < P.gc && kl < T.nvalid)
-        logits[((long)b * P.hk * P.g + head0 + n_) * P.count + T.lcol + kl] = Sa[i] * P.scale;
+        logits[((long)b * P.hk * P.g + head0 + n_) * P.lstride + T.lcol + kl] = Sa[i] * P.scale;
       const float s = kl < T.nvalid ? Sa[i] * sc : -INFINITY;
       Sa[i] = s;
       mx = fmaxf(mx, s);
@@ -198,43 +226,87 @@ __global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_
   }
 }
 
-// Feature `f` of head (b, head) of one branch: log-sum-exp merge of the split-K partials.
+// Log-sum-exp merge of the split-K partials of head (b, head) of one branch by a work-group of D threads: the
+// partials' maxima and sums are read by one thread each and reduced through LDS, then thread f accumulates
+// feature f over the partials that carry weight (loads independent of each other, so they overlap).
+constexpr int kMaxParts = 64 * kDecodeWaves;
+
 template <int D>
-__device__ __forceinline__ float merge_head_partials(const DecodePlan& P, const float* __restrict__ part, int b, int head, int f) {
+__device__ __forceinline__ float merge_head_partials(const DecodePlan& P, const float* __restrict__ part, int b, int head, int f,
+                                                     float* w_s, float* red_s) {
   const int u = (P.units == P.hk) ? head / P.g : head, gi = (P.units == P.hk) ? head % P.g : 0;
   const float* base = part + (long)(b * P.units + u) * P.nparts * P.rec;
   const int om = P.gc * D + gi, ol = om + P.gc;
+  constexpr int PT = (kMaxParts + D - 1) / D;          // partials per thread
+  float mp[PT], lp[PT];
   float M = -INFINITY;
-  for (int p = 0; p < P.nparts; ++p) M = fmaxf(M, base[(long)p * P.rec + om]);
-  if (!(M > -INFINITY)) return 0.f;                    // no wave saw a key
-  float acc = 0.f, L = 0.f;
-  for (int p = 0; p < P.nparts; ++p) {
-    const float* rec = base + (long)p * P.rec;
-    const float w = fast_exp2(rec[om] - M);            // exp2(-inf) = 0 for waves that saw no key
-    L += w * rec[ol];
-    acc += w * rec[gi * D + f];
+#pragma unroll
+  for (int r = 0; r < PT; ++r) {
+    const int p = f + r * D;
+    mp[r] = p < P.nparts ? base[(long)p * P.rec + om] : -INFINITY;
+    lp[r] = p < P.nparts ? base[(long)p * P.rec + ol] : 0.f;
+    M = fmaxf(M, mp[r]);
   }
+  auto block_reduce = [&](float v, bool is_max) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const float t = __shfl_xor(v, o, 64);
+      v = is_max ? fmaxf(v, t) : v + t;
+    }
+    if (D > 64) {
+      __syncthreads();
+      if ((f & 63) == 0) red_s[f >> 6] = v;
+      __syncthreads();
+      v = red_s[0];
+#pragma unroll
+      for (int w = 1; w < D / 64; ++w) v = is_max ? fmaxf(v, red_s[w]) : v + red_s[w];
+    }
+    return v;
+  };
+  M = block_reduce(M, true);
+  const bool any = M > -INFINITY;                      // false: no wave saw a key
+  float L = 0.f;
+  __syncthreads();                                     // w_s may still be read for the previous branch
+#pragma unroll
+  for (int r = 0; r < PT; ++r) {
+    const int p = f + r * D;
+    const float w = any ? fast_exp2(mp[r] - M) : 0.f;  // exp2(-inf) = 0 for waves that saw no key
+    if (p < P.nparts) w_s[p] = w;
+    L += w * lp[r];
+  }
+  L = block_reduce(L, false);
+  __syncthreads();
+  float acc = 0.f;
+  // every wave wrote a finite record (zeros when it saw no key), so the loads need no guard and overlap
+#pragma unroll 8
+  for (int p = 0; p < P.nparts; ++p) acc += w_s[p] * base[(long)p * P.rec + gi * D + f];
   return L > 0.f ? acc / L : 0.f;
 }
 
 // one work-group per query head, one thread per feature
 template <int D>
 __global__ __launch_bounds__(D) void decode_merge_kernel(const DecodePlan P, const float* __restrict__ part, __bf16* __restrict__ out) {
+  __shared__ float w_s[kMaxParts], red_s[4];
   const int hq = P.hk * P.g;
   const int bh = blockIdx.x, b = bh / hq, head = bh % hq;
-  out[(long)bh * D + threadIdx.x] = (__bf16)merge_head_partials<D>(P, part, b, head, threadIdx.x);
+  out[(long)bh * D + threadIdx.x] = (__bf16)merge_head_partials<D>(P, part, b, head, threadIdx.x, w_s, red_s);
 }
 
 // Merge of the three branches' partials, sigmoid strategy gate and head merge in one pass
 // (NSA.py:534-545): out[b, head*D + f] = sum_s sigmoid(logit[b, 3*head + s]) * branch_s.
-// A branch without a workspace (no compressed key cached yet) contributes zero.
+// A branch without a workspace (no compressed key cached yet) contributes zero.  `advance` (optional): the step's
+// position counter, incremented here once every attention kernel of the step has run.
 struct CombineArgs {
   DecodePlan P[3];
   const float* part[3];
+  int* advance;
+  long gate_row;                 // elements between the gate logits of consecutive batch rows
+  const __bf16* gate_bias;       // optional [3 * heads], added to the logits (a projection computed without its bias)
 };
 
 template <int D>
 __global__ __launch_bounds__(D) void decode_combine_kernel(const CombineArgs A, const __bf16* __restrict__ gate_logits, __bf16* __restrict__ out) {
+  __shared__ float w_s[kMaxParts], red_s[4];
   const int hq = A.P[0].hk * A.P[0].g;
   const int bh = blockIdx.x, b = bh / hq, head = bh % hq;
   float res = 0.f;
@@ -242,11 +314,13 @@ __global__ __launch_bounds__(D) void decode_combine_kernel(const CombineArgs A, 
   for (int s = 0; s < 3; ++s) {
     if (A.part[s] == nullptr) continue;
     // branch outputs are rounded to bf16 as when each is merged on its own
-    const float o = (float)(__bf16)merge_head_partials<D>(A.P[s], A.part[s], b, head, threadIdx.x);
-    const float gl = (float)gate_logits[((long)b * hq + head) * 3 + s];
+    const float o = (float)(__bf16)merge_head_partials<D>(A.P[s], A.part[s], b, head, threadIdx.x, w_s, red_s);
+    float gl = (float)gate_logits[(long)b * A.gate_row + head * 3 + s];
+    if (A.gate_bias != nullptr) gl += (float)A.gate_bias[head * 3 + s];
     res += o / (1.f + __expf(-gl));
   }
   out[(long)bh * D + threadIdx.x] = (__bf16)res;
+  if (A.advance != nullptr && blockIdx.x == 0 && threadIdx.x == 0) A.advance[0] += 1;
 }
 
 static int make_decode_plan(const nsa_decode_desc* dsc, DecodePlan& P) {
@@ -288,25 +362,12 @@ static int make_decode_plan(const nsa_decode_desc* dsc, DecodePlan& P) {
   if (ns < 1) ns = 1;
   P.nsplit = ns; P.nparts = ns * kDecodeWaves;
   P.rec = P.gc * P.d + ((2 * P.gc + 3) & ~3);
+  P.sstride = P.S; P.lstride = P.count;
   return 0;
 }
 
-}  // namespace nsa
-
-extern "C" int nsa_decode_workspace_bytes(const nsa_decode_desc* dsc, size_t* bytes) {
-  nsa::DecodePlan P;
-  if (int e = nsa::make_decode_plan(dsc, P)) return e;
-  if (!bytes) return NSA_E_ARG;
-  *bytes = (size_t)P.b * P.units * P.nparts * P.rec * sizeof(float);
-  return 0;
-}
-
-extern "C" int nsa_decode_attend(const nsa_decode_desc* dsc, const void* q, const void* k, const void* v, const void* mem_k,
-                                 const void* mem_v, const void* idx, const uint8_t* fmask, void* ws, size_t ws_bytes, void* out,
-                                 float* logits, void* stream) {
-  using namespace nsa;
-  DecodePlan P;
-  if (int e = make_decode_plan(dsc, P)) return e;
+static int launch_attend(const DecodePlan& P, const void* q, const void* k, const void* v, const void* mem_k, const void* mem_v, const void* idx,
+                         const uint8_t* fmask, void* ws, size_t ws_bytes, void* out, float* logits, void* stream) {
   if (!q || !ws) return NSA_E_ARG;
   if (P.mode == 0 && ((P.count > 0 && (!k || !v)) || (P.mem > 0 && (!mem_k || !mem_v)))) return NSA_E_ARG;
   if (P.mode == 1 && (!k || !v || (P.S > 0 && (!idx || !fmask)))) return NSA_E_ARG;
@@ -327,26 +388,25 @@ extern "C" int nsa_decode_attend(const nsa_decode_desc* dsc, const void* q, cons
   return e == hipSuccess ? 0 : (int)e;
 }
 
-extern "C" int nsa_decode_combine(const nsa_decode_desc* compressed, const void* ws_compressed, const nsa_decode_desc* selected,
-                                  const void* ws_selected, const nsa_decode_desc* sliding, const void* ws_sliding,
-                                  const void* gate_logits, void* out, void* stream) {
-  using namespace nsa;
-  const nsa_decode_desc* dsc[3] = {compressed, selected, sliding};
-  const void* ws[3] = {ws_compressed, ws_selected, ws_sliding};
+static int launch_combine(const DecodePlan* plans[3], const void* const ws[3], const void* gate_logits, int64_t gate_row, const void* gate_bias,
+                          void* out, int* advance, void* stream) {
   if (!gate_logits || !out) return NSA_E_ARG;
   CombineArgs A;
+  A.advance = advance;
   int ref = -1;
   for (int s = 0; s < 3; ++s) {
     A.part[s] = nullptr;
     A.P[s] = DecodePlan{};
     if (!ws[s]) continue;
-    if (int e = make_decode_plan(dsc[s], A.P[s])) return e;
+    A.P[s] = *plans[s];
     A.part[s] = (const float*)ws[s];
     if (ref < 0) ref = s;
     else if (A.P[s].b != A.P[ref].b || A.P[s].hk != A.P[ref].hk || A.P[s].g != A.P[ref].g || A.P[s].d != A.P[ref].d) return NSA_E_ARG;
   }
   if (ref < 0) return NSA_E_ARG;
   if (ref != 0) A.P[0] = A.P[ref];         // the kernel reads the head counts from slot 0
+  A.gate_row = gate_row > 0 ? (long)gate_row : 3L * A.P[ref].hk * A.P[ref].g;
+  A.gate_bias = (const __bf16*)gate_bias;
   const int heads = A.P[ref].b * A.P[ref].hk * A.P[ref].g;
   hipStream_t st = (hipStream_t)stream;
   if (A.P[ref].d == 64)
@@ -355,6 +415,40 @@ extern "C" int nsa_decode_combine(const nsa_decode_desc* compressed, const void*
     hipLaunchKernelGGL((decode_combine_kernel<128>), dim3(heads), dim3(128), 0, st, A, (const __bf16*)gate_logits, (__bf16*)out);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
+}
+
+
+}  // namespace nsa
+
+extern "C" int nsa_decode_workspace_bytes(const nsa_decode_desc* dsc, size_t* bytes) {
+  nsa::DecodePlan P;
+  if (int e = nsa::make_decode_plan(dsc, P)) return e;
+  if (!bytes) return NSA_E_ARG;
+  *bytes = (size_t)P.b * P.units * P.nparts * P.rec * sizeof(float);
+  return 0;
+}
+
+extern "C" int nsa_decode_attend(const nsa_decode_desc* dsc, const void* q, const void* k, const void* v, const void* mem_k,
+                                 const void* mem_v, const void* idx, const uint8_t* fmask, void* ws, size_t ws_bytes, void* out,
+                                 float* logits, void* stream) {
+  using namespace nsa;
+  DecodePlan P;
+  if (int e = make_decode_plan(dsc, P)) return e;
+  return launch_attend(P, q, k, v, mem_k, mem_v, idx, fmask, ws, ws_bytes, out, logits, stream);
+}
+
+extern "C" int nsa_decode_combine(const nsa_decode_desc* compressed, const void* ws_compressed, const nsa_decode_desc* selected,
+                                  const void* ws_selected, const nsa_decode_desc* sliding, const void* ws_sliding,
+                                  const void* gate_logits, void* out, void* stream) {
+  using namespace nsa;
+  const nsa_decode_desc* dsc[3] = {compressed, selected, sliding};
+  const void* ws[3] = {ws_compressed, ws_selected, ws_sliding};
+  DecodePlan P[3];
+  const DecodePlan* pp[3] = {&P[0], &P[1], &P[2]};
+  for (int s = 0; s < 3; ++s)
+    if (ws[s])
+      if (int e = make_decode_plan(dsc[s], P[s])) return e;
+  return launch_combine(pp, ws, gate_logits, 0, nullptr, out, nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------- whole step
@@ -475,4 +569,65 @@ extern "C" int nsa_decode_step(const nsa_decode_step_desc* d, const void* q, con
     return e;
   return nsa_decode_combine(has_c ? &L.c : nullptr, has_c ? w + L.off_wsc : nullptr, &L.f, w + L.off_wsf, &L.s, w + L.off_wss, gate_logits, out,
                             stream);
+}
+
+// Declared in nsa_rope.hip / nsa_topk.hip: the prep and top-k launches with lengths read from device memory.
+namespace nsa {
+int decode_prep_dyn(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v, const int64_t* v_stride,
+                    int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head, const float* freqs, void* rq, void* k_cache,
+                    const int64_t* kc_stride, void* v_cache, const int64_t* vc_stride, void* k_run, const int64_t* krun_stride, void* v_run,
+                    const int64_t* vrun_stride, int32_t ring, const int32_t* state, void* stream);
+int decode_topk_launch(const float* logits, int32_t batch, int32_t kv_heads, int32_t group, int32_t num_compressed, int32_t per_block,
+                       int32_t share, int32_t k, int32_t* idx, float* vals, uint8_t* fmask, const int32_t* state, void* stream);
+}  // namespace nsa
+
+extern "C" int nsa_decode_step_dyn(const nsa_decode_step_desc* cap, int32_t* state, const void* q, const void* k, const void* v,
+                                   const float* freqs, void* k_cache, void* v_cache, const void* ck_cache, const void* cv_cache,
+                                   const void* mem_k, const void* mem_v, void* k_run, void* v_run, int64_t krun_row_stride,
+                                   int64_t vrun_row_stride, int32_t run_ring, const void* gate_logits, int64_t gate_row_stride,
+                                   const void* gate_bias, void* ws, size_t ws_bytes, void* out, int32_t advance, void* stream) {
+  using namespace nsa;
+  StepLayout L;
+  if (int e = make_step_layout(cap, L)) return e;
+  if (!state || !q || !k || !v || !freqs || !k_cache || !v_cache || !gate_logits || !ws || !out) return NSA_E_ARG;
+  if (ws_bytes < L.total) return NSA_E_WORKSPACE;
+  const bool has_c = cap->num_compressed > 0;
+  if (has_c && (!ck_cache || !cv_cache)) return NSA_E_ARG;
+  DecodePlan Pc{}, Pf, Ps;
+  if (has_c)
+    if (int e = make_decode_plan(&L.c, Pc)) return e;
+  if (int e = make_decode_plan(&L.f, Pf)) return e;
+  if (int e = make_decode_plan(&L.s, Ps)) return e;
+  int kind = 1;
+  for (DecodePlan* P : {&Pc, &Pf, &Ps}) {
+    P->dyn = state; P->dyn_kind = kind++;
+    P->window = cap->window; P->per_block = cap->per_block; P->smax = L.k;
+  }
+  Pc.lstride = cap->num_compressed;
+  Pf.sstride = L.k;
+
+  char* w = (char*)ws;
+  void* rq = w + L.off_rq;
+  const int64_t krun_s[3] = {cap->krun_stride[0], cap->krun_stride[1], krun_row_stride};
+  const int64_t vrun_s[3] = {cap->vrun_stride[0], cap->vrun_stride[1], vrun_row_stride};
+  if (int e = decode_prep_dyn(q, cap->q_stride, k, cap->k_stride, v, cap->v_stride, cap->batch, cap->heads, cap->kv_heads, cap->dim_head, freqs, rq,
+                              k_cache, cap->kc_stride, v_cache, cap->vc_stride, k_run, krun_s, v_run, vrun_s, run_ring, state, stream))
+    return e;
+  float* logits = (float*)(w + L.off_logits);
+  if (has_c)
+    if (int e = launch_attend(Pc, q, ck_cache, cv_cache, mem_k, mem_v, nullptr, nullptr, w + L.off_wsc, L.wsc, nullptr, logits, stream)) return e;
+  int32_t* idx = (int32_t*)(w + L.off_idx);
+  uint8_t* fm = (uint8_t*)(w + L.off_fm);
+  if (L.k > 0)
+    if (int e = decode_topk_launch(logits, cap->batch, cap->kv_heads, cap->heads / cap->kv_heads, cap->num_compressed, cap->per_block, cap->share,
+                                   L.k, idx, (float*)(w + L.off_vals), fm, state, stream))
+      return e;
+  if (int e = launch_attend(Pf, rq, k_cache, v_cache, nullptr, nullptr, L.k > 0 ? idx : nullptr, L.k > 0 ? fm : nullptr, w + L.off_wsf, L.wsf,
+                            nullptr, nullptr, stream))
+    return e;
+  if (int e = launch_attend(Ps, rq, k_cache, v_cache, nullptr, nullptr, nullptr, nullptr, w + L.off_wss, L.wss, nullptr, nullptr, stream)) return e;
+  const DecodePlan* pp[3] = {&Pc, &Pf, &Ps};
+  const void* wsp[3] = {has_c ? w + L.off_wsc : nullptr, w + L.off_wsf, w + L.off_wss};
+  if (int e = launch_combine(pp, wsp, gate_logits, gate_row_stride, gate_bias, out, advance ? state : nullptr, stream)) return e;
+  return 0;
 }

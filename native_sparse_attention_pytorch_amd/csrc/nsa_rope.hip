@@ -33,6 +33,14 @@ __global__ __launch_bounds__(256) void rope_kernel(const __bf16* __restrict__ x,
   *reinterpret_cast<bf16x8*>(out + bb * o0 + hh * o1 + i * o2 + 8 * c) = r;
 }
 
+// Run-time addressing of a decode step replayed from a graph: state[0] = rows already cached = the new token's position;
+// the *_row strides turn the cache / ring base addresses into the row's address.
+struct DecodeDyn {
+  const int* state;
+  long kc_row, vc_row, krun_row, vrun_row;
+  int ring;
+};
+
 // Decode step: the new token's query heads rotated to position pos (-> rq), its key heads
 // rotated and written into row pos of the key cache, its value heads copied into row pos of
 // the value cache (NSA.py:384-393) - one launch instead of two rotations and a copy.
@@ -41,8 +49,20 @@ __global__ __launch_bounds__(256) void decode_prep_kernel(const __bf16* __restri
                                                           const __bf16* __restrict__ v, long v0, long v1, int b, int hq, int hk,
                                                           const float* __restrict__ freqs, int pos, __bf16* __restrict__ rq,
                                                           __bf16* __restrict__ krow, long kr0, long kr1, __bf16* __restrict__ vrow, long vr0, long vr1,
-                                                          __bf16* __restrict__ krun, long ku0, long ku1, __bf16* __restrict__ vrun, long vu0, long vu1) {
+                                                          __bf16* __restrict__ krun, long ku0, long ku1, __bf16* __restrict__ vrun, long vu0, long vu1,
+                                                          DecodeDyn dyn) {
   constexpr int LPR = D / 8, RPB = 256 / LPR;
+  if (dyn.state != nullptr) {
+    // position read at run time (the launch is replayed from a graph): row pos of the caches, row pos % ring of the window rings
+    pos = dyn.state[0];
+    krow += (long)pos * dyn.kc_row;
+    vrow += (long)pos * dyn.vc_row;
+    if (krun != nullptr) {
+      const int slot = pos % dyn.ring;
+      krun += (long)slot * dyn.krun_row;
+      vrun += (long)slot * dyn.vrun_row;
+    }
+  }
   const int per = hq + 2 * hk;
   const long row = (long)blockIdx.x * RPB + threadIdx.x / LPR;
   if (row >= (long)b * per) return;
@@ -77,12 +97,12 @@ __global__ __launch_bounds__(256) void decode_prep_kernel(const __bf16* __restri
 
 }  // namespace nsa
 
-extern "C" int nsa_decode_prep(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v,
-                               const int64_t* v_stride, int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head,
-                               const float* freqs, int32_t pos, void* rq, void* k_row, const int64_t* k_row_stride, void* v_row,
-                               const int64_t* v_row_stride, void* k_run_row, const int64_t* k_run_stride, void* v_run_row,
-                               const int64_t* v_run_stride, void* stream) {
-  using namespace nsa;
+namespace nsa {
+int decode_prep_launch(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v,
+                       const int64_t* v_stride, int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head,
+                       const float* freqs, int32_t pos, void* rq, void* k_row, const int64_t* k_row_stride, void* v_row,
+                       const int64_t* v_row_stride, void* k_run_row, const int64_t* k_run_stride, void* v_run_row,
+                       const int64_t* v_run_stride, const DecodeDyn& dyn, void* stream) {
   if (!q || !k || !v || !q_stride || !k_stride || !v_stride || !freqs || !rq || !k_row || !v_row || !k_row_stride || !v_row_stride)
     return NSA_E_ARG;
   if (batch <= 0 || heads <= 0 || kv_heads <= 0 || pos < 0) return NSA_E_ARG;
@@ -102,18 +122,42 @@ extern "C" int nsa_decode_prep(const void* q, const int64_t* q_stride, const voi
                        (long)q_stride[1], (const __bf16*)k, (long)k_stride[0], (long)k_stride[1], (const __bf16*)v, (long)v_stride[0],
                        (long)v_stride[1], batch, heads, kv_heads, freqs, pos, (__bf16*)rq, (__bf16*)k_row, (long)k_row_stride[0],
                        (long)k_row_stride[1], (__bf16*)v_row, (long)v_row_stride[0], (long)v_row_stride[1], (__bf16*)k_run_row, ku[0], ku[1],
-                       (__bf16*)v_run_row, vu[0], vu[1]);
+                       (__bf16*)v_run_row, vu[0], vu[1], dyn);
   } else if (dim_head == 128) {
     hipLaunchKernelGGL((decode_prep_kernel<128>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const __bf16*)q, (long)q_stride[0],
                        (long)q_stride[1], (const __bf16*)k, (long)k_stride[0], (long)k_stride[1], (const __bf16*)v, (long)v_stride[0],
                        (long)v_stride[1], batch, heads, kv_heads, freqs, pos, (__bf16*)rq, (__bf16*)k_row, (long)k_row_stride[0],
                        (long)k_row_stride[1], (__bf16*)v_row, (long)v_row_stride[0], (long)v_row_stride[1], (__bf16*)k_run_row, ku[0], ku[1],
-                       (__bf16*)v_run_row, vu[0], vu[1]);
+                       (__bf16*)v_run_row, vu[0], vu[1], dyn);
   } else {
     return NSA_E_UNSUPPORTED;
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
+}
+
+int decode_prep_dyn(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v, const int64_t* v_stride,
+                    int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head, const float* freqs, void* rq, void* k_cache,
+                    const int64_t* kc_stride, void* v_cache, const int64_t* vc_stride, void* k_run, const int64_t* krun_stride, void* v_run,
+                    const int64_t* vrun_stride, int32_t ring, const int32_t* state, void* stream) {
+  if (!state || !kc_stride || !vc_stride || ((kc_stride[2] | vc_stride[2]) & 7)) return NSA_E_ARG;
+  DecodeDyn dyn{state, (long)kc_stride[2], (long)vc_stride[2], 0, 0, 1};
+  if (k_run || v_run) {
+    if (!krun_stride || !vrun_stride || ring <= 0 || ((krun_stride[2] | vrun_stride[2]) & 7)) return NSA_E_ARG;
+    dyn.krun_row = krun_stride[2]; dyn.vrun_row = vrun_stride[2]; dyn.ring = ring;
+  }
+  return decode_prep_launch(q, q_stride, k, k_stride, v, v_stride, batch, heads, kv_heads, dim_head, freqs, 0, rq, k_cache, kc_stride, v_cache,
+                            vc_stride, k_run, krun_stride, v_run, vrun_stride, dyn, stream);
+}
+}  // namespace nsa
+
+extern "C" int nsa_decode_prep(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v,
+                               const int64_t* v_stride, int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head,
+                               const float* freqs, int32_t pos, void* rq, void* k_row, const int64_t* k_row_stride, void* v_row,
+                               const int64_t* v_row_stride, void* k_run_row, const int64_t* k_run_stride, void* v_run_row,
+                               const int64_t* v_run_stride, void* stream) {
+  return nsa::decode_prep_launch(q, q_stride, k, k_stride, v, v_stride, batch, heads, kv_heads, dim_head, freqs, pos, rq, k_row, k_row_stride,
+                                 v_row, v_row_stride, k_run_row, k_run_stride, v_run_row, v_run_stride, nsa::DecodeDyn{nullptr, 0, 0, 0, 0, 1}, stream);
 }
 
 extern "C" int nsa_rope(const void* x, const int64_t* x_stride, int32_t batch, int32_t heads, int32_t seq, int32_t dim_head,

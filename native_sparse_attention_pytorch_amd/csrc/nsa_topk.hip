@@ -34,31 +34,63 @@ __device__ __forceinline__ float wave_max(float v) {
 // Pooling of raw decode logits in front of the top-k (NSA.py:448-476): row (b, u) of the top-k is the mean of
 // logits[b, u*pg + g, j*npf + c] over g < pg heads and c < npf compressed keys (row stride nc).
 struct PoolArgs { int pg, npf, nc, units; };
+// Run-time row length for a decode step replayed from a graph: state[1] compressed keys are cached, so a row has
+// nb = state[1] / per_block entries and min(k, nb) of them are selected; the outputs keep the row stride kstride.
+struct TopkDyn { const int* state; int per_block; };
 
-template <int VPL>
+template <int VPL, bool POOL>
 __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in, long rows, int nb, int k, int softmax, int vec4, PoolArgs pool,
-                                                   int* __restrict__ idx, float* __restrict__ vals, uint8_t* __restrict__ fmask) {
+                                                   int* __restrict__ idx, float* __restrict__ vals, uint8_t* __restrict__ fmask, int kstride, TopkDyn dyn) {
   const int lane = threadIdx.x & 63;
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
+  if (dyn.state != nullptr) {
+    nb = min(nb, dyn.state[1] / dyn.per_block);
+    k = min(k, nb);
+    if (k <= 0) return;
+  }
   const float* src = in + row * nb;
   float x[VPL];
   bool loaded = false;
-  if (pool.pg > 0) {
+  if constexpr (POOL) {
+    __shared__ float row_s[4][64 * VPL];
+    float* rs = row_s[threadIdx.x >> 6];
     const long b = row / pool.units, u = row % pool.units;
     const float* base = in + (b * pool.units * pool.pg + u * pool.pg) * (long)pool.nc;
     const float norm = 1.0f / (float)(pool.pg * pool.npf);
+    if (pool.npf == 4 && (pool.nc & 3) == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0) {
+      // a block's four logits are one 16-byte load; consecutive lanes take consecutive blocks (whole cache lines per
+      // instruction, all loads of a head independent), the sums go through LDS into the per-lane contiguous layout
+      float acc[VPL];
+#pragma unroll
+      for (int r = 0; r < VPL; ++r) acc[r] = 0.f;
+      constexpr int GU = VPL <= 4 ? 4 : (VPL <= 16 ? 2 : 1);      // heads whose loads are issued together
+#pragma unroll GU
+      for (int g = 0; g < pool.pg; ++g) {
+        floatx4 t[VPL];
+#pragma unroll
+        for (int r = 0; r < VPL; ++r) {
+          const int j = r * 64 + lane;
+          t[r] = j < nb ? *reinterpret_cast<const floatx4*>(base + (long)g * pool.nc + 4L * j) : floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int r = 0; r < VPL; ++r) acc[r] += (t[r][0] + t[r][1]) + (t[r][2] + t[r][3]);
+      }
+#pragma unroll
+      for (int r = 0; r < VPL; ++r) rs[r * 64 + lane] = acc[r];
+    } else {
+      for (int j = lane; j < nb; j += 64) {
+        float a = 0.f;
+        for (int g = 0; g < pool.pg; ++g)
+          for (int c = 0; c < pool.npf; ++c) a += base[(long)g * pool.nc + (long)j * pool.npf + c];
+        rs[j] = a;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();                     // LDS operations of one wave execute in order
 #pragma unroll
     for (int r = 0; r < VPL; ++r) {
       const int j = lane * VPL + r;
-      float acc = -INFINITY;
-      if (j < nb) {
-        acc = 0.f;
-        for (int g = 0; g < pool.pg; ++g)
-          for (int c = 0; c < pool.npf; ++c) acc += base[(long)g * pool.nc + (long)j * pool.npf + c];
-        acc *= norm;
-      }
-      x[r] = acc;
+      x[r] = j < nb ? rs[j] * norm : -INFINITY;
     }
     loaded = true;
   }
@@ -126,14 +158,15 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in,
     }
   }
   if (lane < k) {
-    idx[row * k + lane] = res_j;
-    vals[row * k + lane] = res_v;
-    fmask[row * k + lane] = res_v > 1e-10f ? 1 : 0;
+    idx[row * kstride + lane] = res_j;
+    vals[row * kstride + lane] = res_v;
+    fmask[row * kstride + lane] = res_v > 1e-10f ? 1 : 0;
   }
 }
 
 }  // namespace nsa
 
+#define NSA_TOPK_POOL false
 extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k, int32_t apply_softmax,
                         int32_t* idx, float* vals, uint8_t* fmask, void* stream) {
   using namespace nsa;
@@ -144,7 +177,8 @@ extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k
   const int vpl = (nb + 63) / 64;
   const int vec4 = (nb % 4 == 0) && ((reinterpret_cast<uintptr_t>(scores) & 15) == 0);
   const PoolArgs pool{0, 1, 0, 1};
-#define NSA_TOPK(V) hipLaunchKernelGGL((topk_kernel<V>), grid, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, pool, idx, vals, fmask)
+  const TopkDyn dyn{nullptr, 1};
+#define NSA_TOPK(V) hipLaunchKernelGGL((topk_kernel<V, NSA_TOPK_POOL>), grid, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, pool, idx, vals, fmask, k, dyn)
 #define NSA_TOPK_DISPATCH()            \
   if (vpl <= 1) NSA_TOPK(1);           \
   else if (vpl <= 2) NSA_TOPK(2);      \
@@ -157,8 +191,13 @@ extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k
   return e == hipSuccess ? 0 : (int)e;
 }
 
-extern "C" int nsa_decode_topk(const float* logits, int32_t batch, int32_t kv_heads, int32_t group, int32_t num_compressed,
-                               int32_t per_block, int32_t share, int32_t k, int32_t* idx, float* vals, uint8_t* fmask, void* stream) {
+#undef NSA_TOPK_POOL
+#define NSA_TOPK_POOL true
+namespace nsa {
+// state == nullptr: num_compressed keys are cached; otherwise num_compressed is the capacity (row stride of the logits, upper bound of the
+// row length) and the count is read from state[1] when the kernel runs
+int decode_topk_launch(const float* logits, int32_t batch, int32_t kv_heads, int32_t group, int32_t num_compressed,
+                       int32_t per_block, int32_t share, int32_t k, int32_t* idx, float* vals, uint8_t* fmask, const int32_t* state, void* stream) {
   using namespace nsa;
   if (!logits || !idx || !vals || !fmask || batch <= 0 || kv_heads <= 0 || group <= 0 || per_block <= 0 || num_compressed <= 0) return NSA_E_ARG;
   const int nb = num_compressed / per_block;
@@ -172,9 +211,17 @@ extern "C" int nsa_decode_topk(const float* logits, int32_t batch, int32_t kv_he
   const int vec4 = 0, apply_softmax = 1;
   const float* scores = logits;
   const PoolArgs pool{share ? group : 1, per_block, num_compressed, units};
+  const TopkDyn dyn{state, per_block};
   NSA_TOPK_DISPATCH();
 #undef NSA_TOPK_DISPATCH
 #undef NSA_TOPK
+#undef NSA_TOPK_POOL
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
+}
+}  // namespace nsa
+
+extern "C" int nsa_decode_topk(const float* logits, int32_t batch, int32_t kv_heads, int32_t group, int32_t num_compressed,
+                               int32_t per_block, int32_t share, int32_t k, int32_t* idx, float* vals, uint8_t* fmask, void* stream) {
+  return nsa::decode_topk_launch(logits, batch, kv_heads, group, num_compressed, per_block, share, k, idx, vals, fmask, nullptr, stream);
 }

@@ -1,0 +1,172 @@
+"""Decode steps of one `SparseAttention` layer replayed from a captured HIP graph.
+
+`SparseAttention.forward_inference` (NSA.py:338-547) derives every shape of a step on the host and
+issues about a dozen launches; at small batch the host-side work is several times the kernels' run
+time.  A `DecodeSession` owns fixed-capacity caches, keeps the token position and the number of
+compressed keys in device memory (the kernels read them when they run, `nsa_decode_step_dyn`) and
+records norm, projections, the attention step and the output projection once into a HIP graph that is
+replayed for every token.  Only the compression of a completed window (every
+`compress_block_sliding_stride` tokens, NSA.py:422-441) runs outside the graph.
+
+    out, cache = attn(prompt, return_cache=True)           # prefill, as in the reference
+    session = DecodeSession(attn, cache, max_len=65536)
+    for x in tokens:                                         # x: 'b 1 dim'
+        y = session.step(x)
+    cache = session.cache()                                  # back to the module's cache format
+
+The reference has no counterpart; results equal `forward_inference` up to the order in which split
+partial results are merged (the split is sized for the capacity rather than the current length).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+
+_BF16 = torch.bfloat16
+
+
+class DecodeSession:
+    def __init__(self, module, cache, max_len: int):
+        m = self.module = module
+        assert m.causal, 'inference only relevant for autoregressive'
+        (cache_k, cache_v), ((cache_ck, cache_cv), (run_k, run_v)) = cache
+        if not cache_k.is_cuda:
+            raise RuntimeError("DecodeSession runs on the GPU only (HIP kernels, no CPU fallback)")
+        if m.to_qkv.weight.dtype != _BF16:
+            raise NotImplementedError("DecodeSession needs a bf16 module (the raw key / value window is kept in bf16)")
+        dev = cache_k.device
+        b, hk, t, d = cache_k.shape
+        st, cbs = m.compress_block_sliding_stride, m.compress_block_size
+        nc = cache_ck.shape[-2]
+        if max_len <= t:
+            raise ValueError(f"max_len {max_len} leaves no room after the {t} cached tokens")
+        self.b, self.hk, self.hq, self.d = b, hk, m.heads, d
+        self.st, self.cbs, self.max_len = st, cbs, int(max_len)
+        self.pos, self.nc = t, nc                                   # host mirrors of the device state
+        self.max_nc = (max(self.max_len // st, nc, 1) + 7) // 8 * 8        # rows of 16-byte-aligned fp32 logits
+
+        def grown(src, rows):
+            buf = torch.zeros((b, hk, rows, d), dtype=_BF16, device=dev)
+            buf[:, :, :src.shape[-2]].copy_(src)
+            return buf
+        self.K, self.V = grown(cache_k, self.max_len), grown(cache_v, self.max_len)
+        self.CK, self.CV = grown(cache_ck, self.max_nc), grown(cache_cv, self.max_nc)
+
+        # raw (un-rotated) keys / values of the last tokens, position p in row p % ring; rows never written are zero, which is
+        # also what the window of the first compression steps holds for positions before the sequence start (NSA.py:866)
+        self.ring = R = 2 * cbs
+        self.ring_k = torch.zeros((b, hk, R, d), dtype=_BF16, device=dev)
+        self.ring_v = torch.zeros((b, hk, R, d), dtype=_BF16, device=dev)
+        lr = run_k.shape[-2]
+        if lr > R:
+            raise ValueError("the cache's open compression window is longer than two compression blocks")
+        if lr:
+            rows = torch.arange(t - lr, t, device=dev) % R
+            self.ring_k[:, :, rows] = run_k.to(_BF16)
+            self.ring_v[:, :, rows] = run_v.to(_BF16)
+        # window rows of a compression step whose first position is s (mod ring)
+        self.win_rows = (torch.arange(R, device=dev)[:, None] + torch.arange(cbs, device=dev)[None, :]) % R
+        self.state = torch.tensor([t, nc], dtype=torch.int32, device=dev)
+        self.mem_k = m.compress_mem_kv[0].detach().to(_BF16).contiguous()
+        self.mem_v = m.compress_mem_kv[1].detach().to(_BF16).contiguous()
+        self.freqs = m.rotary_emb.freqs.detach().to(torch.float32).contiguous()
+
+        # q, k, v and the strategy-gate logits come out of one GEMM: the gate projection's rows are appended to the qkv
+        # weight (a copy: the session does not follow later changes of the module's parameters), its bias is added where the
+        # logits are used
+        gate = m.to_strategy_combine[0]
+        pad = -3 * m.heads % 8                                      # rows of the GEMM output stay 16-byte aligned
+        self.w_cat = torch.cat((m.to_qkv.weight.detach(), gate.weight.detach().to(_BF16),
+                                torch.zeros((pad, m.to_qkv.in_features), dtype=_BF16, device=dev)), dim=0).contiguous()
+        self.gate_bias = gate.bias.detach().to(_BF16).contiguous() if gate.bias is not None else None
+        self.x_buf = torch.zeros((b, 1, m.to_qkv.in_features), dtype=_BF16, device=dev)
+        self._desc, self._ws = self._make_desc(dev)
+        # the libraries initialise themselves on first use (outside the capture); the warm-up step writes row `pos` of the
+        # caches, which the first real step overwrites, and leaves the position alone
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side), torch.no_grad():
+            for _ in range(2):
+                self._body(advance=0)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(self.graph):
+            self.out_buf = self._body(advance=1)
+
+    # ---------------------------------------------------------------------------------------
+
+    def _make_desc(self, dev):
+        m = self.module
+        dsc = _lib.DecodeStepDesc()
+        dsc.batch, dsc.heads, dsc.kv_heads, dsc.dim_head = self.b, self.hq, self.hk, self.d
+        dsc.pos, dsc.num_compressed = self.max_len - 1, self.max_nc
+        dsc.per_block, dsc.block = m.selection_block_size // self.st, m.selection_block_size
+        dsc.num_sel, dsc.share = m.num_selected_blocks, int(bool(m.query_heads_share_selected_kv))
+        dsc.window, dsc.scale = m.sliding_window_size, self.d ** -0.5
+        dsc.num_mem = self.mem_k.shape[-2]
+        dsc.kc_stride[:] = self.K.stride()[:3]
+        dsc.vc_stride[:] = self.V.stride()[:3]
+        dsc.ck_stride[:] = self.CK.stride()[:3]
+        dsc.cv_stride[:] = self.CV.stride()[:3]
+        dsc.krun_stride[:] = self.ring_k.stride()[:2]
+        dsc.vrun_stride[:] = self.ring_v.stride()[:2]
+        # q / k / v are views of the qkv projection's output: 'b 1 (h d)' -> strides {row, head}
+        width = self.w_cat.shape[0]
+        for name in ("q_stride", "k_stride", "v_stride"):
+            getattr(dsc, name)[:] = (width, self.d)
+        nbytes = C.c_size_t()
+        _lib.check(_lib.lib().nsa_decode_step_workspace_bytes(C.byref(dsc), C.byref(nbytes), None, None, None),
+                   "nsa_decode_step_workspace_bytes")
+        return dsc, torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+
+    def _body(self, advance: int):
+        m = self.module
+        x = m.norm(self.x_buf)
+        qkvg = torch.nn.functional.linear(x, self.w_cat)             # 'b 1 ((hq + 2 hk) d + 3 hq)', contiguous
+        hq, hk, d = self.hq, self.hk, self.d
+        merged = torch.empty((self.b, 1, hq * d), dtype=_BF16, device=x.device)
+        p = qkvg.data_ptr()
+        _lib.check(_lib.lib().nsa_decode_step_dyn(
+            C.byref(self._desc), self.state.data_ptr(), p, p + 2 * hq * d, p + 2 * (hq + hk) * d, self.freqs.data_ptr(),
+            self.K.data_ptr(), self.V.data_ptr(), self.CK.data_ptr(), self.CV.data_ptr(), self.mem_k.data_ptr(), self.mem_v.data_ptr(),
+            self.ring_k.data_ptr(), self.ring_v.data_ptr(), self.ring_k.stride(2), self.ring_v.stride(2), self.ring,
+            p + 2 * (hq + 2 * hk) * d, qkvg.shape[-1], self.gate_bias.data_ptr() if self.gate_bias is not None else None,
+            self._ws.data_ptr(), self._ws.numel(), merged.data_ptr(), int(advance),
+            torch.cuda.current_stream(x.device).cuda_stream), "nsa_decode_step_dyn")
+        return m.combine_heads(merged)
+
+    @torch.no_grad()
+    def step(self, x: torch.Tensor) -> torch.Tensor:
+        """x 'b 1 dim': the token at position `self.pos`.  Returns the layer output 'b 1 dim' (a new tensor)."""
+        if self.pos >= self.max_len:
+            raise RuntimeError(f"DecodeSession: capacity of {self.max_len} tokens reached")
+        m, st, cbs = self.module, self.st, self.cbs
+        self.x_buf.copy_(x)
+        self.graph.replay()
+        out = self.out_buf.clone()
+        # a compression window is complete: compress it into the next compressed key / value (NSA.py:422-441)
+        if (self.pos + 1) % st == 0 and self.nc < self.max_nc:
+            rows = self.win_rows[(self.pos + 1 - cbs) % self.ring]
+            wk = self.ring_k.index_select(2, rows)
+            wv = self.ring_v.index_select(2, rows)
+            self.CK[:, :, self.nc:self.nc + 1].copy_(m.k_compress((wk + m.k_intrablock_positions)[:, :, None]))
+            self.CV[:, :, self.nc:self.nc + 1].copy_(m.v_compress((wv + m.v_intrablock_positions)[:, :, None]))
+            self.nc += 1
+            self.state[1:2].add_(1)
+        self.pos += 1
+        return out
+
+    def cache(self):
+        """The caches in the module's format `((k, v), ((ck, cv), (run_k, run_v)))` (copies of the filled parts)."""
+        t, st, cbs = self.pos, self.st, self.cbs
+        first = (t // st) * st - (cbs - st)                          # first position of the open window
+        rows = torch.arange(first, t, device=self.K.device) % self.ring
+        run_k, run_v = self.ring_k.index_select(2, rows), self.ring_v.index_select(2, rows)
+        if first < 0:                                                # positions before the sequence start read as zero
+            run_k[:, :, :-first] = 0
+            run_v[:, :, :-first] = 0
+        return ((self.K[:, :, :t].clone(), self.V[:, :, :t].clone()),
+                ((self.CK[:, :, :self.nc].clone(), self.CV[:, :, :self.nc].clone()), (run_k, run_v)))

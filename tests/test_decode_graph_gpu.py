@@ -1,0 +1,75 @@
+"""DecodeSession (decode steps replayed from a captured HIP graph, lengths read from device memory)
+against the module's eager decode step, replay by replay: the outputs within the bf16 forward
+tolerance (the two split the key range differently), the caches bit-equal."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+CONFIGS = [
+    # dim, d, heads, kv, win, cbs, st, B, S, share, prefill, steps
+    (256, 64, 4, 2, 16, 8, 4, 8, 2, True, 37, 45),
+    (256, 128, 2, 1, 32, 16, 8, 16, 3, True, 70, 40),
+    (256, 64, 4, 2, 8, 8, 8, 8, 4, False, 21, 30),        # stride == block, selection per query head
+    (128, 64, 2, 2, 16, 8, 4, 8, 2, True, 2, 40),         # starts before the first compressed key exists
+]
+
+
+@pytest.mark.parametrize("cfg", CONFIGS)
+def test_graph_decode_matches_eager_decode(cfg):
+    from native_sparse_attention_pytorch_amd import SparseAttention
+    from native_sparse_attention_pytorch_amd.decode_session import DecodeSession
+    from tests.util import assert_close
+    dim, d, heads, kv, win, cbs, st, B, S, share, n0, steps = cfg
+    print("graph decode", cfg, flush=True)
+    torch.manual_seed(sum(cfg[:9]))
+    m = SparseAttention(dim=dim, dim_head=d, heads=heads, kv_heads=kv, sliding_window_size=win, compress_block_size=cbs,
+                        compress_block_sliding_stride=st, selection_block_size=B, num_selected_blocks=S, causal=True,
+                        query_heads_share_selected_kv=share).to(DEV).bfloat16()
+    with torch.no_grad():                                          # the gate and memory parameters start at constants
+        m.compress_mem_kv.normal_(std=0.5)
+        m.k_intrablock_positions.normal_(std=0.2)
+        m.v_intrablock_positions.normal_(std=0.2)
+        m.to_strategy_combine[0].weight.normal_(std=0.05)
+    b = 2
+    xs = torch.randn(b, n0 + steps, dim, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        _, cache = m(xs[:, :n0], return_cache=True)
+    sess = DecodeSession(m, cache, max_len=n0 + steps + 5)
+    for i in range(steps):
+        x = xs[:, n0 + i:n0 + i + 1]
+        with torch.no_grad():
+            want, cache = m(x, cache=cache, return_cache=True)
+        got = sess.step(x)
+        torch.cuda.synchronize()
+        assert_close(got, want, 2e-2, 1e-2, f"step {i}")
+    (k, v), ((ck, cv), (rk, rv)) = sess.cache()
+    (k2, v2), ((ck2, cv2), (rk2, rv2)) = cache
+    assert torch.equal(k, k2) and torch.equal(v, v2)
+    assert ck.shape == ck2.shape and torch.equal(ck, ck2.to(ck.dtype)) and torch.equal(cv, cv2.to(cv.dtype))
+    assert rk.shape == rk2.shape and torch.equal(rk, rk2.to(rk.dtype)) and torch.equal(rv, rv2.to(rv.dtype))
+    # and back: the module continues from the session's caches
+    x = torch.randn(b, 1, dim, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        a, _ = m(x, cache=sess.cache(), return_cache=True)
+        bb, _ = m(x, cache=cache, return_cache=True)
+    assert torch.equal(a, bb)
+
+
+def test_graph_decode_capacity_is_enforced():
+    from native_sparse_attention_pytorch_amd import SparseAttention
+    from native_sparse_attention_pytorch_amd.decode_session import DecodeSession
+    torch.manual_seed(0)
+    m = SparseAttention(dim=128, dim_head=64, heads=2, kv_heads=1, sliding_window_size=8, compress_block_size=8,
+                        compress_block_sliding_stride=4, selection_block_size=8, num_selected_blocks=2, causal=True).to(DEV).bfloat16()
+    x = torch.randn(1, 12, 128, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        _, cache = m(x, return_cache=True)
+    with pytest.raises(ValueError):
+        DecodeSession(m, cache, max_len=12)
+    sess = DecodeSession(m, cache, max_len=14)
+    sess.step(x[:, :1])
+    sess.step(x[:, :1])
+    with pytest.raises(RuntimeError):
+        sess.step(x[:, :1])
