@@ -154,27 +154,41 @@ __global__ __launch_bounds__(64) void sel_fill_kernel(const SelPlan P, const voi
   const int q0 = c * kCountChunk;
   const int nq = min(kCountChunk, P.n - q0);
   const int total = nq * P.S;
+  if (total <= 0) return;
+  // the slot mask and block index of an entry are fetched two rounds ahead of their use (branch-free, from a clamped
+  // position): a round is otherwise one dependent global load long
+  struct Fetched { int live, j; };
+  auto fetch = [&](int e0) {
+    const int e = min(e0 + lane, total - 1);
+    const size_t pos = ((size_t)bh * P.n + q0) * P.S + e;
+    Fetched f;
+    f.live = fmask[pos];
+    f.j = read_idx(idx, P.idx64, pos);
+    return f;
+  };
+  Fetched f0 = fetch(0), f1 = fetch(64);
+  const int nbits = 32 - __builtin_clz((unsigned)max(P.W - 1, 1));      // bits of a block index
   for (int e0 = 0; e0 < total; e0 += 64) {
+    const Fetched cur = f0;
+    f0 = f1;
+    f1 = fetch(e0 + 128);
     const int e = e0 + lane;
     int j = -1, entry = 0;
-    if (e < total) {
-      const int qi = q0 + e / P.S, s = e % P.S;
-      const size_t pos = ((size_t)bh * P.n + qi) * P.S + s;
-      if (fmask[pos]) {
-        j = read_idx(idx, P.idx64, pos);
-        if (j >= P.W) j = -1;
-        entry = qi * P.SP + s;
-      }
+    if (e < total && cur.live) {
+      j = cur.j;
+      if (j >= P.W) j = -1;
+      entry = (q0 + e / P.S) * P.SP + e % P.S;
     }
-    const int key = (j >= 0) ? j : (-1 - lane);      // dead lanes never match anything
-    int rank = 0, same = 0;
-#pragma unroll
-    for (int t = 0; t < 64; ++t) {
-      const int kt = __builtin_amdgcn_readlane(key, t);
-      const int eq = (kt == key) ? 1 : 0;
-      rank += (t < lane) ? eq : 0;
-      same += eq;
+    // lanes of this round that name the same block: intersect, bit by bit of the block index, the ballots of the lanes
+    // that agree with this lane (about 10 ballots instead of 64 lane reads); dead lanes are masked out
+    unsigned long long same_m = __ballot(j >= 0);
+    for (int bit = 0; bit < nbits; ++bit) {
+      const bool one = (j >> bit) & 1;
+      const unsigned long long bal = __ballot(one);
+      same_m &= one ? bal : ~bal;
     }
+    const int rank = __popcll(same_m & ((1ull << lane) - 1ull));
+    const int same = __popcll(same_m);
     if (j >= 0) list[base[j] + rank] = entry;
     __syncthreads();
     if (j >= 0 && rank == same - 1) base[j] += same;

@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in,
       for (int r4 = 0; r4 < VPL / 4; ++r4) {
         const int j = lane * VPL + 4 * r4;
         floatx4 t = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-        if (j < nb) t = *reinterpret_cast<const floatx4*>(src + j);
+        if (j < nb) t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(src + j));      // read once
 #pragma unroll
         for (int e = 0; e < 4; ++e) x[4 * r4 + e] = t[e];
       }
