@@ -147,8 +147,8 @@ __global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_
     for (int r = 0; r < NI; ++r) {
       const int row = RPI * r + lr;
       const long rc = row < T.nvalid ? row : 0;
-      kr[r] = load8(T.kb + rc * T.ks + 8 * lc);
-      vr[r] = load8(T.vb + rc * T.vs + 8 * lc);
+      kr[r] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(T.kb + rc * T.ks + 8 * lc));      // every cached row is read once per step
+      vr[r] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(T.vb + rc * T.vs + 8 * lc));
     }
   };
   auto next_tile = [&](int t, DecodeTile& T) {
