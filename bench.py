@@ -330,6 +330,33 @@ def main():
     except Exception as ex:
         res["train_config5"] = dict(error=repr(ex))
 
+    # generation with the same model in bf16: greedy sampling from a 128-token prompt to 384 tokens, batch 8, through the
+    # per-layer caches - launched step by step, and replayed from a captured whole-model HIP graph
+    try:
+        if args.headline_only:
+            raise _Skip()
+        from native_sparse_attention_pytorch_amd.transformer import Transformer
+        torch.manual_seed(0)
+        model = Transformer(num_tokens=256, dim=512, depth=6, dim_head=64, heads=8, kv_heads=4,
+                            sparse_attn_kwargs=dict(sliding_window_size=64, compress_block_size=16, compress_block_sliding_stride=8,
+                                                    selection_block_size=16, num_selected_blocks=4)).to(dev).bfloat16()
+        prompt = torch.randint(0, 256, (8, 128), device=dev)
+        gen = {}
+        for name, kw in (("cached", dict(use_cache_kv=True)), ("graph", dict(use_cache_kv=True, use_graph=True))):
+            model.sample(prompt, 160, temperature=0., **kw)          # warm-up (and one-time library initialisation)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            new = model.sample(prompt, 384, temperature=0., **kw)
+            torch.cuda.synchronize()
+            tg = time.perf_counter() - t0
+            gen[name] = dict(ms_per_token=round(tg / new.shape[1] * 1e3, 3), tokens_per_s=round(new.numel() / tg, 1))
+        res["generate_config5_bf16"] = gen
+        del model
+    except _Skip:
+        pass
+    except Exception as ex:
+        res["generate_config5_bf16"] = dict(error=repr(ex))
+
     if not args.no_cpu:
         torch.set_num_threads(min(16, os.cpu_count() or 1))
         base, ref = cpu_baseline(cfg, q, k, v, do, idx, msk)

@@ -1,12 +1,14 @@
-"""Decode steps of one `SparseAttention` layer replayed from a captured HIP graph.
+"""Decode steps replayed from captured HIP graphs: `DecodeSession` for one `SparseAttention` layer,
+`TransformerDecodeSession` for the whole `Transformer`.
 
 `SparseAttention.forward_inference` (NSA.py:338-547) derives every shape of a step on the host and
 issues about a dozen launches; at small batch the host-side work is several times the kernels' run
 time.  A `DecodeSession` owns fixed-capacity caches, keeps the token position and the number of
 compressed keys in device memory (the kernels read them when they run, `nsa_decode_step_dyn`) and
-records norm, projections, the attention step and the output projection once into a HIP graph that is
-replayed for every token.  Only the compression of a completed window (every
-`compress_block_sliding_stride` tokens, NSA.py:422-441) runs outside the graph.
+records norm, projections, the attention step and the output projection into a HIP graph that is
+replayed for every token.  Every `compress_block_sliding_stride` tokens a compression window is
+complete (NSA.py:422-441); those steps replay a second graph that also gathers the window (rows
+indexed from the device-side position), compresses it and appends the compressed key / value.
 
     out, cache = attn(prompt, return_cache=True)           # prefill, as in the reference
     session = DecodeSession(attn, cache, max_len=65536)
@@ -29,7 +31,7 @@ _BF16 = torch.bfloat16
 
 
 class DecodeSession:
-    def __init__(self, module, cache, max_len: int):
+    def __init__(self, module, cache, max_len: int, capture: bool = True):
         m = self.module = module
         assert m.causal, 'inference only relevant for autoregressive'
         (cache_k, cache_v), ((cache_ck, cache_cv), (run_k, run_v)) = cache
@@ -67,8 +69,7 @@ class DecodeSession:
             rows = torch.arange(t - lr, t, device=dev) % R
             self.ring_k[:, :, rows] = run_k.to(_BF16)
             self.ring_v[:, :, rows] = run_v.to(_BF16)
-        # window rows of a compression step whose first position is s (mod ring)
-        self.win_rows = (torch.arange(R, device=dev)[:, None] + torch.arange(cbs, device=dev)[None, :]) % R
+        self._ar = torch.arange(cbs, device=dev, dtype=torch.int32)
         self.state = torch.tensor([t, nc], dtype=torch.int32, device=dev)
         self.mem_k = m.compress_mem_kv[0].detach().to(_BF16).contiguous()
         self.mem_v = m.compress_mem_kv[1].detach().to(_BF16).contiguous()
@@ -84,17 +85,26 @@ class DecodeSession:
         self.gate_bias = gate.bias.detach().to(_BF16).contiguous() if gate.bias is not None else None
         self.x_buf = torch.zeros((b, 1, m.to_qkv.in_features), dtype=_BF16, device=dev)
         self._desc, self._ws = self._make_desc(dev)
-        # the libraries initialise themselves on first use (outside the capture); the warm-up step writes row `pos` of the
-        # caches, which the first real step overwrites, and leaves the position alone
-        side = torch.cuda.Stream(device=dev)
-        side.wait_stream(torch.cuda.current_stream(dev))
-        with torch.cuda.stream(side), torch.no_grad():
-            for _ in range(2):
-                self._body(advance=0)
-        torch.cuda.current_stream(dev).wait_stream(side)
-        self.graph = torch.cuda.CUDAGraph()
-        with torch.no_grad(), torch.cuda.graph(self.graph):
-            self.out_buf = self._body(advance=1)
+        self.graphs = None
+        if capture:
+            # the libraries initialise themselves on first use (outside the capture); the warm-up steps write row `pos` of
+            # the caches and row `nc` of the compressed caches, which the first real steps overwrite, and leave both counters alone
+            side = torch.cuda.Stream(device=dev)
+            side.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(side), torch.no_grad():
+                for _ in range(2):
+                    self.layer_step(self.x_buf, advance=0)
+                    self.compress_window(count=False)
+            torch.cuda.current_stream(dev).wait_stream(side)
+            self.graphs, self.outs = [], []
+            for event in (False, True):                             # [0]: ordinary step, [1]: step that completes a window
+                g = torch.cuda.CUDAGraph()
+                with torch.no_grad(), torch.cuda.graph(g):
+                    out = self.layer_step(self.x_buf, advance=1)
+                    if event:
+                        self.compress_window()
+                self.graphs.append(g)
+                self.outs.append(out)
 
     # ---------------------------------------------------------------------------------------
 
@@ -122,9 +132,11 @@ class DecodeSession:
                    "nsa_decode_step_workspace_bytes")
         return dsc, torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
 
-    def _body(self, advance: int):
+    def layer_step(self, x_in: torch.Tensor, advance: int):
+        """The layer's decode step on `x_in` 'b 1 dim' as a sequence of launches with no host-side dependence on the
+        position (recordable into a graph); advance != 0 increments the device-side position afterwards."""
         m = self.module
-        x = m.norm(self.x_buf)
+        x = m.norm(x_in)
         qkvg = torch.nn.functional.linear(x, self.w_cat)             # 'b 1 ((hq + 2 hk) d + 3 hq)', contiguous
         hq, hk, d = self.hq, self.hk, self.d
         merged = torch.empty((self.b, 1, hq * d), dtype=_BF16, device=x.device)
@@ -138,26 +150,40 @@ class DecodeSession:
             torch.cuda.current_stream(x.device).cuda_stream), "nsa_decode_step_dyn")
         return m.combine_heads(merged)
 
+    def compress_window(self, count: bool = True):
+        """Compress the window that ends at the device-side position (already advanced past the newest token) and append it
+        to the compressed caches (NSA.py:422-441); every index comes from device memory."""
+        m = self.module
+        rows = torch.remainder(self.state[0] - self.cbs + self._ar, self.ring)
+        wk = self.ring_k.index_select(2, rows)
+        wv = self.ring_v.index_select(2, rows)
+        at = self.state[1:2].long()
+        self.CK.index_copy_(2, at, m.k_compress((wk + m.k_intrablock_positions)[:, :, None]).to(_BF16))
+        self.CV.index_copy_(2, at, m.v_compress((wv + m.v_intrablock_positions)[:, :, None]).to(_BF16))
+        if count:
+            self.state[1:2].add_(1)
+
+    def completes_window(self) -> bool:
+        """Whether the token at the current position completes a compression window."""
+        return (self.pos + 1) % self.st == 0 and self.nc < self.max_nc
+
+    def advance_host(self, event: bool):
+        """Follow on the host what a replayed step did to the device-side counters."""
+        self.pos += 1
+        self.nc += int(event)
+
     @torch.no_grad()
     def step(self, x: torch.Tensor) -> torch.Tensor:
         """x 'b 1 dim': the token at position `self.pos`.  Returns the layer output 'b 1 dim' (a new tensor)."""
+        if self.graphs is None:
+            raise RuntimeError("DecodeSession was built with capture=False (its launches belong to an enclosing graph)")
         if self.pos >= self.max_len:
             raise RuntimeError(f"DecodeSession: capacity of {self.max_len} tokens reached")
-        m, st, cbs = self.module, self.st, self.cbs
+        event = self.completes_window()
         self.x_buf.copy_(x)
-        self.graph.replay()
-        out = self.out_buf.clone()
-        # a compression window is complete: compress it into the next compressed key / value (NSA.py:422-441)
-        if (self.pos + 1) % st == 0 and self.nc < self.max_nc:
-            rows = self.win_rows[(self.pos + 1 - cbs) % self.ring]
-            wk = self.ring_k.index_select(2, rows)
-            wv = self.ring_v.index_select(2, rows)
-            self.CK[:, :, self.nc:self.nc + 1].copy_(m.k_compress((wk + m.k_intrablock_positions)[:, :, None]))
-            self.CV[:, :, self.nc:self.nc + 1].copy_(m.v_compress((wv + m.v_intrablock_positions)[:, :, None]))
-            self.nc += 1
-            self.state[1:2].add_(1)
-        self.pos += 1
-        return out
+        self.graphs[event].replay()
+        self.advance_host(event)
+        return self.outs[event].clone()
 
     def cache(self):
         """The caches in the module's format `((k, v), ((ck, cv), (run_k, run_v)))` (copies of the filled parts)."""
@@ -170,3 +196,57 @@ class DecodeSession:
             run_v[:, :, :-first] = 0
         return ((self.K[:, :, :t].clone(), self.V[:, :, :t].clone()),
                 ((self.CK[:, :, :self.nc].clone(), self.CV[:, :, :self.nc].clone()), (run_k, run_v)))
+
+
+class TransformerDecodeSession:
+    """Token-by-token decoding of a `Transformer` (transformer.py:213-252 with use_cache_kv) as one graph replay per
+    token: embedding, every layer's attention step and feed-forward, final norm and logits.  `caches` is what
+    `model(prompt, return_cache=True)` returned; `max_len` the longest sequence to decode to."""
+
+    def __init__(self, model, caches, max_len: int):
+        self.model = model
+        dev = caches[0][0][0].device
+        b = caches[0][0][0].shape[0]
+        self.layers = [DecodeSession(attn, cache, max_len, capture=False) for (attn, _), cache in zip(model.layers, caches)]
+        self.tok = torch.zeros((b, 1), dtype=torch.long, device=dev)
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side), torch.no_grad():
+            for _ in range(2):
+                self._body(advance=0, event=True, count=False)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        self.graphs, self.outs = [], []
+        for event in (False, True):
+            g = torch.cuda.CUDAGraph()
+            with torch.no_grad(), torch.cuda.graph(g):
+                out = self._body(advance=1, event=event, count=True)
+            self.graphs.append(g)
+            self.outs.append(out)
+
+    def _body(self, advance: int, event: bool, count: bool):
+        model = self.model
+        x = model.token_emb(self.tok)
+        for sess, (_, ff) in zip(self.layers, model.layers):
+            a = sess.layer_step(x, advance)
+            if event:
+                sess.compress_window(count)
+            x = a + x
+            x = ff(x) + x
+        return model.to_logits(model.norm(x))
+
+    @property
+    def pos(self) -> int:
+        return self.layers[0].pos
+
+    @torch.no_grad()
+    def step(self, token: torch.Tensor) -> torch.Tensor:
+        """token 'b' or 'b 1' (int64): the token at the current position.  Returns the logits 'b 1 vocab' for the next one."""
+        first = self.layers[0]
+        if first.pos >= first.max_len:
+            raise RuntimeError(f"TransformerDecodeSession: capacity of {first.max_len} tokens reached")
+        event = first.completes_window()
+        self.tok.copy_(token.reshape(self.tok.shape))
+        self.graphs[event].replay()
+        for sess in self.layers:
+            sess.advance_host(event)
+        return self.outs[event].clone()

@@ -63,15 +63,23 @@ class Transformer(nn.Module):
 
 
     @torch.no_grad()
-    def sample(self, prompt, seq_len, temperature=1., filter_thres=0.9, use_cache_kv=False):
+    def sample(self, prompt, seq_len, temperature=1., filter_thres=0.9, use_cache_kv=False, use_graph=False):
         """Extend `prompt` to seq_len tokens and return the new ones (transformer.py:213-252).
         temperature <= 0 is greedy; otherwise gumbel sampling over the top (1 - filter_thres)
-        share of the vocabulary.  With use_cache_kv every step after the first is a decode step."""
-        out, cache = prompt.clone(), None
+        share of the vocabulary.  With use_cache_kv every step after the first is a decode step;
+        use_graph (with use_cache_kv, bf16 models) replays those steps from a captured HIP graph
+        (decode_session.TransformerDecodeSession) instead of launching them one by one."""
+        out, cache, session = prompt.clone(), None, None
         for _ in range(max(0, seq_len - prompt.shape[-1])):
-            logits, next_cache = self.forward(out, cache=cache, return_cache=True)
-            if use_cache_kv:
-                cache = next_cache
+            if session is not None:
+                logits = session.step(out[:, -1:])
+            else:
+                logits, next_cache = self.forward(out, cache=cache, return_cache=True)
+                if use_cache_kv:
+                    cache = next_cache
+                    if use_graph:
+                        from .decode_session import TransformerDecodeSession
+                        session = TransformerDecodeSession(self, cache, max_len=seq_len)
             logits = logits[:, -1].float()
             if temperature <= 0.:
                 tok = logits.argmax(dim=-1, keepdim=True)
