@@ -13,6 +13,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # never let the compiler form packed-fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results in ordinary vector registers: the walks' accumulators feed VALU code (softmax, scaling, stores), and from
+    # accumulation registers every element would first need a copy instruction (a sixth of the forward walk's VALU work)
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
 
 
