@@ -108,7 +108,16 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="only the headline workload (for profiler runs): no compressed-branch, module or decode legs")
+    ap.add_argument("--skip", default="", help="comma-separated legs to leave out: compressed, module, decode, train, generate")
     args = ap.parse_args()
+    skip = set(filter(None, args.skip.split(","))) | ({"compressed", "module", "decode", "train", "generate"} if args.headline_only else set())
+
+    def leg(name):
+        """Announce a leg on stderr (a long profiler run must not look hung) or skip it."""
+        if name in skip:
+            raise _Skip()
+        print(f"bench.py: {name} leg", file=sys.stderr, flush=True)
+
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
         sys.exit(2)
@@ -196,8 +205,7 @@ def main():
     # the other half of BASELINE configs[3]: compressed attention with fused importance logits +
     # top-k over 2048 compressed keys (+1 memory slot), forward and backward, reported beside the headline
     try:
-        if args.headline_only:
-            raise _Skip()
+        leg("compressed")
         g2 = torch.Generator(device=dev).manual_seed(1)
         nc = n // 16
         ck = (torch.randn(b, hk, nc + 1, d, generator=g2, device=dev) * d ** -0.5).to(torch.bfloat16).requires_grad_()
@@ -228,8 +236,7 @@ def main():
     # module (BASELINE configs[2]: b4 n4096 dim1024, forward + backward) and one decode step of a
     # configs[3]-sized layer over a 32k-token cache
     try:
-        if args.headline_only:
-            raise _Skip()
+        leg("module")
         from native_sparse_attention_pytorch_amd import SparseAttention
         torch.manual_seed(0)
         mod = SparseAttention(dim=1024, dim_head=64, heads=16, kv_heads=4, sliding_window_size=512, compress_block_size=32,
@@ -251,8 +258,7 @@ def main():
     except Exception as ex:
         res["module_config3"] = dict(error=repr(ex))
     try:
-        if args.headline_only:
-            raise _Skip()
+        leg("decode")
         from native_sparse_attention_pytorch_amd import SparseAttention
         torch.manual_seed(0)
         ctx = 32768
@@ -298,8 +304,7 @@ def main():
     # BASELINE configs[4]: end-to-end training step of the small NSA transformer on byte tokens
     # (depth 6, dim 512, 8/4 heads, batch 8 x 1024 tokens; fp32 master weights, bf16 autocast, Adam)
     try:
-        if args.headline_only:
-            raise _Skip()
+        leg("train")
         from native_sparse_attention_pytorch_amd.transformer import Transformer
         torch.manual_seed(0)
         model = Transformer(num_tokens=256, dim=512, depth=6, dim_head=64, heads=8, kv_heads=4,
@@ -333,8 +338,7 @@ def main():
     # generation with the same model in bf16: greedy sampling from a 128-token prompt to 384 tokens, batch 8, through the
     # per-layer caches - launched step by step, and replayed from a captured whole-model HIP graph
     try:
-        if args.headline_only:
-            raise _Skip()
+        leg("generate")
         from native_sparse_attention_pytorch_amd.transformer import Transformer
         torch.manual_seed(0)
         model = Transformer(num_tokens=256, dim=512, depth=6, dim_head=64, heads=8, kv_heads=4,
