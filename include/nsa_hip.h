@@ -243,7 +243,8 @@ int nsa_decode_step(const nsa_decode_step_desc* desc, const void* q, const void*
  * krun_row_stride / vrun_row_stride; the un-rotated key / value of the new token go to row state[0] % run_ring.
  * gate_logits: bf16, row b at gate_logits + b * gate_row_stride (0: rows are contiguous), gate_bias (optional, bf16
  * [3 * heads]) is added to them - so the gate projection can be columns of the same GEMM as q, k, v.
- * advance != 0: the call's last kernel adds 1 to state[0].  The call neither allocates nor synchronises. */
+ * advance != 0: the call's last kernel adds 1 to state[0].  Counters beyond the capacities are clamped (a step replayed
+ * past the last cache row writes nothing).  The call neither allocates nor synchronises. */
 int nsa_decode_step_dyn(const nsa_decode_step_desc* capacity, int32_t* state, const void* q, const void* k, const void* v,
                         const float* freqs, void* k_cache, void* v_cache, const void* ck_cache, const void* cv_cache,
                         const void* mem_k, const void* mem_v, void* k_run, void* v_run, int64_t krun_row_stride,

@@ -35,11 +35,13 @@ struct DecodePlan {
   const int* dyn;
   int dyn_kind;                      // 1 compressed range, 2 selected blocks, 3 sliding window
   int window, per_block, smax;
+  int cap_len, cap_nc;               // rows the key / value caches and the compressed caches hold: the counters are clamped to them
 };
 
 __device__ __forceinline__ void resolve(DecodePlan& P) {
   if (P.dyn == nullptr) return;
-  const int kv_len = P.dyn[0] + 1, nc = P.dyn[1];
+  // a caller that replays the step more often than the caches have rows must not make the kernels read or write past them
+  const int kv_len = min(max(P.dyn[0], 0) + 1, P.cap_len), nc = min(max(P.dyn[1], 0), P.cap_nc);
   if (P.dyn_kind == 1) {
     P.count = nc;
     if (nc == 0) P.mem = 0;                            // no compressed key yet: the branch contributes nothing (NSA.py:401)
@@ -576,7 +578,7 @@ namespace nsa {
 int decode_prep_dyn(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v, const int64_t* v_stride,
                     int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head, const float* freqs, void* rq, void* k_cache,
                     const int64_t* kc_stride, void* v_cache, const int64_t* vc_stride, void* k_run, const int64_t* krun_stride, void* v_run,
-                    const int64_t* vrun_stride, int32_t ring, const int32_t* state, void* stream);
+                    const int64_t* vrun_stride, int32_t ring, int32_t last_pos, const int32_t* state, void* stream);
 int decode_topk_launch(const float* logits, int32_t batch, int32_t kv_heads, int32_t group, int32_t num_compressed, int32_t per_block,
                        int32_t share, int32_t k, int32_t* idx, float* vals, uint8_t* fmask, const int32_t* state, void* stream);
 }  // namespace nsa
@@ -602,6 +604,7 @@ extern "C" int nsa_decode_step_dyn(const nsa_decode_step_desc* cap, int32_t* sta
   for (DecodePlan* P : {&Pc, &Pf, &Ps}) {
     P->dyn = state; P->dyn_kind = kind++;
     P->window = cap->window; P->per_block = cap->per_block; P->smax = L.k;
+    P->cap_len = cap->pos + 1; P->cap_nc = cap->num_compressed;
   }
   Pc.lstride = cap->num_compressed;
   Pf.sstride = L.k;
@@ -611,7 +614,7 @@ extern "C" int nsa_decode_step_dyn(const nsa_decode_step_desc* cap, int32_t* sta
   const int64_t krun_s[3] = {cap->krun_stride[0], cap->krun_stride[1], krun_row_stride};
   const int64_t vrun_s[3] = {cap->vrun_stride[0], cap->vrun_stride[1], vrun_row_stride};
   if (int e = decode_prep_dyn(q, cap->q_stride, k, cap->k_stride, v, cap->v_stride, cap->batch, cap->heads, cap->kv_heads, cap->dim_head, freqs, rq,
-                              k_cache, cap->kc_stride, v_cache, cap->vc_stride, k_run, krun_s, v_run, vrun_s, run_ring, state, stream))
+                              k_cache, cap->kc_stride, v_cache, cap->vc_stride, k_run, krun_s, v_run, vrun_s, run_ring, cap->pos, state, stream))
     return e;
   float* logits = (float*)(w + L.off_logits);
   if (has_c)

@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void rope_kernel(const __bf16* __restrict__ x,
 struct DecodeDyn {
   const int* state;
   long kc_row, vc_row, krun_row, vrun_row;
-  int ring;
+  int ring, last_pos;                // last_pos: the last row the caches have
 };
 
 // Decode step: the new token's query heads rotated to position pos (-> rq), its key heads
@@ -55,6 +55,7 @@ __global__ __launch_bounds__(256) void decode_prep_kernel(const __bf16* __restri
   if (dyn.state != nullptr) {
     // position read at run time (the launch is replayed from a graph): row pos of the caches, row pos % ring of the window rings
     pos = dyn.state[0];
+    if (pos < 0 || pos > dyn.last_pos) return;       // replayed past the caches' capacity: write nothing
     krow += (long)pos * dyn.kc_row;
     vrow += (long)pos * dyn.vc_row;
     if (krun != nullptr) {
@@ -139,9 +140,9 @@ int decode_prep_launch(const void* q, const int64_t* q_stride, const void* k, co
 int decode_prep_dyn(const void* q, const int64_t* q_stride, const void* k, const int64_t* k_stride, const void* v, const int64_t* v_stride,
                     int32_t batch, int32_t heads, int32_t kv_heads, int32_t dim_head, const float* freqs, void* rq, void* k_cache,
                     const int64_t* kc_stride, void* v_cache, const int64_t* vc_stride, void* k_run, const int64_t* krun_stride, void* v_run,
-                    const int64_t* vrun_stride, int32_t ring, const int32_t* state, void* stream) {
+                    const int64_t* vrun_stride, int32_t ring, int32_t last_pos, const int32_t* state, void* stream) {
   if (!state || !kc_stride || !vc_stride || ((kc_stride[2] | vc_stride[2]) & 7)) return NSA_E_ARG;
-  DecodeDyn dyn{state, (long)kc_stride[2], (long)vc_stride[2], 0, 0, 1};
+  DecodeDyn dyn{state, (long)kc_stride[2], (long)vc_stride[2], 0, 0, 1, last_pos};
   if (k_run || v_run) {
     if (!krun_stride || !vrun_stride || ring <= 0 || ((krun_stride[2] | vrun_stride[2]) & 7)) return NSA_E_ARG;
     dyn.krun_row = krun_stride[2]; dyn.vrun_row = vrun_stride[2]; dyn.ring = ring;
@@ -157,7 +158,7 @@ extern "C" int nsa_decode_prep(const void* q, const int64_t* q_stride, const voi
                                const int64_t* v_row_stride, void* k_run_row, const int64_t* k_run_stride, void* v_run_row,
                                const int64_t* v_run_stride, void* stream) {
   return nsa::decode_prep_launch(q, q_stride, k, k_stride, v, v_stride, batch, heads, kv_heads, dim_head, freqs, pos, rq, k_row, k_row_stride,
-                                 v_row, v_row_stride, k_run_row, k_run_stride, v_run_row, v_run_stride, nsa::DecodeDyn{nullptr, 0, 0, 0, 0, 1}, stream);
+                                 v_row, v_row_stride, k_run_row, k_run_stride, v_run_row, v_run_stride, nsa::DecodeDyn{nullptr, 0, 0, 0, 0, 1, 0}, stream);
 }
 
 extern "C" int nsa_rope(const void* x, const int64_t* x_stride, int32_t batch, int32_t heads, int32_t seq, int32_t dim_head,

@@ -73,6 +73,13 @@ def test_graph_decode_capacity_is_enforced():
     sess.step(x[:, :1])
     with pytest.raises(RuntimeError):
         sess.step(x[:, :1])
+    # a caller that replays the graph anyway finds the device-side counters clamped to the capacity: nothing is written
+    k_before, v_before = sess.K.clone(), sess.V.clone()
+    for _ in range(3):
+        sess.graphs[0].replay()
+    torch.cuda.synchronize()
+    assert torch.equal(sess.K, k_before) and torch.equal(sess.V, v_before)
+    assert int(sess.state[0]) == 17
 
 
 def test_transformer_graph_decode_matches_cached_decode():
