@@ -72,6 +72,11 @@ def select_fwd(q: Tensor, k: Tensor, v: Tensor, idx: Tensor, fmask: Tensor, sel_
     fm = fmask.contiguous().view(torch.uint8) if fmask.dtype == torch.bool else fmask.contiguous().to(torch.uint8)
     if idx.dtype not in (torch.int64, torch.int32):
         raise RuntimeError("selected_block_indices must be int64 or int32")
+    hk = k.shape[1]
+    if k.shape != (b, hk, n, d) or v.shape != k.shape or hq % hk:
+        raise RuntimeError(f"q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}: expected 'b hq n d' and 'b hk n d' with hk dividing hq")
+    if idx.dim() != 4 or idx.shape[:3] != (b, hk, n) or fm.shape != idx.shape or not idx.is_cuda or not fm.is_cuda:
+        raise RuntimeError(f"selected_block_indices {tuple(idx.shape)} / fmask {tuple(fm.shape)}: expected device tensors 'b hk n S' with hk = {hk}")
     out = torch.empty((b, hq, n, d), dtype=_BF16, device=q.device)
     lse = torch.empty((b, hq, n), dtype=torch.float32, device=q.device)
     dsc = _select_desc(q, k, v, out, idx.shape[-1], block, causal, scale, idx.dtype == torch.int64)
@@ -206,6 +211,8 @@ def dense_fwd(q: Tensor, k: Tensor, v: Tensor, mode: int, causal: bool, window: 
     q, k, v = _prep(q), _prep(k), _prep(v)
     b, hq, n, d = q.shape
     hk = k.shape[1]
+    if k.dim() != 4 or k.shape[0] != b or k.shape[3] != d or v.shape != k.shape or hq % hk or k.shape[2] < num_mem:
+        raise RuntimeError(f"q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}: expected 'b hq n d' and 'b hk keys d' with hk dividing hq")
     out = torch.empty((b, hq, n, d), dtype=_BF16, device=q.device)
     lse = torch.empty((b, hq, n), dtype=torch.float32, device=q.device)
     nb = 0
