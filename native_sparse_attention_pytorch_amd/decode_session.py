@@ -30,6 +30,13 @@ from . import _lib
 _BF16 = torch.bfloat16
 
 
+def ring_rows(first, count_range: torch.Tensor, ring: int) -> torch.Tensor:
+    """Rows of a position-indexed ring (position p lives in row p % ring) that hold positions first, first+1, ...:
+    `first` is an int or a 0-dim integer tensor (e.g. a device-side counter), `count_range` = arange(count).  Positions
+    before the sequence start map to rows that have not been written yet (ring >= count), i.e. to zeros."""
+    return torch.remainder(first + count_range, ring)
+
+
 class DecodeSession:
     def __init__(self, module, cache, max_len: int, capture: bool = True):
         m = self.module = module
@@ -66,7 +73,7 @@ class DecodeSession:
         if lr > R:
             raise ValueError("the cache's open compression window is longer than two compression blocks")
         if lr:
-            rows = torch.arange(t - lr, t, device=dev) % R
+            rows = ring_rows(t - lr, torch.arange(lr, device=dev), R)
             self.ring_k[:, :, rows] = run_k.to(_BF16)
             self.ring_v[:, :, rows] = run_v.to(_BF16)
         self._ar = torch.arange(cbs, device=dev, dtype=torch.int32)
@@ -154,7 +161,7 @@ class DecodeSession:
         """Compress the window that ends at the device-side position (already advanced past the newest token) and append it
         to the compressed caches (NSA.py:422-441); every index comes from device memory."""
         m = self.module
-        rows = torch.remainder(self.state[0] - self.cbs + self._ar, self.ring)
+        rows = ring_rows(self.state[0] - self.cbs, self._ar, self.ring)
         wk = self.ring_k.index_select(2, rows)
         wv = self.ring_v.index_select(2, rows)
         at = self.state[1:2].long()
@@ -189,7 +196,7 @@ class DecodeSession:
         """The caches in the module's format `((k, v), ((ck, cv), (run_k, run_v)))` (copies of the filled parts)."""
         t, st, cbs = self.pos, self.st, self.cbs
         first = (t // st) * st - (cbs - st)                          # first position of the open window
-        rows = torch.arange(first, t, device=self.K.device) % self.ring
+        rows = ring_rows(first, torch.arange(t - first, device=self.K.device), self.ring)
         run_k, run_v = self.ring_k.index_select(2, rows), self.ring_v.index_select(2, rows)
         if first < 0:                                                # positions before the sequence start read as zero
             run_k[:, :, :-first] = 0

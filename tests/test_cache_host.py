@@ -56,3 +56,24 @@ def test_empty_cache_and_views_that_do_not_start_at_the_buffer():
     tail = g2[:, :, 1:]              # a suffix view (what the running window keeps after a compression step)
     h, _ = _append_rows(tail)
     assert h._base is not g2._base and h.shape[2] == 2
+
+
+def test_ring_rows_hold_the_last_positions():
+    """The graph-replayed decode keeps the un-rotated keys of the last tokens in a ring (position p in row p % ring);
+    the compression window ending at position `end` must read exactly positions end-cbs .. end-1, zeros before the
+    sequence start, for every alignment and across the wrap."""
+    from native_sparse_attention_pytorch_amd.decode_session import ring_rows
+    for cbs, st in ((8, 4), (16, 16), (32, 8), (5, 5)):
+        ring = 2 * cbs
+        buf = torch.zeros(ring)
+        ar = torch.arange(cbs, dtype=torch.int32)
+        for pos in range(5 * ring + 3):
+            buf[pos % ring] = pos + 1                         # value = position + 1, so that 0 means "never written"
+            end = pos + 1
+            if end % st:
+                continue
+            for first in (end - cbs, torch.tensor(end - cbs, dtype=torch.int32)):      # host int and device-style counter
+                rows = ring_rows(first, ar, ring)
+                got = buf[rows.long()]
+                want = torch.tensor([float(p + 1) if p >= 0 else 0.0 for p in range(end - cbs, end)])
+                assert torch.equal(got, want), (cbs, st, pos)
