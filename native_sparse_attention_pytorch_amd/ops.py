@@ -156,15 +156,20 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     fp16, TRI.py:1845).  `sel_scale` must be all ones (straight-through gates, as the reference
     asserts at TRI.py:1861 - not re-checked here to avoid a device sync); it receives the gradient
     TRI.py:1061-1080 computes.  `block_dk_dv_use_dot` is accepted and ignored (a Triton tuning
-    switch)."""
+    switch).  With `return_sliding_window_out` the outputs become pairs `(out, sliding_out)` / `(lse, sliding_lse)`
+    as in the reference (TRI.py:1975-1985)."""
     q_heads, kv_heads, sel_heads = fq.shape[1], fk.shape[1], selected_block_indices.shape[1]
     assert q_heads % kv_heads == 0
     assert sel_heads in (q_heads, kv_heads)
     assert block_size in (8, 16, 32, 64), 'the HIP kernels are compiled for selection blocks of 8, 16, 32 or 64 keys'
-    if return_sliding_window_out:
-        raise NotImplementedError("the fused sliding-window output is experimental in the reference "
-                                  "(test_triton_nsa.py:144) and is served by sliding_attend here")
     dtype = fq.dtype
+    sliding_out = sliding_lse = None
+    if return_sliding_window_out:
+        # the reference's second output (TRI.py:195-277 with SLIDING): causal attention over the last block_size + 1 keys,
+        # 0 <= i - j <= block_size (test_triton_nsa.py:45-51); here it is the sliding-window kernel with that window
+        sliding_out, sliding_lse, _ = dense_fwd(fq.to(_BF16), fk.to(_BF16), fv.to(_BF16), 0, True, int(block_size), 1, 0, False, 1, True,
+                                                float(fq.shape[-1] ** -0.5))
+        sliding_out = sliding_out.to(dtype)
     if kv_heads != sel_heads:                         # per-query-head selection: TRI.py:1961-1962
         g = q_heads // kv_heads
         fk, fv = fk.repeat_interleave(g, dim=1), fv.repeat_interleave(g, dim=1)
@@ -187,6 +192,8 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
         g = q_heads // hs
         out = torch.where(dead.repeat_interleave(g, dim=1)[..., None], avg.repeat_interleave(g, dim=1).to(out.dtype), out)
     out = out.to(dtype)
+    if return_sliding_window_out:
+        out, lse = (out, sliding_out), (lse, sliding_lse)
     return (out, lse) if return_lse else out
 
 

@@ -196,3 +196,26 @@ def _oracle_rows(q, k, v, idx, msk, B, sl):
                     p = torch.softmax((keys @ q[bi, h * g + gg, i]) * d ** -0.5, dim=0)
                     out[bi, h * g + gg, t] = p @ vals
     return out
+
+
+def test_select_with_sliding_window_output():
+    """return_sliding_window_out (TRI.py:1975-1985, test_triton_nsa.py:45-51, 184-189): the second output is causal
+    attention over the last block_size + 1 keys; forward and the gradients of the summed loss against the oracle."""
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    b, hq, hk, n, d, B, S = 2, 8, 2, 300, 64, 16, 3
+    q, k, v, _ = _inputs(b, hq, hk, n, d, seed=21)
+    idx, msk = causal_random_selection(b, hk, n, B, S, seed=22)
+    qr, kr, vr = (t.float().requires_grad_() for t in (q, k, v))
+    ref, ref_lse = O.select_attend(qr, kr, vr, idx, msk, B, causal=True, return_lse=True)
+    ref_s = O.sliding_attend(qr, kr, vr, B, causal=True)
+    (ref.sum() + ref_s.sum()).backward()
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    (out, s_out), (lse, s_lse) = native_sparse_attend(qg, kg, vg, B, idx.to(DEV), msk.to(DEV), return_lse=True, return_sliding_window_out=True)
+    (out.float().sum() + s_out.float().sum()).backward()
+    torch.cuda.synchronize()
+    assert_close(out, ref, 2e-2, 1e-2, "out")
+    assert_close(s_out, ref_s, 2e-2, 1e-2, "sliding out")
+    assert_close(lse, ref_lse, 1e-2, 1e-3, "lse")
+    assert s_lse.shape == lse.shape and torch.isfinite(s_lse).all()
+    for name, got, want in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
+        assert_close(got, want, 2e-2 * want.abs().max().item(), 5e-2, name)
