@@ -36,7 +36,7 @@ static inline int make_plan(const nsa_select_desc* d, SelPlan& P) {
   if (!d) return NSA_E_ARG;
   if (d->batch <= 0 || d->kv_heads <= 0 || d->group <= 0 || d->seq <= 0 || d->num_sel < 0 || d->block <= 0) return NSA_E_ARG;
   if (d->dim_head != 64 && d->dim_head != 128) return NSA_E_UNSUPPORTED;
-  if (d->block != 8 && d->block != 16 && d->block != 32 && d->block != 64) return NSA_E_UNSUPPORTED;
+  if (d->block > 64) return NSA_E_UNSUPPORTED;                 // a block is one or two 32-key register tiles; keys past the block are masked
   if (d->group > 32 || (d->group & (d->group - 1))) return NSA_E_UNSUPPORTED;
   if (d->num_sel > 62) return NSA_E_UNSUPPORTED;
   if (!d->causal && d->num_sel == 0) return NSA_E_ARG;

@@ -161,7 +161,7 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     q_heads, kv_heads, sel_heads = fq.shape[1], fk.shape[1], selected_block_indices.shape[1]
     assert q_heads % kv_heads == 0
     assert sel_heads in (q_heads, kv_heads)
-    assert block_size in (8, 16, 32, 64), 'the HIP kernels are compiled for selection blocks of 8, 16, 32 or 64 keys'
+    assert 1 <= block_size <= 64, 'the HIP kernels hold a selection block in one or two 32-key tiles: block sizes up to 64'
     dtype = fq.dtype
     sliding_out = sliding_lse = None
     if return_sliding_window_out:
@@ -332,8 +332,21 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
     importance logits of NSA.py:652-691 before the softmax (None if sel_block is None or no full
     fine block exists): the logits matrix itself is never written to memory."""
     pool = sel_block is not None
-    out, _, pooled = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), pool, int(sel_block or stride), bool(share),
-                               float(q.shape[-1] ** -0.5))
+    scale = float(q.shape[-1] ** -0.5)
+    npf = int(sel_block) // int(stride) if pool else 1
+    if pool and (npf > 32 or npf & (npf - 1)):
+        # The kernel pools groups of 1, 2, 4 .. 32 compressed keys.  Other ratios (a selection block of 20 over stride 4, as in
+        # the reference's own inference test) take the per-key logits from the kernel (a "block" of one key: head mean and
+        # visibility as usual) and finish NSA.py:676-689 with three elementwise ops: mean over the block's keys (-inf as
+        # soon as one key is invisible), own block masked.
+        out, _, per_key = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), True, int(stride), bool(share), scale)
+        n, nb = q.shape[2], per_key.shape[-1] // npf
+        if nb == 0:
+            return out, None
+        imp = per_key[..., :nb * npf].unflatten(-1, (nb, npf)).mean(dim=-1)
+        own = (torch.arange(n, device=q.device) // int(sel_block))[:, None] == torch.arange(nb, device=q.device)[None, :]
+        return out, imp.masked_fill(own, float("-inf"))
+    out, _, pooled = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), pool, int(sel_block or stride), bool(share), scale)
     return out, (pooled if pool and pooled.shape[-1] > 0 else None)
 
 

@@ -58,6 +58,9 @@ COMPRESS = [
     (1, 8, 2, 40, 64, 16, 64, 1, True, True),        # n < B: no full fine block
     (1, 4, 2, 3, 64, 4, 16, 1, True, True),          # n < stride: only the memory slot
     (1, 4, 2, 300, 64, 2, 32, 1, True, True),        # npf 16
+    (1, 4, 2, 333, 64, 4, 20, 1, True, True),        # npf 5 (selection block 20: the reference's inference test grid)
+    (1, 4, 2, 150, 64, 2, 20, 2, True, False),       # npf 10, per-head selection
+    (1, 4, 2, 100, 64, 4, 12, 1, False, True),       # npf 3, non-causal
 ]
 
 

@@ -47,6 +47,12 @@ CONFIGS = [
     dict(dim=256, dim_head=64, heads=8, kv_heads=2, sliding_window_size=64, compress_block_size=16,
          compress_block_sliding_stride=8, selection_block_size=32, num_selected_blocks=4, causal=True, use_diff_topk=True,
          compress_mlp="grouped"),
+    # the reference's own inference-test shapes (tests/test_sparse_attn.py:50-86): compress block 5, selection block 20
+    dict(dim=128, dim_head=64, heads=4, kv_heads=2, sliding_window_size=2, compress_block_size=5,
+         compress_block_sliding_stride=4, selection_block_size=20, num_selected_blocks=2, causal=True),
+    # the reference README's configuration (README.md:35-50): 4-token blocks, non-causal by default
+    dict(dim=128, dim_head=64, heads=8, kv_heads=8, sliding_window_size=2, compress_block_size=4,
+         compress_block_sliding_stride=2, selection_block_size=4, num_selected_blocks=2),
 ]
 
 

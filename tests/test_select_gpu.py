@@ -44,6 +44,10 @@ CASES = [
     (1, 8, 2, 1000, 128, 32, 7),     # ragged, d=128, B=32
     (2, 8, 4, 77, 64, 8, 3),         # 8-key blocks (below the reference Triton path's minimum), ragged
     (1, 4, 1, 250, 128, 8, 6),       # 8-key blocks, G=4, d=128
+    (2, 4, 2, 61, 64, 4, 3),         # 4-key blocks: the reference's README / default transformer configuration
+    (1, 8, 2, 333, 64, 20, 4),       # 20-key blocks (the reference's inference test grid), ragged
+    (1, 4, 2, 200, 128, 48, 2),      # 48 keys: a second, partly filled 32-key tile
+    (1, 2, 2, 50, 64, 5, 3),         # odd block size
 ]
 
 
