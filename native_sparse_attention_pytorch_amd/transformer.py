@@ -25,8 +25,10 @@ class Transformer(nn.Module):
         super().__init__()
         if not use_sparse_attn:
             raise NotImplementedError("only the sparse-attention model is provided (the dense baseline is not part of the hot path)")
-        if use_flex_sliding_window or use_flex_fine_selection:
-            raise NotImplementedError("flex-attention backends are not provided; the HIP kernels implement the same masks")
+        # use_flex_sliding_window / use_flex_fine_selection / use_triton_fine_selection choose between the reference's
+        # backends for the same masks (transformer.py:154-177, 281-296); accepted so that the reference's training script
+        # constructs this model unchanged, and ignored: the HIP kernels always run
+        assert not (use_flex_fine_selection and use_triton_fine_selection), 'either using flex or custom triton kernel for fine attn, but not both'
         sparse_attn_kwargs = dict(sparse_attn_kwargs or dict(sliding_window_size=32, compress_block_size=4,
                                                              compress_block_sliding_stride=4, selection_block_size=4,
                                                              num_selected_blocks=4))

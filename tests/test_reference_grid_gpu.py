@@ -61,3 +61,32 @@ def test_readme_configuration():
     assert tokens.shape == attended.shape and attended.dtype == tokens.dtype and torch.isfinite(attended).all()
     attended.sum().backward()
     assert all(p.grad is None or torch.isfinite(p.grad).all() for p in attn.parameters())
+
+
+def test_training_script_model_configuration():
+    """The model exactly as the reference's train.py:87-113 builds it (flex sliding window flag, per-head grouped compression
+    MLP, differentiable top-k): one Adam step and cached sampling, as the script's loop does (train.py:150-200)."""
+    from native_sparse_attention_pytorch_amd.transformer import Transformer
+    from native_sparse_attention_pytorch_amd.compress_networks import GroupedMLP
+    torch.manual_seed(0)
+    model = Transformer(num_tokens=256, dim=512, depth=6, heads=8, dim_head=64, kv_heads=4, use_sparse_attn=True,
+                        use_flex_sliding_window=True, use_triton_fine_selection=True, use_flex_fine_selection=False,
+                        sparse_attn_kwargs=dict(sliding_window_size=64, compress_block_size=16, compress_block_sliding_stride=8,
+                                                compress_mlp=GroupedMLP(dim_head=64, compress_window_size=16, heads=4),
+                                                selection_block_size=16, num_selected_blocks=4, use_diff_topk=True,
+                                                query_heads_share_selected_kv=True)).to(DEV)
+    optim = torch.optim.Adam(model.parameters(), lr=1e-4)
+    data = torch.randint(0, 256, (4, 513), device=DEV)
+    losses = []
+    for _ in range(3):
+        loss = model(data, return_loss=True)
+        loss.backward()
+        torch.nn.utils.clip_grad_norm_(model.parameters(), 0.5)
+        optim.step()
+        optim.zero_grad()
+        losses.append(loss.item())
+    assert all(torch.isfinite(torch.tensor(losses))) and losses[-1] < losses[0]
+    model.eval()
+    prime = data[:1, :64]
+    sampled = model.sample(prime, 128, use_cache_kv=True)
+    assert sampled.shape == (1, 64) and int(sampled.min()) >= 0 and int(sampled.max()) < 256
