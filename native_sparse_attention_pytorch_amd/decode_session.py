@@ -86,10 +86,14 @@ class DecodeSession:
         # weight (a copy: the session does not follow later changes of the module's parameters), its bias is added where the
         # logits are used
         gate = m.to_strategy_combine[0]
-        pad = -3 * m.heads % 8                                      # rows of the GEMM output stay 16-byte aligned
-        self.w_cat = torch.cat((m.to_qkv.weight.detach(), gate.weight.detach().to(_BF16),
-                                torch.zeros((pad, m.to_qkv.in_features), dtype=_BF16, device=dev)), dim=0).contiguous()
-        self.gate_bias = gate.bias.detach().to(_BF16).contiguous() if gate.bias is not None else None
+        self.fused_gate = isinstance(gate, torch.nn.Linear) and gate.in_features == m.to_qkv.in_features and gate.out_features == 3 * m.heads
+        if self.fused_gate:
+            pad = -3 * m.heads % 8                                  # rows of the GEMM output stay 16-byte aligned
+            self.w_cat = torch.cat((m.to_qkv.weight.detach(), gate.weight.detach().to(_BF16),
+                                    torch.zeros((pad, m.to_qkv.in_features), dtype=_BF16, device=dev)), dim=0).contiguous()
+            self.gate_bias = gate.bias.detach().to(_BF16).contiguous() if gate.bias is not None else None
+        else:                                                       # a caller-supplied strategy network runs as it is
+            self.w_cat, self.gate_bias = m.to_qkv.weight.detach(), None
         self.x_buf = torch.zeros((b, 1, m.to_qkv.in_features), dtype=_BF16, device=dev)
         self._desc, self._ws = self._make_desc(dev)
         self.graphs = None
@@ -148,11 +152,16 @@ class DecodeSession:
         hq, hk, d = self.hq, self.hk, self.d
         merged = torch.empty((self.b, 1, hq * d), dtype=_BF16, device=x.device)
         p = qkvg.data_ptr()
+        if self.fused_gate:
+            gate_ptr, gate_row = p + 2 * (hq + 2 * hk) * d, qkvg.shape[-1]
+        else:
+            gl = m.to_strategy_combine[0](x).to(_BF16).contiguous()
+            gate_ptr, gate_row = gl.data_ptr(), 0
         _lib.check(_lib.lib().nsa_decode_step_dyn(
             C.byref(self._desc), self.state.data_ptr(), p, p + 2 * hq * d, p + 2 * (hq + hk) * d, self.freqs.data_ptr(),
             self.K.data_ptr(), self.V.data_ptr(), self.CK.data_ptr(), self.CV.data_ptr(), self.mem_k.data_ptr(), self.mem_v.data_ptr(),
             self.ring_k.data_ptr(), self.ring_v.data_ptr(), self.ring_k.stride(2), self.ring_v.stride(2), self.ring,
-            p + 2 * (hq + 2 * hk) * d, qkvg.shape[-1], self.gate_bias.data_ptr() if self.gate_bias is not None else None,
+            gate_ptr, gate_row, self.gate_bias.data_ptr() if self.gate_bias is not None else None,
             self._ws.data_ptr(), self._ws.numel(), merged.data_ptr(), int(advance),
             torch.cuda.current_stream(x.device).cuda_stream), "nsa_decode_step_dyn")
         return m.combine_heads(merged)

@@ -113,3 +113,27 @@ def test_transformer_graph_decode_matches_cached_decode():
     assert a.shape == b.shape == (2, 28) and b.dtype == torch.long
     assert torch.equal(a[:, 0], b[:, 0])                     # the first new token comes from the same prefill
     assert (a == b).float().mean() > 0.5                     # greedy paths agree until a near-tie flips a token
+
+
+def test_graph_decode_with_custom_strategy_network():
+    """A caller-supplied strategy_combine_mlp (NSA.py:315-327) is not a plain projection: the session then runs it as it is
+    instead of folding it into the qkv GEMM."""
+    from torch import nn
+    from native_sparse_attention_pytorch_amd import SparseAttention
+    from native_sparse_attention_pytorch_amd.decode_session import DecodeSession
+    from tests.util import assert_close
+    torch.manual_seed(11)
+    dim, heads = 128, 4
+    m = SparseAttention(dim=dim, dim_head=64, heads=heads, kv_heads=2, sliding_window_size=8, compress_block_size=8,
+                        compress_block_sliding_stride=4, selection_block_size=8, num_selected_blocks=2, causal=True,
+                        strategy_combine_mlp=nn.Sequential(nn.Linear(dim, 32), nn.ReLU(), nn.Linear(32, 3 * heads))).to(DEV).bfloat16()
+    xs = torch.randn(2, 40, dim, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        _, cache = m(xs[:, :13], return_cache=True)
+    sess = DecodeSession(m, cache, max_len=40)
+    assert not sess.fused_gate
+    for i in range(13, 40):
+        with torch.no_grad():
+            want, cache = m(xs[:, i:i + 1], cache=cache, return_cache=True)
+        got = sess.step(xs[:, i:i + 1])
+        assert_close(got, want, 2e-2, 1e-2, f"step {i}")
