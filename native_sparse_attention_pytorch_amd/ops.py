@@ -41,6 +41,27 @@ def _prep(t: Tensor) -> Tensor:
     return t if _rows_ok(t) else t.contiguous()
 
 
+def _pad_groups(q: Tensor, hk: int):
+    """The attention kernels lay the G query heads of a kv head side by side in a 32-row tile, so G must be a power of
+    two.  Any other group size is padded with zero query heads (they attend uniformly, are sliced away again and get a
+    zero upstream gradient, so they add nothing to dk / dv).  Returns (q', G, G')."""
+    b, hq, n, d = q.shape
+    g = hq // hk
+    gp = 1 << max(g - 1, 0).bit_length()
+    if gp == g:
+        return q, g, g
+    qp = torch.nn.functional.pad(q.reshape(b, hk, g, n, d), (0, 0, 0, 0, 0, gp - g)).reshape(b, hk * gp, n, d)
+    return qp, g, gp
+
+
+def _unpad_groups(t: Tensor, hk: int, g: int, gp: int) -> Tensor:
+    """'b (hk G') n ...' -> 'b (hk G) n ...'"""
+    if g == gp:
+        return t
+    b = t.shape[0]
+    return t.reshape(b, hk, gp, *t.shape[2:])[:, :, :g].reshape(b, hk * g, *t.shape[2:])
+
+
 def _select_desc(q, k, v, o, num_sel, block, causal, scale, idx_is_int64) -> _lib.SelectDesc:
     b, hq, n, d = q.shape
     hk = k.shape[1]
@@ -167,15 +188,19 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     if return_sliding_window_out:
         # the reference's second output (TRI.py:195-277 with SLIDING): causal attention over the last block_size + 1 keys,
         # 0 <= i - j <= block_size (test_triton_nsa.py:45-51); here it is the sliding-window kernel with that window
-        sliding_out, sliding_lse, _ = dense_fwd(fq.to(_BF16), fk.to(_BF16), fv.to(_BF16), 0, True, int(block_size), 1, 0, False, 1, True,
+        qp, g0, gp0 = _pad_groups(fq.to(_BF16), kv_heads)
+        sliding_out, sliding_lse, _ = dense_fwd(qp, fk.to(_BF16), fv.to(_BF16), 0, True, int(block_size), 1, 0, False, 1, True,
                                                 float(fq.shape[-1] ** -0.5))
-        sliding_out = sliding_out.to(dtype)
+        sliding_out = _unpad_groups(sliding_out, kv_heads, g0, gp0).to(dtype)
+        sliding_lse = _unpad_groups(sliding_lse, kv_heads, g0, gp0)
     if kv_heads != sel_heads:                         # per-query-head selection: TRI.py:1961-1962
         g = q_heads // kv_heads
         fk, fv = fk.repeat_interleave(g, dim=1), fv.repeat_interleave(g, dim=1)
     scale = fq.shape[-1] ** -0.5
-    out, lse, _ = select_fwd(fq.to(_BF16), fk.to(_BF16), fv.to(_BF16), selected_block_indices, fmask, sel_scale,
+    qp, g0, gp0 = _pad_groups(fq.to(_BF16), fk.shape[1])
+    out, lse, _ = select_fwd(qp, fk.to(_BF16), fv.to(_BF16), selected_block_indices, fmask, sel_scale,
                              int(block_size), bool(include_block_causal), float(scale))
+    out, lse = _unpad_groups(out, fk.shape[1], g0, gp0), _unpad_groups(lse, fk.shape[1], g0, gp0)
     if not include_block_causal and selected_block_indices.shape[-1] > 0:
         # A query whose slots are all dead attends nothing in the kernel.  The reference's torch
         # path (NSA.py:809-815) fills every logit of such a row with the same value, i.e. it
@@ -321,8 +346,9 @@ def sliding_attend(q: Tensor, k: Tensor, v: Tensor, window_size: int, causal: bo
     """Sliding-window branch: what `self.sliding_window(sq, sk, sv)` computes at NSA.py:841-850
     (LocalAttention with exact window, autopad) without materialising the repeated k/v:
     q [b,Hq,n,d], k/v [b,Hkv,n,d]; query i sees 0 <= i-j <= window_size (causal) or |i-j| <= it."""
-    out, _, _ = dense_fwd(q, k, v, 0, bool(causal), int(window_size), 1, 0, False, 1, True, float(q.shape[-1] ** -0.5))
-    return out
+    qp, g, gp = _pad_groups(q, k.shape[1])
+    out, _, _ = dense_fwd(qp, k, v, 0, bool(causal), int(window_size), 1, 0, False, 1, True, float(q.shape[-1] ** -0.5))
+    return _unpad_groups(out, k.shape[1], g, gp)
 
 
 def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int, causal: bool,
@@ -334,20 +360,30 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
     pool = sel_block is not None
     scale = float(q.shape[-1] ** -0.5)
     npf = int(sel_block) // int(stride) if pool else 1
+    hk = ck.shape[1]
+    q, g, gp = _pad_groups(q, hk)
+
+    def logits_of(pooled):
+        # zero padding heads add nothing to a group's sum: the kernel's mean over G' heads becomes the mean over G;
+        # per-head logits of the padding heads are dropped
+        if g == gp:
+            return pooled
+        return pooled * (gp / g) if share else _unpad_groups(pooled, hk, g, gp)
     if pool and (npf > 32 or npf & (npf - 1)):
         # The kernel pools groups of 1, 2, 4 .. 32 compressed keys.  Other ratios (a selection block of 20 over stride 4, as in
         # the reference's own inference test) take the per-key logits from the kernel (a "block" of one key: head mean and
         # visibility as usual) and finish NSA.py:676-689 with three elementwise ops: mean over the block's keys (-inf as
         # soon as one key is invisible), own block masked.
         out, _, per_key = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), True, int(stride), bool(share), scale)
+        out = _unpad_groups(out, hk, g, gp)
         n, nb = q.shape[2], per_key.shape[-1] // npf
         if nb == 0:
             return out, None
-        imp = per_key[..., :nb * npf].unflatten(-1, (nb, npf)).mean(dim=-1)
+        imp = logits_of(per_key)[..., :nb * npf].unflatten(-1, (nb, npf)).mean(dim=-1)
         own = (torch.arange(n, device=q.device) // int(sel_block))[:, None] == torch.arange(nb, device=q.device)[None, :]
         return out, imp.masked_fill(own, float("-inf"))
     out, _, pooled = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), pool, int(sel_block or stride), bool(share), scale)
-    return out, (pooled if pool and pooled.shape[-1] > 0 else None)
+    return _unpad_groups(out, hk, g, gp), (logits_of(pooled) if pool and pooled.shape[-1] > 0 else None)
 
 
 # ------------------------------------------------------------------------------------ top-k

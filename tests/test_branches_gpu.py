@@ -26,6 +26,7 @@ SLIDING = [
     (1, 4, 4, 257, 64, 512, True),        # window >= n: full causal attention
     (2, 4, 1, 200, 64, 17, False),
     (1, 16, 4, 1024, 64, 64, True),
+    (1, 6, 2, 200, 64, 32, True),         # G=3: not a power of two (padded with zero heads)
 ]
 
 
@@ -61,6 +62,9 @@ COMPRESS = [
     (1, 4, 2, 333, 64, 4, 20, 1, True, True),        # npf 5 (selection block 20: the reference's inference test grid)
     (1, 4, 2, 150, 64, 2, 20, 2, True, False),       # npf 10, per-head selection
     (1, 4, 2, 100, 64, 4, 12, 1, False, True),       # npf 3, non-causal
+    (1, 6, 2, 200, 64, 4, 16, 1, True, True),        # G=3, shared selection: the group mean must be over 3 heads
+    (1, 6, 2, 200, 64, 4, 16, 1, True, False),       # G=3, per-head selection
+    (1, 12, 2, 100, 64, 4, 20, 1, True, True),       # G=6 with npf 5
 ]
 
 

@@ -13,6 +13,7 @@ CONFIGS = [
     (256, 128, 2, 1, 32, 16, 8, 16, 3, True, 70, 40),
     (256, 64, 4, 2, 8, 8, 8, 8, 4, False, 21, 30),        # stride == block, selection per query head
     (128, 64, 2, 2, 16, 8, 4, 8, 2, True, 2, 40),         # starts before the first compressed key exists
+    (192, 64, 6, 2, 16, 8, 4, 8, 2, True, 30, 30),        # group of 3 query heads per kv head
 ]
 
 

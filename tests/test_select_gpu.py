@@ -48,6 +48,8 @@ CASES = [
     (1, 8, 2, 333, 64, 20, 4),       # 20-key blocks (the reference's inference test grid), ragged
     (1, 4, 2, 200, 128, 48, 2),      # 48 keys: a second, partly filled 32-key tile
     (1, 2, 2, 50, 64, 5, 3),         # odd block size
+    (2, 6, 2, 300, 64, 16, 3),       # G=3: not a power of two (padded with zero heads)
+    (1, 5, 1, 130, 128, 32, 2),      # G=5
 ]
 
 
