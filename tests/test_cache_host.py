@@ -77,3 +77,20 @@ def test_ring_rows_hold_the_last_positions():
                 got = buf[rows.long()]
                 want = torch.tensor([float(p + 1) if p >= 0 else 0.0 for p in range(end - cbs, end)])
                 assert torch.equal(got, want), (cbs, st, pos)
+
+
+def test_group_padding_round_trip():
+    """Query heads of a kv group are padded to a power of two with zero heads at the end of each group, and come back
+    in their original order."""
+    from native_sparse_attention_pytorch_amd.ops import _pad_groups, _unpad_groups
+    for hk, g in ((2, 3), (1, 5), (4, 6), (3, 7), (2, 4), (5, 1)):
+        q = torch.randn(2, hk * g, 7, 8)
+        qp, g0, gp = _pad_groups(q, hk)
+        assert g0 == g and gp >= g and gp & (gp - 1) == 0 and gp < 2 * g + (g == 1)
+        assert qp.shape == (2, hk * gp, 7, 8)
+        grouped = qp.reshape(2, hk, gp, 7, 8)
+        assert torch.equal(grouped[:, :, :g].reshape(2, hk * g, 7, 8), q)
+        assert (grouped[:, :, g:] == 0).all()
+        assert torch.equal(_unpad_groups(qp, hk, g, gp), q)
+        lse = torch.randn(2, hk * gp, 7)
+        assert _unpad_groups(lse, hk, g, gp).shape == (2, hk * g, 7)
