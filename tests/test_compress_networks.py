@@ -1,9 +1,7 @@
 """Alternative compression networks (compress_networks.py:19-241): each checked on the CPU
 against an independent formulation - the einops mixing layer the reference builds them from
 (a library routine, loaded with the same parameters), a per-window loop, or a closed form."""
-import pytest
 import torch
-from torch import nn
 
 from native_sparse_attention_pytorch_amd import compress_networks as CN
 

@@ -1,6 +1,5 @@
 """Parity of the HIP block-selection attention (through the C ABI) against the CPU oracle.
 Tolerances are BASELINE.json's: forward 2e-2 abs / 1e-2 rel in bf16, gradients 5e-2 rel."""
-import ctypes as C
 
 import pytest
 import torch
