@@ -43,6 +43,8 @@ int nsa_selftest_mfma(const void* A, const void* B, float* C, const void* X, flo
  * twice counts twice, keys at or beyond `seq` count with logit 0 and value 0) plus, if `causal`,
  * the keys j <= i of its own block (TRI.py include_block_causal).  The `group` query heads
  * h*group .. h*group+group-1 share kv head h and its selection.
+ * Limits (NSA_E_UNSUPPORTED otherwise): dim_head 64 or 128, 1 <= block <= 64, group a power of two <= 32,
+ * num_sel <= 62, at most 16384 blocks.
  * ------------------------------------------------------------------------------------------ */
 typedef struct nsa_select_desc {
   int32_t batch, kv_heads, group, seq, num_sel, block, dim_head, causal;
@@ -98,6 +100,8 @@ int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const
  *                     fine block j and, if `share`, over the group's heads; -inf where the
  *                     reference's fill values (-finfo.max/10 for an invisible key, -finfo.max for
  *                     the query's own block when stride != sel_block) make the softmax term zero.
+ *                     sel_block / stride must be a power of two <= 32 (with sel_block == stride the
+ *                     output holds one logit per compressed key, which serves every other ratio).
  * out/lse as for nsa_select_fwd; dq contiguous [batch, heads, seq, d]; dk, dv contiguous
  * [batch, kv_heads, num_mem + num_keys, d].  bf16 in, fp32 accumulate, bf16 out.
  * ------------------------------------------------------------------------------------------ */
