@@ -168,6 +168,32 @@ def _select_backward(ctx, dout, dlse, dws):
 select_fwd.register_autograd(_select_backward, setup_context=_select_setup)
 
 
+def _split_blocks(idx: Tensor, fmask: Tensor, sel_scale: Tensor | None, block: int, n: int, causal: bool):
+    """The selection kernels hold a block in one or two 32-key register tiles (<= 64 keys).  A larger block is handed to
+    them as m equal sub-blocks: slot s naming block j becomes the m slots 's*m + r' naming sub-blocks 'j*m + r'; under the
+    causal own-block rule the sub-blocks of the query's own block that lie before the query's own sub-block are fully
+    visible and become m - 1 further slots.  The softmax over the concatenated keys is the same; a gate on slot s reaches
+    the kernel once per sub-block, so its gradient comes back summed.  Returns (idx, fmask, sel_scale, sub-block size)."""
+    m = -(-block // 64)
+    while block % m:
+        m += 1
+    if m == 1:
+        return idx, fmask, sel_scale, block
+    sub = block // m
+    r = torch.arange(m, device=idx.device)
+    idx_k = (idx.long()[..., None] * m + r).flatten(-2)
+    fm_k = fmask.bool()[..., None].expand(*fmask.shape, m).flatten(-2)
+    sc_k = None if sel_scale is None else sel_scale[..., None].expand(*sel_scale.shape, m).flatten(-2)
+    if causal:
+        pos = torch.arange(n, device=idx.device)
+        own_idx = ((pos // block)[:, None] * m + r[None, :m - 1]).expand(*idx.shape[:2], n, m - 1)
+        own_live = (r[None, :m - 1] < ((pos % block) // sub)[:, None]).expand(*idx.shape[:2], n, m - 1)
+        idx_k, fm_k = torch.cat((idx_k, own_idx), dim=-1), torch.cat((fm_k, own_live), dim=-1)
+        if sc_k is not None:
+            sc_k = torch.cat((sc_k, sc_k.new_ones(*idx.shape[:3], m - 1)), dim=-1)
+    return idx_k.contiguous(), fm_k.contiguous(), sc_k, sub
+
+
 def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, selected_block_indices: Tensor, fmask: Tensor,
                          sel_scale: Tensor | None = None, include_block_causal: bool = True, return_lse: bool = False,
                          block_dk_dv_use_dot=None, return_sliding_window_out: bool = False):
@@ -182,7 +208,7 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     q_heads, kv_heads, sel_heads = fq.shape[1], fk.shape[1], selected_block_indices.shape[1]
     assert q_heads % kv_heads == 0
     assert sel_heads in (q_heads, kv_heads)
-    assert 1 <= block_size <= 64, 'the HIP kernels hold a selection block in one or two 32-key tiles: block sizes up to 64'
+    assert block_size >= 1
     dtype = fq.dtype
     sliding_out = sliding_lse = None
     if return_sliding_window_out:
@@ -198,8 +224,8 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
         fk, fv = fk.repeat_interleave(g, dim=1), fv.repeat_interleave(g, dim=1)
     scale = fq.shape[-1] ** -0.5
     qp, g0, gp0 = _pad_groups(fq.to(_BF16), fk.shape[1])
-    out, lse, _ = select_fwd(qp, fk.to(_BF16), fv.to(_BF16), selected_block_indices, fmask, sel_scale,
-                             int(block_size), bool(include_block_causal), float(scale))
+    idx_k, fm_k, sc_k, block_k = _split_blocks(selected_block_indices, fmask, sel_scale, int(block_size), fq.shape[2], bool(include_block_causal))
+    out, lse, _ = select_fwd(qp, fk.to(_BF16), fv.to(_BF16), idx_k, fm_k, sc_k, block_k, bool(include_block_causal), float(scale))
     out, lse = _unpad_groups(out, fk.shape[1], g0, gp0), _unpad_groups(lse, fk.shape[1], g0, gp0)
     if not include_block_causal and selected_block_indices.shape[-1] > 0:
         # A query whose slots are all dead attends nothing in the kernel.  The reference's torch

@@ -53,6 +53,9 @@ CONFIGS = [
     # the reference README's configuration (README.md:35-50): 4-token blocks, non-causal by default
     dict(dim=128, dim_head=64, heads=8, kv_heads=8, sliding_window_size=2, compress_block_size=4,
          compress_block_sliding_stride=2, selection_block_size=4, num_selected_blocks=2),
+    # 128-token selection blocks (two 64-key sub-blocks per slot in the kernels)
+    dict(dim=128, dim_head=64, heads=4, kv_heads=2, sliding_window_size=32, compress_block_size=32,
+         compress_block_sliding_stride=16, selection_block_size=128, num_selected_blocks=2, causal=True, use_diff_topk=True),
     # 6 query heads over 2 kv heads: a group of 3
     dict(dim=192, dim_head=64, heads=6, kv_heads=2, sliding_window_size=32, compress_block_size=16,
          compress_block_sliding_stride=8, selection_block_size=16, num_selected_blocks=3, causal=True, use_diff_topk=True),

@@ -49,6 +49,9 @@ CASES = [
     (1, 2, 2, 50, 64, 5, 3),         # odd block size
     (2, 6, 2, 300, 64, 16, 3),       # G=3: not a power of two (padded with zero heads)
     (1, 5, 1, 130, 128, 32, 2),      # G=5
+    (1, 8, 2, 1000, 64, 128, 3),     # 128-key blocks: two 64-key sub-blocks per slot, ragged
+    (2, 4, 2, 700, 128, 192, 2),     # 192 keys: three sub-blocks
+    (1, 4, 1, 400, 64, 96, 2),       # 96 keys: two 48-key sub-blocks
 ]
 
 
@@ -102,7 +105,7 @@ def test_select_gate_gradient_matches_oracle():
     gather path with gates multiplying the selected keys (NSA.py:793-797); tolerance of
     test_triton_nsa.py:194 scaled to the gradient's magnitude."""
     from native_sparse_attention_pytorch_amd import native_sparse_attend
-    for (b, hq, hk, n, d, B, S) in [(2, 4, 2, 300, 64, 16, 3), (1, 8, 2, 512, 128, 64, 4)]:
+    for (b, hq, hk, n, d, B, S) in [(2, 4, 2, 300, 64, 16, 3), (1, 8, 2, 512, 128, 64, 4), (1, 4, 2, 900, 64, 128, 3)]:
         q, k, v, do = _inputs(b, hq, hk, n, d, seed=n)
         idx, msk = causal_random_selection(b, hk, n, B, S, seed=5)
         gr = torch.ones(b, hk, n, S, requires_grad=True)
