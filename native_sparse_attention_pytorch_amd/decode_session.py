@@ -44,6 +44,8 @@ class DecodeSession:
         (cache_k, cache_v), ((cache_ck, cache_cv), (run_k, run_v)) = cache
         if not cache_k.is_cuda:
             raise RuntimeError("DecodeSession runs on the GPU only (HIP kernels, no CPU fallback)")
+        if m.dim_head not in (64, 128):
+            raise NotImplementedError("DecodeSession needs dim_head 64 or 128 (the module's step-by-step decode pads other sizes)")
         if m.to_qkv.weight.dtype != _BF16:
             raise NotImplementedError("DecodeSession needs a bf16 module (the raw key / value window is kept in bf16)")
         dev = cache_k.device

@@ -41,6 +41,19 @@ def _prep(t: Tensor) -> Tensor:
     return t if _rows_ok(t) else t.contiguous()
 
 
+def _kernel_dim(d: int) -> int:
+    """The kernels are compiled for 64 and 128 features per head; other head dimensions are zero-padded up to the next
+    of the two by the wrappers below (zero features change neither the logits nor the outputs' first d features; the
+    softmax scale stays that of the original dimension)."""
+    if d > 128:
+        raise RuntimeError(f"dim_head {d}: the HIP kernels hold at most 128 features per head")
+    return 64 if d <= 64 else 128
+
+
+def _pad_dim(t: Tensor, D: int) -> Tensor:
+    return t if t.shape[-1] == D else torch.nn.functional.pad(t, (0, D - t.shape[-1]))
+
+
 def _pad_groups(q: Tensor, hk: int):
     """The attention kernels lay the G query heads of a kv head side by side in a 32-row tile, so G must be a power of
     two.  Any other group size is padded with zero query heads (they attend uniformly, are sliced away again and get a
@@ -210,30 +223,34 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     assert sel_heads in (q_heads, kv_heads)
     assert block_size >= 1
     dtype = fq.dtype
+    d_head = fq.shape[-1]
+    scale = d_head ** -0.5
+    D = _kernel_dim(d_head)
+    fv_given = fv
+    fq, fk, fv = _pad_dim(fq.to(_BF16), D), _pad_dim(fk.to(_BF16), D), _pad_dim(fv.to(_BF16), D)
     sliding_out = sliding_lse = None
     if return_sliding_window_out:
         # the reference's second output (TRI.py:195-277 with SLIDING): causal attention over the last block_size + 1 keys,
         # 0 <= i - j <= block_size (test_triton_nsa.py:45-51); here it is the sliding-window kernel with that window
         qp, g0, gp0 = _pad_groups(fq.to(_BF16), kv_heads)
-        sliding_out, sliding_lse, _ = dense_fwd(qp, fk.to(_BF16), fv.to(_BF16), 0, True, int(block_size), 1, 0, False, 1, True,
-                                                float(fq.shape[-1] ** -0.5))
-        sliding_out = _unpad_groups(sliding_out, kv_heads, g0, gp0).to(dtype)
+        sliding_out, sliding_lse, _ = dense_fwd(qp, fk, fv, 0, True, int(block_size), 1, 0, False, 1, True, float(scale))
+        sliding_out = _unpad_groups(sliding_out, kv_heads, g0, gp0)[..., :d_head].to(dtype)
         sliding_lse = _unpad_groups(sliding_lse, kv_heads, g0, gp0)
     if kv_heads != sel_heads:                         # per-query-head selection: TRI.py:1961-1962
         g = q_heads // kv_heads
         fk, fv = fk.repeat_interleave(g, dim=1), fv.repeat_interleave(g, dim=1)
-    scale = fq.shape[-1] ** -0.5
-    qp, g0, gp0 = _pad_groups(fq.to(_BF16), fk.shape[1])
+    qp, g0, gp0 = _pad_groups(fq, fk.shape[1])
     idx_k, fm_k, sc_k, block_k = _split_blocks(selected_block_indices, fmask, sel_scale, int(block_size), fq.shape[2], bool(include_block_causal))
-    out, lse, _ = select_fwd(qp, fk.to(_BF16), fv.to(_BF16), idx_k, fm_k, sc_k, block_k, bool(include_block_causal), float(scale))
-    out, lse = _unpad_groups(out, fk.shape[1], g0, gp0), _unpad_groups(lse, fk.shape[1], g0, gp0)
+    out, lse, _ = select_fwd(qp, fk, fv, idx_k, fm_k, sc_k, block_k, bool(include_block_causal), float(scale))
+    out, lse = _unpad_groups(out, fk.shape[1], g0, gp0)[..., :d_head], _unpad_groups(lse, fk.shape[1], g0, gp0)
+    fv = fv_given if kv_heads == sel_heads else fv_given.repeat_interleave(q_heads // kv_heads, dim=1)
     if not include_block_causal and selected_block_indices.shape[-1] > 0:
         # A query whose slots are all dead attends nothing in the kernel.  The reference's torch
         # path (NSA.py:809-815) fills every logit of such a row with the same value, i.e. it
         # attends uniformly over the keys of the (dead) slots' blocks, zero padding included;
         # reproduce that corner with a few elementwise ops (no sync, differentiable in v).
         b, hs, n, S = selected_block_indices.shape
-        hk2, d = fk.shape[1], fk.shape[-1]
+        hk2, d = fk.shape[1], d_head
         W = (n + block_size - 1) // block_size
         vpad = torch.nn.functional.pad(fv, (0, 0, 0, W * block_size - n)).reshape(b, hk2, W, block_size, d)
         vmean = vpad.float().mean(dim=3)                                                  # [b,hk,W,d]
@@ -372,9 +389,11 @@ def sliding_attend(q: Tensor, k: Tensor, v: Tensor, window_size: int, causal: bo
     """Sliding-window branch: what `self.sliding_window(sq, sk, sv)` computes at NSA.py:841-850
     (LocalAttention with exact window, autopad) without materialising the repeated k/v:
     q [b,Hq,n,d], k/v [b,Hkv,n,d]; query i sees 0 <= i-j <= window_size (causal) or |i-j| <= it."""
-    qp, g, gp = _pad_groups(q, k.shape[1])
-    out, _, _ = dense_fwd(qp, k, v, 0, bool(causal), int(window_size), 1, 0, False, 1, True, float(q.shape[-1] ** -0.5))
-    return _unpad_groups(out, k.shape[1], g, gp)
+    d = q.shape[-1]
+    D = _kernel_dim(d)
+    qp, g, gp = _pad_groups(_pad_dim(q, D), k.shape[1])
+    out, _, _ = dense_fwd(qp, _pad_dim(k, D), _pad_dim(v, D), 0, bool(causal), int(window_size), 1, 0, False, 1, True, float(d ** -0.5))
+    return _unpad_groups(out, k.shape[1], g, gp)[..., :d]
 
 
 def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int, causal: bool,
@@ -384,10 +403,13 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
     importance logits of NSA.py:652-691 before the softmax (None if sel_block is None or no full
     fine block exists): the logits matrix itself is never written to memory."""
     pool = sel_block is not None
-    scale = float(q.shape[-1] ** -0.5)
+    d = q.shape[-1]
+    scale = float(d ** -0.5)
+    D = _kernel_dim(d)
     npf = int(sel_block) // int(stride) if pool else 1
     hk = ck.shape[1]
-    q, g, gp = _pad_groups(q, hk)
+    q, g, gp = _pad_groups(_pad_dim(q, D), hk)
+    ck, cv = _pad_dim(ck, D), _pad_dim(cv, D)
 
     def logits_of(pooled):
         # zero padding heads add nothing to a group's sum: the kernel's mean over G' heads becomes the mean over G;
@@ -401,7 +423,7 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
         # visibility as usual) and finish NSA.py:676-689 with three elementwise ops: mean over the block's keys (-inf as
         # soon as one key is invisible), own block masked.
         out, _, per_key = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), True, int(stride), bool(share), scale)
-        out = _unpad_groups(out, hk, g, gp)
+        out = _unpad_groups(out, hk, g, gp)[..., :d]
         n, nb = q.shape[2], per_key.shape[-1] // npf
         if nb == 0:
             return out, None
@@ -409,7 +431,7 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
         own = (torch.arange(n, device=q.device) // int(sel_block))[:, None] == torch.arange(nb, device=q.device)[None, :]
         return out, imp.masked_fill(own, float("-inf"))
     out, _, pooled = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), pool, int(sel_block or stride), bool(share), scale)
-    return _unpad_groups(out, hk, g, gp), (logits_of(pooled) if pool and pooled.shape[-1] > 0 else None)
+    return _unpad_groups(out, hk, g, gp)[..., :d], (logits_of(pooled) if pool and pooled.shape[-1] > 0 else None)
 
 
 # ------------------------------------------------------------------------------------ top-k
@@ -533,7 +555,10 @@ gate_fwd.register_autograd(_gate_backward, setup_context=_gate_setup)
 def gate_combine(logits: Tensor, compressed: Tensor, selected: Tensor, sliding: Tensor) -> Tensor:
     """sigmoid(logits) 'b n (h s) -> b h n s' weighted sum of the three branches, merged to
     'b n (h d)' (NSA.py:323-327, 854-860).  logits are the pre-sigmoid gate projection."""
-    return gate_fwd(logits.to(_BF16), compressed, selected, sliding)
+    b, h, n, d = compressed.shape
+    D = _kernel_dim(d)
+    out = gate_fwd(logits.to(_BF16), _pad_dim(compressed, D), _pad_dim(selected, D), _pad_dim(sliding, D))
+    return out if D == d else out.reshape(b, n, h, D)[..., :d].reshape(b, n, h * d)
 
 
 # ---------------------------------------------------------------------------------- rotary
@@ -570,7 +595,12 @@ rope_op.register_autograd(_rope_backward, setup_context=_rope_setup)
 
 def rotary(x: Tensor, freqs: Tensor, offset: int = 0) -> Tensor:
     """Rotary embedding of 'b h n d' queries or keys at positions offset .. offset+n-1 (NSA.py:643)."""
-    return rope_op(x, freqs, int(offset), False)
+    d = x.shape[-1]
+    D = _kernel_dim(d)
+    if D == d:
+        return rope_op(x, freqs, int(offset), False)
+    # padded feature pairs get frequency 0: they stay zero
+    return rope_op(_pad_dim(x, D), _pad_dim(freqs, D // 2), int(offset), False)[..., :d]
 
 
 def rotary_into(x: Tensor, freqs: Tensor, offset: int, out: Tensor) -> None:
@@ -772,7 +802,10 @@ def compress_windows(x: Tensor, pos: Tensor | None, block: int, stride: int) -> 
     """'b h n d' -> 'b h w block d' with w = n // stride: window w = tokens (w+1)*stride - block ..
     (w+1)*stride - 1, zeros left of token 0, plus the intra-window positions 'h block d'
     (NSA.py:270-275, 589-603)."""
-    return windows_fwd(x, pos, int(block), int(stride))
+    d = x.shape[-1]
+    D = _kernel_dim(d)
+    out = windows_fwd(_pad_dim(x, D), None if pos is None else _pad_dim(pos, D), int(block), int(stride))
+    return out[..., :d]
 
 
 @torch.no_grad()
@@ -797,7 +830,7 @@ def decode_importance_topk(logits: Tensor, kv_heads: int, per_block: int, share:
 @torch.no_grad()
 def decode_step(q: Tensor, k: Tensor, v: Tensor, freqs: Tensor, pos: int, keys: Tensor, vals: Tensor, ck: Tensor | None, cv: Tensor | None,
                 mem_k: Tensor | None, mem_v: Tensor | None, k_run_row: Tensor | None, v_run_row: Tensor | None, gate_logits: Tensor,
-                *, per_block: int, block: int, num_sel: int, share: bool, window: int):
+                *, per_block: int, block: int, num_sel: int, share: bool, window: int, scale: float | None = None):
     """The attention part of one decode step in a single library call (see nsa_decode_step in
     include/nsa_hip.h).  q 'b hq 1 d', k, v 'b hk 1 d': the new token's projections; keys, vals: the
     caches with row `pos` free ('b hk >=pos+1 d' views from the start of their buffers); ck, cv: the
@@ -815,7 +848,7 @@ def decode_step(q: Tensor, k: Tensor, v: Tensor, freqs: Tensor, pos: int, keys: 
     dsc = _lib.DecodeStepDesc()
     dsc.batch, dsc.heads, dsc.kv_heads, dsc.dim_head = b, hq, hk, d
     dsc.pos, dsc.num_compressed, dsc.per_block, dsc.block = int(pos), nc, int(per_block), int(block)
-    dsc.num_sel, dsc.share, dsc.window, dsc.scale = int(num_sel), int(bool(share)), int(window), d ** -0.5
+    dsc.num_sel, dsc.share, dsc.window, dsc.scale = int(num_sel), int(bool(share)), int(window), (d ** -0.5 if scale is None else float(scale))
     m = 0
     if nc and mem_k is not None:
         mem_k, mem_v = mem_k.to(_BF16).contiguous(), mem_v.to(_BF16).contiguous()

@@ -48,20 +48,22 @@ class RotaryEmbedding(nn.Module):
         return self.rotate(q, offset=k.shape[-2] - q.shape[-2]), self.rotate(k)
 
 
-def _append_rows(t: torch.Tensor, extra: int = 1, dtype=torch.bfloat16, min_capacity: int = 128):
+def _append_rows(t: torch.Tensor, extra: int = 1, dtype=torch.bfloat16, min_capacity: int = 128, feat: int | None = None):
     """Grow the 'b h n d' cache `t` by `extra` rows.  Returns (view of n+extra rows, view of the
     new rows).  When `t` is the filled prefix of a buffer made here, the rows are taken from the
     buffer's spare capacity; otherwise (a cache from the parallel forward, a branch point that
     re-uses an older cache, no capacity left) the contents move to a new bf16 buffer of twice
     the size first, so a caller that keeps an old cache tuple never sees it change."""
     b, h, n, d = t.shape
+    feat = d if feat is None else feat                # buffers may be wider than the rows handed in (zero-padded features)
     base = t._base
-    ok = (base is not None and getattr(base, "_nsa_filled", -1) == n and base.dtype == dtype
+    ok = (base is not None and getattr(base, "_nsa_filled", -1) == n and base.dtype == dtype and d == feat
           and base.dim() == 4 and base.shape[2] >= n + extra and base.shape[:2] == t.shape[:2] and base.shape[3] == d
           and t.data_ptr() == base.data_ptr() and t.stride() == base.stride())
     if not ok:
-        base = torch.empty((b, h, max(2 * (n + extra), min_capacity), d), dtype=dtype, device=t.device)
-        base[:, :, :n].copy_(t)
+        make = torch.empty if d == feat else torch.zeros
+        base = make((b, h, max(2 * (n + extra), min_capacity), feat), dtype=dtype, device=t.device)
+        base[:, :, :n, :d].copy_(t)
     base._nsa_filled = n + extra
     return base[:, :, :n + extra], base[:, :, n:n + extra]
 
@@ -175,17 +177,23 @@ class SparseAttention(nn.Module):
         x = self.norm(inp)
         q, k, v = self.to_qkv(x).split(self.qkv_split, dim=-1)
         q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
-        q16, k16, v16 = q.to(bf16), k.to(bf16), v.to(bf16)
+        # head dimensions other than the kernels' 64 / 128 run zero-padded: caches and window rows are then kept D wide
+        # (the padding features stay zero), the projections and the compression network see the first d features
+        d, D = self.dim_head, ops._kernel_dim(self.dim_head)
+        pad = (lambda u: u) if D == d else (lambda u: F.pad(u, (0, D - d)))
+        q16, k16, v16 = pad(q.to(bf16)), pad(k.to(bf16)), pad(v.to(bf16))
+        if D != d:
+            freqs = F.pad(freqs.detach().float(), (0, (D - d) // 2))
 
         # raw tokens of the open compression window (not rotated, NSA.py:377-380) and the caches' new row
-        run_k, rk_row = _append_rows(run_k, dtype=run_k.dtype, min_capacity=cbs)
-        run_v, rv_row = _append_rows(run_v, dtype=run_v.dtype, min_capacity=cbs)
+        run_k, rk_row = _append_rows(run_k, dtype=run_k.dtype, min_capacity=cbs, feat=D)
+        run_v, rv_row = _append_rows(run_v, dtype=run_v.dtype, min_capacity=cbs, feat=D)
         fused_run = run_k.dtype == bf16 and run_v.dtype == bf16
         if not fused_run:
-            rk_row.copy_(k)
-            rv_row.copy_(v)
-        keys, _ = _append_rows(cache_k)
-        vals, _ = _append_rows(cache_v)
+            rk_row[..., :d].copy_(k)
+            rv_row[..., :d].copy_(v)
+        keys, _ = _append_rows(cache_k, feat=D)
+        vals, _ = _append_rows(cache_v, feat=D)
 
         # one library call for the attention part of the step: rotation of q / k and the new cache rows
         # (NSA.py:384-393), compressed branch over every cached compressed key (NSA.py:396-420), block
@@ -194,24 +202,26 @@ class SparseAttention(nn.Module):
         nc = cache_ck.shape[-2]
         ck16 = cv16 = None
         if nc > 0:
-            ck16 = cache_ck if cache_ck.dtype == bf16 else cache_ck.to(bf16)
-            cv16 = cache_cv if cache_cv.dtype == bf16 else cache_cv.to(bf16)
-        merged, _, _ = ops.decode_step(q16, k16, v16, freqs, t, keys, vals, ck16, cv16, self.compress_mem_kv[0], self.compress_mem_kv[1],
+            ck16 = pad(cache_ck if cache_ck.dtype == bf16 else cache_ck.to(bf16))
+            cv16 = pad(cache_cv if cache_cv.dtype == bf16 else cache_cv.to(bf16))
+        merged, _, _ = ops.decode_step(q16, k16, v16, freqs, t, keys, vals, ck16, cv16, pad(self.compress_mem_kv[0]), pad(self.compress_mem_kv[1]),
                                        rk_row if fused_run else None, rv_row if fused_run else None, self.to_strategy_combine[0](x),
                                        per_block=B // st, block=B, num_sel=self.num_selected_blocks,
-                                       share=self.query_heads_share_selected_kv, window=self.sliding_window_size)
+                                       share=self.query_heads_share_selected_kv, window=self.sliding_window_size, scale=self.scale)
 
         # a compression window is complete: compress it, keep the overlap (NSA.py:422-441)
         ck, cv = cache_ck, cache_cv
         if run_k.shape[-2] % cbs == 0:
-            next_ck = self.k_compress((run_k + self.k_intrablock_positions)[:, :, None])
-            next_cv = self.v_compress((run_v + self.v_intrablock_positions)[:, :, None])
+            next_ck = self.k_compress((run_k[..., :d] + self.k_intrablock_positions)[:, :, None])
+            next_cv = self.v_compress((run_v[..., :d] + self.v_intrablock_positions)[:, :, None])
             run_k, run_v = run_k[..., st:, :], run_v[..., st:, :]
             ck, ck_row = _append_rows(cache_ck)
             cv, cv_row = _append_rows(cache_cv)
             ck_row.copy_(next_ck)
             cv_row.copy_(next_cv)
 
+        if D != d:
+            merged = merged.reshape(b, 1, self.heads, D)[..., :d].reshape(b, 1, self.heads * d)
         out = self.combine_heads(merged.to(x.dtype))
         if not return_cache:
             return out

@@ -27,6 +27,8 @@ SLIDING = [
     (2, 4, 1, 200, 64, 17, False),
     (1, 16, 4, 1024, 64, 64, True),
     (1, 6, 2, 200, 64, 32, True),         # G=3: not a power of two (padded with zero heads)
+    (1, 4, 2, 150, 32, 20, True),         # dim_head 32 (zero-padded to 64)
+    (1, 2, 1, 150, 96, 20, False),        # dim_head 96 (-> 128)
 ]
 
 
@@ -65,6 +67,8 @@ COMPRESS = [
     (1, 6, 2, 200, 64, 4, 16, 1, True, True),        # G=3, shared selection: the group mean must be over 3 heads
     (1, 6, 2, 200, 64, 4, 16, 1, True, False),       # G=3, per-head selection
     (1, 12, 2, 100, 64, 4, 20, 1, True, True),       # G=6 with npf 5
+    (1, 4, 2, 200, 32, 4, 16, 1, True, True),        # dim_head 32
+    (1, 4, 2, 200, 96, 8, 16, 2, True, False),       # dim_head 96
 ]
 
 

@@ -56,6 +56,11 @@ CONFIGS = [
     # 128-token selection blocks (two 64-key sub-blocks per slot in the kernels)
     dict(dim=128, dim_head=64, heads=4, kv_heads=2, sliding_window_size=32, compress_block_size=32,
          compress_block_sliding_stride=16, selection_block_size=128, num_selected_blocks=2, causal=True, use_diff_topk=True),
+    # head dimensions the kernels are not compiled for (zero-padded to 64 / 128)
+    dict(dim=128, dim_head=32, heads=4, kv_heads=2, sliding_window_size=32, compress_block_size=16,
+         compress_block_sliding_stride=8, selection_block_size=16, num_selected_blocks=3, causal=True, use_diff_topk=True),
+    dict(dim=192, dim_head=96, heads=2, kv_heads=1, sliding_window_size=32, compress_block_size=16,
+         compress_block_sliding_stride=8, selection_block_size=32, num_selected_blocks=2, causal=True),
     # 6 query heads over 2 kv heads: a group of 3
     dict(dim=192, dim_head=64, heads=6, kv_heads=2, sliding_window_size=32, compress_block_size=16,
          compress_block_sliding_stride=8, selection_block_size=16, num_selected_blocks=3, causal=True, use_diff_topk=True),

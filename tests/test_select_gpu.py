@@ -52,6 +52,9 @@ CASES = [
     (1, 8, 2, 1000, 64, 128, 3),     # 128-key blocks: two 64-key sub-blocks per slot, ragged
     (2, 4, 2, 700, 128, 192, 2),     # 192 keys: three sub-blocks
     (1, 4, 1, 400, 64, 96, 2),       # 96 keys: two 48-key sub-blocks
+    (2, 4, 2, 200, 32, 16, 3),       # dim_head 32: zero-padded to the kernels' 64
+    (1, 4, 2, 300, 96, 32, 2),       # dim_head 96 -> 128
+    (1, 2, 1, 100, 40, 8, 2),        # dim_head 40
 ]
 
 
