@@ -94,3 +94,17 @@ def test_group_padding_round_trip():
         assert torch.equal(_unpad_groups(qp, hk, g, gp), q)
         lse = torch.randn(2, hk * gp, 7)
         assert _unpad_groups(lse, hk, g, gp).shape == (2, hk * g, 7)
+
+
+def test_append_rows_into_wider_buffers():
+    """A cache of d features moves into a buffer of `feat` >= d features (the padding stays zero) and grows in place
+    from then on."""
+    from native_sparse_attention_pytorch_amd.sparse_attention import _append_rows
+    t = torch.randn(2, 3, 5, 40).to(torch.bfloat16)
+    full, row = _append_rows(t, feat=64)
+    assert full.shape == (2, 3, 6, 64) and row.shape == (2, 3, 1, 64)
+    assert torch.equal(full[:, :, :5, :40], t) and (full[:, :, :5, 40:] == 0).all()
+    row.copy_(torch.ones_like(row))
+    again, row2 = _append_rows(full, feat=64)
+    assert again.data_ptr() == full.data_ptr() and again.shape == (2, 3, 7, 64)       # in place: same buffer
+    assert torch.equal(again[:, :, 5], torch.ones(2, 3, 64, dtype=torch.bfloat16))
