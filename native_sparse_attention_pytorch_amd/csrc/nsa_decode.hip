@@ -107,16 +107,32 @@ __device__ __forceinline__ DecodeTile decode_tile(const DecodePlan& P, int D, in
   return T;
 }
 
+// One branch of a decode step: what a launch needs besides the grid.
+struct AttendArgs {
+  DecodePlan P;
+  const __bf16 *q, *k, *v, *mem_k, *mem_v;
+  const void* idx;
+  const unsigned char* fmask;
+  float* part;
+  float* logits;
+};
+
+// Work-group (bx, blockIdx.y) of a branch: bx = index among the branch's split-K work-groups.
 template <int D>
-__global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_eu(2))) void decode_attend_kernel(const DecodePlan P_launch, const __bf16* __restrict__ q,
-                                                                          const __bf16* __restrict__ k, const __bf16* __restrict__ v,
-                                                                          const __bf16* __restrict__ mem_k, const __bf16* __restrict__ mem_v,
-                                                                          const void* __restrict__ idx, const unsigned char* __restrict__ fmask,
-                                                                          float* __restrict__ part, float* __restrict__ logits) {
+__device__ __forceinline__ void decode_attend_body(const AttendArgs& A, const int bx) {
   constexpr int KS = D / 16, DT = D / 32, RS = D + 8, RSV = D + 16;   // row reads want 4 banks per row, transpose loads 8
   constexpr int LPR = D / 8, RPI = 64 / LPR, NI = 32 / RPI;      // lanes per row, rows per load instruction, instructions per tile
-  DecodePlan P = P_launch;
+  DecodePlan P = A.P;
   resolve(P);
+  const __bf16* __restrict__ q = A.q;
+  const __bf16* __restrict__ k = A.k;
+  const __bf16* __restrict__ v = A.v;
+  const __bf16* __restrict__ mem_k = A.mem_k;
+  const __bf16* __restrict__ mem_v = A.mem_v;
+  const void* __restrict__ idx = A.idx;
+  const unsigned char* __restrict__ fmask = A.fmask;
+  float* __restrict__ part = A.part;
+  float* __restrict__ logits = A.logits;
   __shared__ __align__(16) __bf16 kv_s[kDecodeWaves][2][32 * RSV];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_ = lane & 31, h = lane >> 5;
   const int lr = lane / LPR, lc = lane % LPR;
@@ -125,7 +141,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_
   const int ug = blockIdx.y, b = ug / P.units, u = ug % P.units;
   const int hk = (P.units == P.hk) ? u : u / P.g;
   const int head0 = (P.units == P.hk) ? u * P.g : u;
-  const int wid = blockIdx.x * kDecodeWaves + wave, nw = P.nsplit * kDecodeWaves;
+  const int wid = bx * kDecodeWaves + wave, nw = P.nsplit * kDecodeWaves;
 
   bf16x8 Qf[KS];
   {
@@ -226,6 +242,19 @@ __global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_
         *reinterpret_cast<floatx4*>(o + 32 * dt + 8 * i4 + 4 * h) = w;
       }
   }
+}
+
+template <int D>
+__global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_eu(2))) void decode_attend_kernel(const AttendArgs A) {
+  decode_attend_body<D>(A, blockIdx.x);
+}
+
+// Two independent branches of a step (the compressed keys and the sliding window) in one launch: the work-groups of the
+// second follow those of the first along x, so the short branch fills the chip while the long one drains.
+template <int D>
+__global__ __launch_bounds__(64 * kDecodeWaves) __attribute__((amdgpu_waves_per_eu(2))) void decode_attend_pair_kernel(const AttendArgs A, const AttendArgs B) {
+  if ((int)blockIdx.x < A.P.nsplit) decode_attend_body<D>(A, blockIdx.x);
+  else decode_attend_body<D>(B, blockIdx.x - A.P.nsplit);
 }
 
 // Log-sum-exp merge of the split-K partials of head (b, head) of one branch by a work-group of D threads: the
@@ -368,24 +397,47 @@ static int make_decode_plan(const nsa_decode_desc* dsc, DecodePlan& P) {
   return 0;
 }
 
-static int launch_attend(const DecodePlan& P, const void* q, const void* k, const void* v, const void* mem_k, const void* mem_v, const void* idx,
-                         const uint8_t* fmask, void* ws, size_t ws_bytes, void* out, float* logits, void* stream) {
+static int check_attend(const DecodePlan& P, const void* q, const void* k, const void* v, const void* mem_k, const void* mem_v,
+                        const void* idx, const uint8_t* fmask, void* ws, size_t ws_bytes) {
   if (!q || !ws) return NSA_E_ARG;
   if (P.mode == 0 && ((P.count > 0 && (!k || !v)) || (P.mem > 0 && (!mem_k || !mem_v)))) return NSA_E_ARG;
   if (P.mode == 1 && (!k || !v || (P.S > 0 && (!idx || !fmask)))) return NSA_E_ARG;
   if (ws_bytes < (size_t)P.b * P.units * P.nparts * P.rec * sizeof(float)) return NSA_E_WORKSPACE;
+  return 0;
+}
+
+static AttendArgs attend_args(const DecodePlan& P, const void* q, const void* k, const void* v, const void* mem_k, const void* mem_v,
+                              const void* idx, const uint8_t* fmask, void* ws, float* logits) {
+  return AttendArgs{P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (const __bf16*)mem_k, (const __bf16*)mem_v, idx, fmask, (float*)ws, logits};
+}
+
+static int launch_attend(const DecodePlan& P, const void* q, const void* k, const void* v, const void* mem_k, const void* mem_v, const void* idx,
+                         const uint8_t* fmask, void* ws, size_t ws_bytes, void* out, float* logits, void* stream) {
+  if (int e = check_attend(P, q, k, v, mem_k, mem_v, idx, fmask, ws, ws_bytes)) return e;
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(P.nsplit, P.b * P.units);
   const int heads = P.b * P.hk * P.g;
+  const AttendArgs A = attend_args(P, q, k, v, mem_k, mem_v, idx, fmask, ws, logits);
   if (P.d == 64) {
-    hipLaunchKernelGGL((decode_attend_kernel<64>), grid, dim3(64 * kDecodeWaves), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
-                       (const __bf16*)mem_k, (const __bf16*)mem_v, idx, fmask, (float*)ws, logits);
+    hipLaunchKernelGGL((decode_attend_kernel<64>), grid, dim3(64 * kDecodeWaves), 0, st, A);
     if (out) hipLaunchKernelGGL((decode_merge_kernel<64>), dim3(heads), dim3(64), 0, st, P, (const float*)ws, (__bf16*)out);
   } else {
-    hipLaunchKernelGGL((decode_attend_kernel<128>), grid, dim3(64 * kDecodeWaves), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
-                       (const __bf16*)mem_k, (const __bf16*)mem_v, idx, fmask, (float*)ws, logits);
+    hipLaunchKernelGGL((decode_attend_kernel<128>), grid, dim3(64 * kDecodeWaves), 0, st, A);
     if (out) hipLaunchKernelGGL((decode_merge_kernel<128>), dim3(heads), dim3(128), 0, st, P, (const float*)ws, (__bf16*)out);
   }
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
+
+// two range branches over the same (batch, kv head) units in one launch; partials only (merged later by the combine kernel)
+static int launch_attend_pair(const AttendArgs& A, size_t wsa_bytes, const AttendArgs& B, size_t wsb_bytes, void* stream) {
+  if (int e = check_attend(A.P, A.q, A.k, A.v, A.mem_k, A.mem_v, A.idx, A.fmask, A.part, wsa_bytes)) return e;
+  if (int e = check_attend(B.P, B.q, B.k, B.v, B.mem_k, B.mem_v, B.idx, B.fmask, B.part, wsb_bytes)) return e;
+  if (A.P.b * A.P.units != B.P.b * B.P.units || A.P.d != B.P.d) return NSA_E_ARG;
+  const dim3 grid(A.P.nsplit + B.P.nsplit, A.P.b * A.P.units);
+  hipStream_t st = (hipStream_t)stream;
+  if (A.P.d == 64) hipLaunchKernelGGL((decode_attend_pair_kernel<64>), grid, dim3(64 * kDecodeWaves), 0, st, A, B);
+  else hipLaunchKernelGGL((decode_attend_pair_kernel<128>), grid, dim3(64 * kDecodeWaves), 0, st, A, B);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
 }
@@ -555,9 +607,17 @@ extern "C" int nsa_decode_step(const nsa_decode_step_desc* d, const void* q, con
     return e;
   const bool has_c = d->num_compressed > 0;
   float* logits = (float*)(w + L.off_logits);
-  if (has_c)
-    if (int e = nsa_decode_attend(&L.c, q, ck_cache, cv_cache, mem_k, mem_v, nullptr, nullptr, w + L.off_wsc, L.wsc, nullptr, logits, stream))
+  // the compressed range and the sliding window are independent of each other: one launch for both
+  DecodePlan Pc_{}, Ps_;
+  if (int e = make_decode_plan(&L.s, Ps_)) return e;
+  if (has_c) {
+    if (int e = make_decode_plan(&L.c, Pc_)) return e;
+    if (int e = launch_attend_pair(attend_args(Pc_, q, ck_cache, cv_cache, mem_k, mem_v, nullptr, nullptr, w + L.off_wsc, logits), L.wsc,
+                                   attend_args(Ps_, rq, k_cache, v_cache, nullptr, nullptr, nullptr, nullptr, w + L.off_wss, nullptr), L.wss, stream))
       return e;
+  } else if (int e = launch_attend(Ps_, rq, k_cache, v_cache, nullptr, nullptr, nullptr, nullptr, w + L.off_wss, L.wss, nullptr, nullptr, stream)) {
+    return e;
+  }
   int32_t* idx = (int32_t*)(w + L.off_idx);
   uint8_t* fm = (uint8_t*)(w + L.off_fm);
   if (L.k > 0)
@@ -566,8 +626,6 @@ extern "C" int nsa_decode_step(const nsa_decode_step_desc* d, const void* q, con
       return e;
   if (int e = nsa_decode_attend(&L.f, rq, k_cache, v_cache, nullptr, nullptr, L.k > 0 ? idx : nullptr, L.k > 0 ? fm : nullptr, w + L.off_wsf,
                                 L.wsf, nullptr, nullptr, stream))
-    return e;
-  if (int e = nsa_decode_attend(&L.s, rq, k_cache, v_cache, nullptr, nullptr, nullptr, nullptr, w + L.off_wss, L.wss, nullptr, nullptr, stream))
     return e;
   return nsa_decode_combine(has_c ? &L.c : nullptr, has_c ? w + L.off_wsc : nullptr, &L.f, w + L.off_wsf, &L.s, w + L.off_wss, gate_logits, out,
                             stream);
@@ -617,8 +675,13 @@ extern "C" int nsa_decode_step_dyn(const nsa_decode_step_desc* cap, int32_t* sta
                               k_cache, cap->kc_stride, v_cache, cap->vc_stride, k_run, krun_s, v_run, vrun_s, run_ring, cap->pos, state, stream))
     return e;
   float* logits = (float*)(w + L.off_logits);
-  if (has_c)
-    if (int e = launch_attend(Pc, q, ck_cache, cv_cache, mem_k, mem_v, nullptr, nullptr, w + L.off_wsc, L.wsc, nullptr, logits, stream)) return e;
+  if (has_c) {
+    if (int e = launch_attend_pair(attend_args(Pc, q, ck_cache, cv_cache, mem_k, mem_v, nullptr, nullptr, w + L.off_wsc, logits), L.wsc,
+                                   attend_args(Ps, rq, k_cache, v_cache, nullptr, nullptr, nullptr, nullptr, w + L.off_wss, nullptr), L.wss, stream))
+      return e;
+  } else if (int e = launch_attend(Ps, rq, k_cache, v_cache, nullptr, nullptr, nullptr, nullptr, w + L.off_wss, L.wss, nullptr, nullptr, stream)) {
+    return e;
+  }
   int32_t* idx = (int32_t*)(w + L.off_idx);
   uint8_t* fm = (uint8_t*)(w + L.off_fm);
   if (L.k > 0)
@@ -628,7 +691,6 @@ extern "C" int nsa_decode_step_dyn(const nsa_decode_step_desc* cap, int32_t* sta
   if (int e = launch_attend(Pf, rq, k_cache, v_cache, nullptr, nullptr, L.k > 0 ? idx : nullptr, L.k > 0 ? fm : nullptr, w + L.off_wsf, L.wsf,
                             nullptr, nullptr, stream))
     return e;
-  if (int e = launch_attend(Ps, rq, k_cache, v_cache, nullptr, nullptr, nullptr, nullptr, w + L.off_wss, L.wss, nullptr, nullptr, stream)) return e;
   const DecodePlan* pp[3] = {&Pc, &Pf, &Ps};
   const void* wsp[3] = {has_c ? w + L.off_wsc : nullptr, w + L.off_wsf, w + L.off_wss};
   if (int e = launch_combine(pp, wsp, gate_logits, gate_row_stride, gate_bias, out, advance ? state : nullptr, stream)) return e;
