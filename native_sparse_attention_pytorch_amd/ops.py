@@ -239,10 +239,20 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     if kv_heads != sel_heads:                         # per-query-head selection: TRI.py:1961-1962
         g = q_heads // kv_heads
         fk, fv = fk.repeat_interleave(g, dim=1), fv.repeat_interleave(g, dim=1)
+    n = fq.shape[2]
+    idx_in, fm_in, sc_in = selected_block_indices, fmask, sel_scale
+    if block_size > 64 and n % block_size:
+        # Sub-blocks that lie wholly past the sequence end would drop out of the kernel's block grid, while the reference
+        # counts a selected block's zero padding (logit 0, value 0: NSA.py:744-752).  Pad to whole blocks first, as it does.
+        extra = block_size - n % block_size
+        padn = lambda t, value=0: torch.nn.functional.pad(t, (0, 0, 0, extra), value=value)
+        fq, fk, fv = padn(fq), padn(fk), padn(fv)
+        idx_in, fm_in = padn(idx_in), padn(fm_in.bool(), False)
+        sc_in = None if sc_in is None else padn(sc_in, 1.0)
     qp, g0, gp0 = _pad_groups(fq, fk.shape[1])
-    idx_k, fm_k, sc_k, block_k = _split_blocks(selected_block_indices, fmask, sel_scale, int(block_size), fq.shape[2], bool(include_block_causal))
+    idx_k, fm_k, sc_k, block_k = _split_blocks(idx_in, fm_in, sc_in, int(block_size), fq.shape[2], bool(include_block_causal))
     out, lse, _ = select_fwd(qp, fk, fv, idx_k, fm_k, sc_k, block_k, bool(include_block_causal), float(scale))
-    out, lse = _unpad_groups(out, fk.shape[1], g0, gp0)[..., :d_head], _unpad_groups(lse, fk.shape[1], g0, gp0)
+    out, lse = _unpad_groups(out, fk.shape[1], g0, gp0)[:, :, :n, :d_head], _unpad_groups(lse, fk.shape[1], g0, gp0)[:, :, :n]
     fv = fv_given if kv_heads == sel_heads else fv_given.repeat_interleave(q_heads // kv_heads, dim=1)
     if not include_block_causal and selected_block_indices.shape[-1] > 0:
         # A query whose slots are all dead attends nothing in the kernel.  The reference's torch

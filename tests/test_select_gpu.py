@@ -103,6 +103,28 @@ def test_select_reference_script_contract():
     assert_close(kg.grad, kr.grad, 2e-2 * kr.grad.abs().max().item(), 5e-2, "dk")
 
 
+def test_select_large_blocks_non_causal_ragged():
+    """Blocks of 192 keys (three sub-blocks in the kernels) without the causal own block, ragged sequence: a selected
+    last block counts its zero padding past the sequence end, sub-blocks that lie wholly in the padding included."""
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    b, hq, hk, n, d, B, S = 2, 6, 3, 468, 64, 192, 2
+    q, k, v, do = _inputs(b, hq, hk, n, d, seed=31)
+    g = torch.Generator().manual_seed(32)
+    idx = torch.randint(0, 3, (b, hk, n, S), generator=g)
+    msk = torch.rand(b, hk, n, S, generator=g) < 0.8
+    msk[..., 0] = True
+    qr, kr, vr = (t.float().requires_grad_() for t in (q, k, v))
+    ref = O.select_attend(qr, kr, vr, idx, msk, B, causal=False)
+    (ref * do.float()).sum().backward()
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    out = native_sparse_attend(qg, kg, vg, B, idx.to(DEV), msk.to(DEV), include_block_causal=False)
+    (out.float() * do.to(DEV).float()).sum().backward()
+    torch.cuda.synchronize()
+    assert_close(out, ref, 2e-2, 1e-2, "out")
+    for name, got, want in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
+        assert_close(got, want, 2e-2 * want.abs().max().item(), 5e-2, name)
+
+
 def test_select_gate_gradient_matches_oracle():
     """sel_scale (straight-through top-k gates, value 1): its gradient against the oracle's
     gather path with gates multiplying the selected keys (NSA.py:793-797); tolerance of
