@@ -613,15 +613,20 @@ __global__ __launch_bounds__(256) void dense_bwd_dkv_reduce_kernel(const DensePl
   const int keys = min(kBK, P.krows - kBK * T);
   const float* base = part + ((size_t)bh * P.key_tiles + T) * P.chunks * (2 * kBK * D);
   constexpr int CPR = D / 4;
+  // the chunks that hold queries for this tile are consecutive; only those were written
+  int clo = P.chunks, chi = 0;
+  for (int c = 0; c < P.chunks; ++c) {
+    int qlo, qhi, c0, c1;
+    chunk_range(P, T, c, qlo, qhi, c0, c1);
+    if (c0 < c1) { clo = min(clo, c); chi = c + 1; }
+  }
   for (int e = threadIdx.x; e < 2 * keys * CPR; e += 256) {
     const int which = e / (keys * CPR), rem = e % (keys * CPR);
     const int key = rem / CPR, dd = (rem % CPR) * 4;
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int c = 0; c < P.chunks; ++c) {
-      int qlo, qhi, c0, c1;
-      chunk_range(P, T, c, qlo, qhi, c0, c1);
-      if (c0 < c1) acc += *reinterpret_cast<const floatx4*>(base + (size_t)c * (2 * kBK * D) + (size_t)which * kBK * D + (size_t)key * D + dd);
-    }
+    const float* src = base + (size_t)which * kBK * D + (size_t)key * D + dd;
+#pragma unroll 8
+    for (int c = clo; c < chi; ++c) acc += __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(src + (size_t)c * (2 * kBK * D)));
     const float s = which == 0 ? P.scale : 1.0f;
     __bf16* dst = (which == 0 ? dk : dv) + ((size_t)bh * P.krows + (size_t)kBK * T + key) * D + dd;
     store4_bf16(dst, acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s);
