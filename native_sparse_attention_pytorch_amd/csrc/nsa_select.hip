@@ -965,18 +965,26 @@ __global__ __launch_bounds__(256) void sel_bwd_dkv_reduce_kernel(const SelPlan P
   const int u0 = unit_off[j], u1 = unit_off[j + 1];
   const float* part = reinterpret_cast<const float*>(bws + P.off_dkvpart) + (size_t)bh * P.ub_kv * (2 * 32 * KT * D);
   const int keys = min(P.B, P.n - j * P.B);
-  constexpr int CPR = D / 4;
-  for (int c = threadIdx.x; c < 2 * keys * CPR; c += 256) {
-    const int which = c / (keys * CPR), rem = c % (keys * CPR);
+  // a unit's partial is 2 x ROWS x D floats in the order (dk | dv, key, feature): the work group reads
+  // it as consecutive float4 and every thread keeps its N slices of the sum in registers
+  constexpr int CPR = D / 4, ROWS = 32 * KT, UNIT = 2 * ROWS * D, N = 2 * ROWS * CPR / 256;
+  floatx4 acc[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int u = u0; u < u1; ++u) {
+    const floatx4* src = reinterpret_cast<const floatx4*>(part + (size_t)u * UNIT) + threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < N; ++i) acc[i] += __builtin_nontemporal_load(src + 256 * i);
+  }
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const int e = threadIdx.x + 256 * i;
+    const int which = e / (ROWS * CPR), rem = e % (ROWS * CPR);
     const int key = rem / CPR, dd = (rem % CPR) * 4;
-    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int u = u0; u < u1; ++u) {
-      const floatx4 x = *reinterpret_cast<const floatx4*>(part + (size_t)u * (2 * 32 * KT * D) + (size_t)which * (32 * KT * D) + (size_t)key * D + dd);
-      acc += x;
-    }
+    if (key >= keys) continue;
     const float s = which == 0 ? P.scale : 1.0f;
     __bf16* dst = (which == 0 ? dk : dv) + (((size_t)bh * P.n) + (size_t)j * P.B + key) * D + dd;
-    store4_bf16(dst, acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s);
+    store4_bf16(dst, acc[i][0] * s, acc[i][1] * s, acc[i][2] * s, acc[i][3] * s);
   }
 }
 
