@@ -101,7 +101,13 @@ __device__ __forceinline__ bf16x8 lds_row_operand(const __bf16* tile_s, int RS, 
 
 // s_waitcnt vmcnt(0) (expcnt / lgkmcnt left at their maxima): all outstanding global loads
 // and stores of this wave have completed.
-__device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// Wait for every outstanding vector memory operation.  The plain s_waitcnt builtin does not order
+// loads around itself (the compiler moved gathers issued before it to after it), hence the fence.
+__device__ __forceinline__ void wait_all_loads() {
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);      // the builtin, not inline assembly: the compiler's own wait counting sees it
+  __builtin_amdgcn_sched_barrier(0);
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

@@ -451,6 +451,10 @@ __device__ __forceinline__ void chunk_of(const DensePlan& P, int x, int& T, int&
   chunk_range(P, T, c, qlo, qhi, c0, c1);
 }
 
+#ifndef NSA_DKV_STAGES
+#define NSA_DKV_STAGES 1      // measured on MI355X (compressed branch, seq 32k, d 128): 1, 2 or 3 tiles ahead all 4.7 ms
+#endif
+
 // dK/dV of one 64-row tile of k/v over one chunk of the queries that can see it (key-stationary);
 // wave kt owns rows 32kt .. 32kt+31 of the tile.  Rows are indexed from the start of the arrays,
 // so in stride mode row r is visible to query i iff r <= hi(i) + mem.
@@ -499,49 +503,44 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
   const __bf16* gbase = dout + b * P.sdo[0] + (long)(hk * P.g) * P.sdo[1];
   constexpr int CPR = D / 8, RPI = 64 / CPR, NT = 32 / RPI;
 
-  // wave 0 gathers the tile's Q rows, wave 1 its dO rows (coalesced), one tile ahead
-  bf16x8 raw[NT];
-  auto issue = [&](int i0) {
+  // wave 0 gathers the tile's Q rows, wave 1 its dO rows (coalesced), NSA_DKV_STAGES tiles ahead: at
+  // one wave per SIMD the depth of this pipeline is the only latency hiding there is
+  struct Stage { bf16x8 raw[NT]; float lse_r, del_r; };
+  auto issue = [&](Stage& st, int i0) {
     const __bf16* base = kt == 0 ? qbase : gbase;
     const long sh = kt == 0 ? P.sq[1] : P.sdo[1], sn = kt == 0 ? P.sq[2] : P.sdo[2];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int rr = t * RPI + lane / CPR;
       const int qi = min(i0 + (rr >> P.lg), P.n - 1);
-      raw[t] = load8(base + (long)(rr & (P.g - 1)) * sh + (long)qi * sn + 8 * (lane % CPR));
+      st.raw[t] = load8(base + (long)(rr & (P.g - 1)) * sh + (long)qi * sn + 8 * (lane % CPR));
     }
-  };
-  issue(c0);
-  float lse_r, del_r;
-  {
-    const int qi = min(c0 + pq, P.n - 1);
+    const int qi = min(i0 + pq, P.n - 1);
     const long srow = ((long)b * P.hkv * P.g + hq) * P.n + qi;
-    lse_r = lse[srow] * kLog2e; del_r = delta[srow];
-  }
+    st.lse_r = lse[srow]; st.del_r = delta[srow];        // scaled where it is used: arithmetic here would wait for the loads
+  };
+  constexpr int NS = NSA_DKV_STAGES;
+  Stage stg[NS];
+#pragma unroll
+  for (int s2 = 0; s2 < NS; ++s2) issue(stg[s2], c0 + s2 * ppt);
   wait_all_loads();
-  for (int i0 = c0; i0 < c1; i0 += ppt) {
+  auto step = [&](int i0, Stage& cur) {
     const bool valid = i0 + pq < c1;
     const int i = min(i0 + pq, P.n - 1);
     {
       __bf16* dst = kt == 0 ? xq_s : xg_s;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) *reinterpret_cast<bf16x8*>(dst + (t * RPI + lane / CPR) * RS + 8 * (lane % CPR)) = raw[t];
+      for (int t = 0; t < NT; ++t) *reinterpret_cast<bf16x8*>(dst + (t * RPI + lane / CPR) * RS + 8 * (lane % CPR)) = cur.raw[t];
     }
     if (kt == 0 && h == 0) {
-      lse_s[n_] = valid ? lse_r : INFINITY;                // +inf: a padding row gets p = 0
-      del_s[n_] = del_r;
+      lse_s[n_] = valid ? cur.lse_r * kLog2e : INFINITY;   // +inf: a padding row gets p = 0
+      del_s[n_] = cur.del_r;
       const Interval me = visible_range(P, i);
       lo_s[n_] = P.mode == 0 ? me.lo : 0;
       hi_s[n_] = P.mode == 0 ? me.hi : me.hi + P.mem;
     }
     __syncthreads();
-    issue(i0 + ppt);
-    float lse_n, del_n;
-    {
-      const int qi = min(i0 + ppt + pq, P.n - 1);
-      const long srow = ((long)b * P.hkv * P.g + hq) * P.n + qi;
-      lse_n = lse[srow] * kLog2e; del_n = delta[srow];
-    }
+    issue(cur, i0 + NS * ppt);                             // the freed stage takes the tile NS steps ahead
     __builtin_amdgcn_sched_barrier(0);
 
     // the whole tile's arithmetic as one straight-line block per variant (masked / unmasked), so that
@@ -590,8 +589,21 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
       else tile_math(std::true_type{});
     }
     __syncthreads();
-    lse_r = lse_n; del_r = del_n;
+  };
+  // whole rounds of NS tiles first: a round's steps are unconditional, so the wait before each step's
+  // commit counts exactly the loads issued after that stage's
+  int i0 = c0;
+  if (i0 + (NS - 1) * ppt < c1) {
+    wait_all_loads();      // again: the compiler sinks the later stages' first loads to here, past the wait above
+    do {
+#pragma unroll
+      for (int s2 = 0; s2 < NS; ++s2) step(i0 + s2 * ppt, stg[s2]);
+      i0 += NS * ppt;
+    } while (i0 + (NS - 1) * ppt < c1);
   }
+#pragma unroll
+  for (int s2 = 0; s2 < NS - 1; ++s2)
+    if (i0 + s2 * ppt < c1) step(i0 + s2 * ppt, stg[s2]);
   // partial [bh][tile][chunk][2][64][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][row 32kt + n_]
   float* pk = part + (((size_t)bh * P.key_tiles + T) * P.chunks + c) * (2 * kBK * D) + (size_t)(32 * kt + n_) * D + 4 * h;
   float* pv = pk + kBK * D;

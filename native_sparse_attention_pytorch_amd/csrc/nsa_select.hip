@@ -347,7 +347,7 @@ __device__ __forceinline__ void store_tile_rows(const floatx16 (&acc)[D / 32], f
 // ------------------------------------------------------------------------------- forward
 
 #ifndef NSA_FWD_STAGES
-#define NSA_FWD_STAGES 1      // measured on MI355X (seq 32k, d 128): 1 stage 1.69 ms, 2 or 3 stages 1.77 ms
+#define NSA_FWD_STAGES 1      // measured on MI355X (seq 32k, d 128): 1 stage 1.56 ms, 2 stages 1.60 ms
 #endif
 template <int D, int KT>
 __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
@@ -418,9 +418,12 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
     const RowInfo r = cur.r;
     commit_tile<D>(cur.raw, xq_s, RS, lane);
     __syncthreads();
+    // the list entry is fetched before the row gathers that follow it: the wait for an entry (memory
+    // operations retire in order) then never covers the gathers issued in the same step
     cur.r = decode_entry(P, ui, e_n, n_);
-    issue_tile_loads<D>(cur.raw, qbase, P.sq[1], P.sq[2], cur.r.i, P.g - 1, lane);
     e_n = fetch_entry(P, list, ui, vt + (NS + 1) * ppt, n_);
+    __builtin_amdgcn_sched_barrier(0);
+    issue_tile_loads<D>(cur.raw, qbase, P.sq[1], P.sq[2], cur.r.i, P.g - 1, lane);
     __builtin_amdgcn_sched_barrier(0);
 
     bf16x8 Qf[KS];
@@ -477,11 +480,20 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
       if (h == 0) lsepart[row] = (mx + fast_log2(l)) * kLn2;
     }
   };
-  for (int vt = ui.v0; vt < ui.v1; vt += NS * ppt) {
+  // whole rounds of NS tiles first: their steps are unconditional, so each wait counts exactly the
+  // memory operations issued after the loads it needs
+  int vt = ui.v0;
+  if (vt + (NS - 1) * ppt < ui.v1) {
+    wait_all_loads();      // again: the compiler sinks the later stages' first loads to here, past the wait above
+    do {
 #pragma unroll
-    for (int s2 = 0; s2 < NS; ++s2)
-      if (vt + s2 * ppt < ui.v1) step(vt + s2 * ppt, stg[s2]);
+      for (int s2 = 0; s2 < NS; ++s2) step(vt + s2 * ppt, stg[s2]);
+      vt += NS * ppt;
+    } while (vt + (NS - 1) * ppt < ui.v1);
   }
+#pragma unroll
+  for (int s2 = 0; s2 < NS - 1; ++s2)
+    if (vt + s2 * ppt < ui.v1) step(vt + s2 * ppt, stg[s2]);
 }
 
 // live-slot bitmask of query (bh, i): bit s < S = selected slot s, bit S = own block
@@ -754,7 +766,7 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 // transpose load (K block row-major in LDS, loaded once per unit), each wave taking half of the
 // features, and the finished 32 x D tile leaves through coalesced row stores.
 #ifndef NSA_BWD_STAGES
-#define NSA_BWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1 stage 3.86 ms, 2: 3.44, 3: 3.53, 4: 3.60
+#define NSA_BWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1 stage 3.8 ms, 2 and 3 stages 3.27 ms
 #endif
 template <int D, int KT, bool FUSE_DQ>
 __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1))) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
@@ -829,7 +841,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
       issue_tile_loads<D>(st.raw[0], load_q ? qbase : gbase, load_q ? P.sq[1] : P.so[1], load_q ? P.sq[2] : P.so[2], rr.i, P.g - 1, lane);
     }
     const size_t srow = ((size_t)b * HQ + hk * P.g + rr.g) * P.n + rr.i;
-    st.lse_r = lse[srow] * kLog2e;
+    st.lse_r = lse[srow];                                  // scaled where it is used: arithmetic here would wait for the loads
     st.del_r = delta[srow];
   };
   constexpr int NS = KT == 1 ? 1 : NSA_BWD_STAGES;      // a single wave gathers both tiles: no registers for a second stage
@@ -849,7 +861,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
       commit_tile<D>(cur.raw[0], load_q ? xq_s : xg_s, RS, lane);
     }
     if (kt == 0 && h == 0) {
-      lse_s[n_] = r.valid ? cur.lse_r : INFINITY;          // +inf: a padding row gets p = 0
+      lse_s[n_] = r.valid ? cur.lse_r * kLog2e : INFINITY; // +inf: a padding row gets p = 0
       del_s[n_] = cur.del_r;
       lim_s[n_] = r.lim;
       if (FUSE_DQ) row_s[n_] = r.valid ? (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g : P.prow;
@@ -857,8 +869,11 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
     __syncthreads();
 
     // the freed stage takes the loads of the tile two steps ahead; fetch the entry of the tile after that
-    issue(cur, decode_entry(P, ui, e_n, n_));
+    // (the entry first, then the gathers: see the forward walk)
+    const RowInfo rn = decode_entry(P, ui, e_n, n_);
     e_n = fetch_entry(P, list, ui, vt + (NS + 1) * ppt, n_);
+    __builtin_amdgcn_sched_barrier(0);
+    issue(cur, rn);
     __builtin_amdgcn_sched_barrier(0);
 
     floatx16 Sa = zero_acc(), Pa = zero_acc();
@@ -934,11 +949,20 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
       __syncthreads();
     }
   };
-  for (int vt = ui.v0; vt < ui.v1; vt += NS * ppt) {
+  // whole rounds of NS tiles first: their steps are unconditional, so each wait counts exactly the
+  // memory operations issued after the loads it needs
+  int vt = ui.v0;
+  if (vt + (NS - 1) * ppt < ui.v1) {
+    wait_all_loads();      // again: the compiler sinks the later stages' first loads to here, past the wait above
+    do {
 #pragma unroll
-    for (int s2 = 0; s2 < NS; ++s2)
-      if (vt + s2 * ppt < ui.v1) step(vt + s2 * ppt, stg[s2]);
+      for (int s2 = 0; s2 < NS; ++s2) step(vt + s2 * ppt, stg[s2]);
+      vt += NS * ppt;
+    } while (vt + (NS - 1) * ppt < ui.v1);
   }
+#pragma unroll
+  for (int s2 = 0; s2 < NS - 1; ++s2)
+    if (vt + s2 * ppt < ui.v1) step(vt + s2 * ppt, stg[s2]);
 
   // partial [unit][2][32*KT keys][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][key kl]
   float* part = reinterpret_cast<float*>(bws + P.off_dkvpart) + ((size_t)bh * P.ub_kv + u) * (2 * 32 * KT * D);
