@@ -116,6 +116,7 @@ __device__ __forceinline__ CellInfo cell_info(const SelPlan& P, const char* iws,
 // unit_off[t][bh][cell] = exclusive prefix sum of ceil(pairs(cell) / chunk[t]), cells phase-major
 __global__ __launch_bounds__(256) void sel_units_kernel(const SelPlan P, char* iws) {
   __shared__ int part[256];
+  __shared__ int total_s;
   const int bh = blockIdx.x, t = blockIdx.y, tid = threadIdx.x;
   const int cells = P.np[t] * P.W;
   int* uo = reinterpret_cast<int*>(iws + P.off_unit[t]) + (size_t)bh * (cells + 1);
@@ -132,13 +133,27 @@ __global__ __launch_bounds__(256) void sel_units_kernel(const SelPlan P, char* i
     int acc = 0;
     for (int k = 0; k < 256; ++k) { const int v = part[k]; part[k] = acc; acc += v; }
     uo[cells] = acc;
+    total_s = acc;
   }
   __syncthreads();
+  // besides the prefix sums, one record per unit: a walk's work-group then finds its unit with one
+  // load instead of a binary search over the prefix sums (a dozen dependent loads at one wave per SIMD)
+  int4* rec = reinterpret_cast<int4*>(iws + P.off_urec[t]) + (size_t)bh * P.ub[t] * 2;
   int acc = part[tid];
   for (int c = lo; c < hi; ++c) {
-    const CellInfo ci = cell_info(P, iws, bh, t, c / P.W, c % P.W);
+    const int j = c % P.W;
+    const CellInfo ci = cell_info(P, iws, bh, t, c / P.W, j);
     uo[c] = acc;
-    acc += (ci.own + ci.count + P.chunk[t] - 1) / P.chunk[t];
+    const int L = ci.own + ci.count, nu = (L + P.chunk[t] - 1) / P.chunk[t];
+    for (int k = 0; k < nu; ++k) {
+      rec[2 * (acc + k)] = int4{j, ci.own, ci.first, k * P.chunk[t]};
+      rec[2 * (acc + k) + 1] = int4{min(L, (k + 1) * P.chunk[t]), 0, 0, 0};
+    }
+    acc += nu;
+  }
+  for (int u = total_s + tid; u < P.ub[t]; u += 256) {       // padding units: empty range
+    rec[2 * u] = int4{0, 0, 0, 0};
+    rec[2 * u + 1] = int4{0, 0, 0, 0};
   }
 }
 
@@ -205,22 +220,13 @@ struct UnitInfo {
 // unit u of table t -> (block j, range [v0, v1) of the cell's virtual list: `own` own-block
 // positions first, then list[lst0 ...]).  Returns false for padding units.
 __device__ __forceinline__ bool locate_unit(const SelPlan& P, const char* iws, int t, int bh, int u, UnitInfo& ui) {
-  const int cells = P.np[t] * P.W;
-  const int* unit_off = reinterpret_cast<const int*>(iws + P.off_unit[t]) + (size_t)bh * (cells + 1);
-  if (u >= unit_off[cells]) return false;
-  int lo = 0, hi = cells - 1;
-  while (lo < hi) {                       // last cell with unit_off[cell] <= u (empty cells own no unit)
-    const int mid = (lo + hi + 1) >> 1;
-    if (unit_off[mid] <= u) lo = mid; else hi = mid - 1;
-  }
-  const int p = lo / P.W, j = lo % P.W;
-  const CellInfo ci = cell_info(P, iws, bh, t, p, j);
-  ui.j = j;
-  ui.own = ci.own;
-  ui.lst0 = ci.first;                     // index into the per-(batch, head) list
-  const int L = ci.own + ci.count;
-  ui.v0 = (u - unit_off[lo]) * P.chunk[t];
-  ui.v1 = min(L, ui.v0 + P.chunk[t]);
+  const int4* rec = reinterpret_cast<const int4*>(iws + P.off_urec[t]) + ((size_t)bh * P.ub[t] + u) * 2;
+  const int4 r0 = rec[0], r1 = rec[1];
+  ui.j = r0.x;
+  ui.own = r0.y;
+  ui.lst0 = r0.z;                         // index into the per-(batch, head) list
+  ui.v0 = r0.w;
+  ui.v1 = r1.x;
   return ui.v0 < ui.v1;
 }
 
@@ -365,42 +371,45 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
   if (!locate_unit(P, iws, TBL, bh, u, ui)) return;
   const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
 
+  // Set-up in three memory round trips: (1) the unit record above, (2) the first list entries, the
+  // block's K rows and its V rows, all requested before anything waits, (3) the first Q gathers,
+  // requested as soon as the entries are there and in flight while V is transposed.  At one wave
+  // per SIMD every dependent load here is exposed latency, and a unit is only a few dozen tiles.
+  const int ppt = 32 >> P.lg;
+  constexpr int NS = NSA_FWD_STAGES;
+  RawEntry e0[NS];
+#pragma unroll
+  for (int s2 = 0; s2 < NS; ++s2) e0[s2] = fetch_entry(P, list, ui, ui.v0 + s2 * ppt, n_);
+  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + NS * ppt, n_);
+  __builtin_amdgcn_sched_barrier(0);
+
   bf16x8 Kf[KT][KS];
-  bf16x8 VT[DT][KT][2];
-  {
-    bf16x8 ilo, ihi;
-    make_ident(lane, ilo, ihi);
+  bf16x8 Vraw[KT][DT][2];
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
-      const int kl = 32 * kt + n_;
-      const long key = (long)ui.j * P.B + kl;
-      const bool ok = kl < P.B && key < P.n;
-      const long keyc = ok ? key : 0;
-      const __bf16* kp = k + b * P.sk[0] + hk * P.sk[1] + keyc * P.sk[2] + 8 * h;
-      const __bf16* vp = v + b * P.sv[0] + hk * P.sv[1] + keyc * P.sv[2] + 8 * h;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int kl = 32 * kt + n_;
+    const long key = (long)ui.j * P.B + kl;
+    const bool ok = kl < P.B && key < P.n;
+    const long keyc = ok ? key : 0;
+    const __bf16* kp = k + b * P.sk[0] + hk * P.sk[1] + keyc * P.sk[2] + 8 * h;
+    const __bf16* vp = v + b * P.sv[0] + hk * P.sv[1] + keyc * P.sv[2] + 8 * h;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) Kf[kt][ks] = ok ? load8(kp + 16 * ks) : zero_frag();
+    for (int ks = 0; ks < KS; ++ks) Kf[kt][ks] = ok ? load8(kp + 16 * ks) : zero_frag();
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const bf16x8 va = ok ? load8(vp + 32 * dt) : zero_frag();
-        const bf16x8 vb = ok ? load8(vp + 32 * dt + 16) : zero_frag();
-        floatx16 t = mfma32(va, ilo, zero_acc());
-        t = mfma32(vb, ihi, t);
-        VT[dt][kt][0] = pack8(t, 0);
-        VT[dt][kt][1] = pack8(t, 8);
-      }
+    for (int dt = 0; dt < DT; ++dt) {
+      Vraw[kt][dt][0] = ok ? load8(vp + 32 * dt) : zero_frag();
+      Vraw[kt][dt][1] = ok ? load8(vp + 32 * dt + 16) : zero_frag();
     }
   }
+  __builtin_amdgcn_sched_barrier(0);
 
   __bf16* opart = reinterpret_cast<__bf16*>(fws + P.off_opart);
   float* lsepart = reinterpret_cast<float*>(fws + P.off_lsepart);
   const float sc = P.scale * kLog2e;
-  const int ppt = 32 >> P.lg;
 
   // software pipeline: NS tiles of Q rows (coalesced gathers) in flight, list entries one more tile
   // ahead; a stage's registers take the loads of the tile NS steps ahead once it is committed to LDS
   const __bf16* qbase = q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1];
-  constexpr int NS = NSA_FWD_STAGES;
   struct Stage {
     RowInfo r;
     bf16x8 raw[KS];
@@ -408,10 +417,25 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
   Stage stg[NS];
 #pragma unroll
   for (int s2 = 0; s2 < NS; ++s2) {
-    stg[s2].r = decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0 + s2 * ppt, n_), n_);
+    stg[s2].r = decode_entry(P, ui, e0[s2], n_);
     issue_tile_loads<D>(stg[s2].raw, qbase, P.sq[1], P.sq[2], stg[s2].r.i, P.g - 1, lane);
   }
-  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + NS * ppt, n_);
+  __builtin_amdgcn_sched_barrier(0);
+
+  bf16x8 VT[DT][KT][2];
+  {
+    bf16x8 ilo, ihi;
+    make_ident(lane, ilo, ihi);
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        floatx16 t = mfma32(Vraw[kt][dt][0], ilo, zero_acc());
+        t = mfma32(Vraw[kt][dt][1], ihi, t);
+        VT[dt][kt][0] = pack8(t, 0);
+        VT[dt][kt][1] = pack8(t, 8);
+      }
+  }
 
   wait_all_loads();        // enter the loop with nothing pending, so the loop itself only waits for what it needs
   auto step = [&](int vt, Stage& cur) {

@@ -18,6 +18,7 @@ struct SelPlan {
   // possible).
   int chunk[3], phase[3], np[3], ub[3];
   size_t off_unit[3];
+  size_t off_urec[3];        // per (batch*kv head, unit) a record of 8 ints: block, own, list start, v0, v1
   int ub_kv;                 // = ub[2]
   long list_cap;             // inverse-index entries reserved per (batch, kv head)
   size_t prow;               // number of partial rows; row `prow` is a spare that padding rows write to
@@ -79,6 +80,7 @@ static inline int make_plan(const nsa_select_desc* d, SelPlan& P) {
   P.off_cnt = o;    o = align_up(o + (size_t)bh * P.nch * P.W * 4);
   P.off_blk = o;    o = align_up(o + (size_t)bh * (P.W + 1) * 4);
   for (int t = 0; t < 3; ++t) { P.off_unit[t] = o; o = align_up(o + (size_t)bh * ((size_t)P.np[t] * P.W + 1) * 4); }
+  for (int t = 0; t < 3; ++t) { P.off_urec[t] = o; o = align_up(o + (size_t)bh * (size_t)P.ub[t] * 32); }
   P.off_list = o;   o = align_up(o + (size_t)bh * P.list_cap * 4);
   P.index_total = o;
 
