@@ -819,6 +819,15 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
   const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
   const bool load_q = kt == 0;                 // with two waves: wave 0 gathers Q rows, wave 1 dO rows; one wave does both
 
+  // the first list entries, then the block's K / V rows: all requested before anything waits
+  const int ppt = 32 >> P.lg;
+  constexpr int NS = KT == 1 ? 1 : NSA_BWD_STAGES;      // a single wave gathers both tiles: no registers for a second stage
+  RawEntry e0[NS];
+#pragma unroll
+  for (int s2 = 0; s2 < NS; ++s2) e0[s2] = fetch_entry(P, list, ui, ui.v0 + s2 * ppt, n_);
+  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + NS * ppt, n_);
+  __builtin_amdgcn_sched_barrier(0);
+
   bf16x8 Kf[KS], Vf[KS];
   const int kl = 32 * kt + n_;                 // this lane's key inside the block
   {
@@ -832,17 +841,13 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
       Kf[ks] = ok ? load8(kp + 16 * ks) : zero_frag();
       Vf[ks] = ok ? load8(vp + 16 * ks) : zero_frag();
     }
-    if (FUSE_DQ) {
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<bf16x8*>(kb_s + kl * RSK + 16 * ks + 8 * h) = Kf[ks];
-    }
   }
+  __builtin_amdgcn_sched_barrier(0);
   floatx16 dKa[DT], dVa[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) { dKa[dt] = zero_acc(); dVa[dt] = zero_acc(); }
 
   const float sc = P.scale * kLog2e;
-  const int ppt = 32 >> P.lg;
   const int HQ = P.hkv * P.g;
   const __bf16* qbase = q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1];
   const __bf16* gbase = dout + b * P.so[0] + (long)(hk * P.g) * P.so[1];
@@ -868,11 +873,14 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
     st.lse_r = lse[srow];                                  // scaled where it is used: arithmetic here would wait for the loads
     st.del_r = delta[srow];
   };
-  constexpr int NS = KT == 1 ? 1 : NSA_BWD_STAGES;      // a single wave gathers both tiles: no registers for a second stage
   Stage stg[NS];
 #pragma unroll
-  for (int s2 = 0; s2 < NS; ++s2) issue(stg[s2], decode_entry(P, ui, fetch_entry(P, list, ui, ui.v0 + s2 * ppt, n_), n_));
-  RawEntry e_n = fetch_entry(P, list, ui, ui.v0 + NS * ppt, n_);
+  for (int s2 = 0; s2 < NS; ++s2) issue(stg[s2], decode_entry(P, ui, e0[s2], n_));
+  __builtin_amdgcn_sched_barrier(0);
+  if (FUSE_DQ) {           // the row-major copy of the K block for dQ (waits for K, with the gathers already under way)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<bf16x8*>(kb_s + kl * RSK + 16 * ks + 8 * h) = Kf[ks];
+  }
 
   wait_all_loads();        // enter the loop with nothing pending, so the loop itself only waits for what it needs
   auto step = [&](int vt, Stage& cur) {

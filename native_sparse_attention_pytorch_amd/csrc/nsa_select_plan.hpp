@@ -6,6 +6,10 @@
 #include <stdint.h>
 #include "../../include/nsa_hip.h"
 
+#ifndef NSA_PHASE_BYTES
+#define NSA_PHASE_BYTES (1L << 22)
+#endif
+
 namespace nsa {
 
 struct SelPlan {
@@ -62,7 +66,7 @@ static inline int make_plan(const nsa_select_desc* d, SelPlan& P) {
   // work units too small, longer ones lose the L2 reuse of the gathered rows)
   const long row_bytes = (long)P.g * P.D * 2;
   long ph = 256;
-  while (ph * 2 * row_bytes <= (1L << 22) && ph < (1L << 20)) ph *= 2;
+  while (ph * 2 * row_bytes <= (long)NSA_PHASE_BYTES && ph < (1L << 20)) ph *= 2;
   P.chunk[0] = 256;  P.phase[0] = (int)ph;
   P.chunk[1] = 256;  P.phase[1] = (int)(ph > 256 ? ph / 2 : ph);
   P.chunk[2] = 1024; P.phase[2] = ((P.n + 255) / 256) * 256;
