@@ -109,7 +109,8 @@ __device__ __forceinline__ CellInfo cell_info(const SelPlan& P, const char* iws,
   CellInfo ci;
   ci.first = blk[j] + s0;
   ci.count = s1 - s0;
-  ci.own = (P.causal && (j * P.B) / P.phase[t] == p) ? min(P.B, P.n - j * P.B) : 0;
+  const long k0 = (long)j * P.B, ph0 = (long)p * P.phase[t];
+  ci.own = (P.causal && k0 >= ph0 && k0 < ph0 + P.phase[t]) ? min(P.B, P.n - j * P.B) : 0;
   return ci;
 }
 
@@ -122,10 +123,17 @@ __global__ __launch_bounds__(256) void sel_units_kernel(const SelPlan P, char* i
   int* uo = reinterpret_cast<int*>(iws + P.off_unit[t]) + (size_t)bh * (cells + 1);
   const int per = (cells + 255) / 256;
   const int lo = min(cells, tid * per), hi = min(cells, lo + per);
+  // (phase, block) of a cell are carried along instead of divided out: this kernel has few waves and
+  // is bound by its integer arithmetic; chunk[] is a power of two
+  const int csh = 31 - __clz(P.chunk[t]);
   int sum = 0;
-  for (int c = lo; c < hi; ++c) {
-    const CellInfo ci = cell_info(P, iws, bh, t, c / P.W, c % P.W);
-    sum += (ci.own + ci.count + P.chunk[t] - 1) / P.chunk[t];
+  {
+    int pp = lo / P.W, j = lo % P.W;
+    for (int c = lo; c < hi; ++c) {
+      const CellInfo ci = cell_info(P, iws, bh, t, pp, j);
+      sum += (ci.own + ci.count + P.chunk[t] - 1) >> csh;
+      if (++j == P.W) { j = 0; ++pp; }
+    }
   }
   part[tid] = sum;
   __syncthreads();
@@ -140,16 +148,19 @@ __global__ __launch_bounds__(256) void sel_units_kernel(const SelPlan P, char* i
   // load instead of a binary search over the prefix sums (a dozen dependent loads at one wave per SIMD)
   int4* rec = reinterpret_cast<int4*>(iws + P.off_urec[t]) + (size_t)bh * P.ub[t] * 2;
   int acc = part[tid];
-  for (int c = lo; c < hi; ++c) {
-    const int j = c % P.W;
-    const CellInfo ci = cell_info(P, iws, bh, t, c / P.W, j);
-    uo[c] = acc;
-    const int L = ci.own + ci.count, nu = (L + P.chunk[t] - 1) / P.chunk[t];
-    for (int k = 0; k < nu; ++k) {
-      rec[2 * (acc + k)] = int4{j, ci.own, ci.first, k * P.chunk[t]};
-      rec[2 * (acc + k) + 1] = int4{min(L, (k + 1) * P.chunk[t]), 0, 0, 0};
+  {
+    int pp = lo / P.W, j = lo % P.W;
+    for (int c = lo; c < hi; ++c) {
+      const CellInfo ci = cell_info(P, iws, bh, t, pp, j);
+      uo[c] = acc;
+      const int L = ci.own + ci.count, nu = (L + P.chunk[t] - 1) >> csh;
+      for (int k = 0; k < nu; ++k) {
+        rec[2 * (acc + k)] = int4{j, ci.own, ci.first, k << csh};
+        rec[2 * (acc + k) + 1] = int4{min(L, (k + 1) << csh), 0, 0, 0};
+      }
+      acc += nu;
+      if (++j == P.W) { j = 0; ++pp; }
     }
-    acc += nu;
   }
   for (int u = total_s + tid; u < P.ub[t]; u += 256) {       // padding units: empty range
     rec[2 * u] = int4{0, 0, 0, 0};
