@@ -92,8 +92,9 @@ __device__ __forceinline__ DecodeTile decode_tile(const DecodePlan& P, int D, in
     bool live = true;
     if (slot < P.S) {
       const long e = (long)ug * P.sstride + slot;
+      const unsigned char fm = fmask[e];              // requested together with the index: one round trip, not two
       blk = P.idx64 ? reinterpret_cast<const long*>(idx)[e] : (long)reinterpret_cast<const int*>(idx)[e];
-      live = fmask[e] != 0 && blk >= 0 && blk * P.B < P.kv_len;
+      live = (fm != 0) & (blk >= 0) & (blk * P.B < P.kv_len);
       if (!live) blk = 0;
     } else {
       blk = (P.kv_len - 1) / P.B;                     // the query's own block, up to itself
