@@ -26,6 +26,7 @@ import ctypes as C
 import torch
 
 from . import _lib
+from .ops import _kernel_dim, _pad_dim
 
 _BF16 = torch.bfloat16
 
@@ -44,12 +45,16 @@ class DecodeSession:
         (cache_k, cache_v), ((cache_ck, cache_cv), (run_k, run_v)) = cache
         if not cache_k.is_cuda:
             raise RuntimeError("DecodeSession runs on the GPU only (HIP kernels, no CPU fallback)")
-        if m.dim_head not in (64, 128):
-            raise NotImplementedError("DecodeSession needs dim_head 64 or 128 (the module's step-by-step decode pads other sizes)")
         if m.to_qkv.weight.dtype != _BF16:
             raise NotImplementedError("DecodeSession needs a bf16 module (the raw key / value window is kept in bf16)")
         dev = cache_k.device
-        b, hk, t, d = cache_k.shape
+        b, hk, t, _ = cache_k.shape
+        d0 = m.dim_head
+        # the kernels hold 64 or 128 features per head: any other head dimension lives zero-padded in the session's
+        # buffers (zero features change neither logits nor outputs; the softmax scale stays that of d0), and the
+        # projection weights are copied with zero rows / columns so that the GEMMs read and write the padded layout
+        d = _kernel_dim(d0)
+        self.d0 = d0
         st, cbs = m.compress_block_sliding_stride, m.compress_block_size
         nc = cache_ck.shape[-2]
         if max_len <= t:
@@ -61,7 +66,7 @@ class DecodeSession:
 
         def grown(src, rows):
             buf = torch.zeros((b, hk, rows, d), dtype=_BF16, device=dev)
-            buf[:, :, :src.shape[-2]].copy_(src)
+            buf[:, :, :src.shape[-2], :src.shape[-1]].copy_(src)      # the module's own decode steps hand back padded rows
             return buf
         self.K, self.V = grown(cache_k, self.max_len), grown(cache_v, self.max_len)
         self.CK, self.CV = grown(cache_ck, self.max_nc), grown(cache_cv, self.max_nc)
@@ -76,13 +81,24 @@ class DecodeSession:
             raise ValueError("the cache's open compression window is longer than two compression blocks")
         if lr:
             rows = ring_rows(t - lr, torch.arange(lr, device=dev), R)
-            self.ring_k[:, :, rows] = run_k.to(_BF16)
-            self.ring_v[:, :, rows] = run_v.to(_BF16)
+            self.ring_k[:, :, rows] = _pad_dim(run_k.to(_BF16), d)
+            self.ring_v[:, :, rows] = _pad_dim(run_v.to(_BF16), d)
         self._ar = torch.arange(cbs, device=dev, dtype=torch.int32)
         self.state = torch.tensor([t, nc], dtype=torch.int32, device=dev)
-        self.mem_k = m.compress_mem_kv[0].detach().to(_BF16).contiguous()
-        self.mem_v = m.compress_mem_kv[1].detach().to(_BF16).contiguous()
-        self.freqs = m.rotary_emb.freqs.detach().to(torch.float32).contiguous()
+        self.mem_k = _pad_dim(m.compress_mem_kv[0].detach().to(_BF16), d).contiguous()
+        self.mem_v = _pad_dim(m.compress_mem_kv[1].detach().to(_BF16), d).contiguous()
+        self.freqs = _pad_dim(m.rotary_emb.freqs.detach().to(torch.float32), d // 2).contiguous()   # frequency 0: no rotation
+
+        def padded_heads(w, dim):            # 'heads * d0' along `dim` of a weight -> 'heads * d' with zeros
+            if d == d0:
+                return w
+            shape = list(w.shape)
+            shape[dim:dim + 1] = [shape[dim] // d0, d0]
+            w = _pad_dim(w.reshape(shape).movedim(dim + 1, -1), d).movedim(-1, dim + 1)
+            shape[dim:dim + 2] = [shape[dim] * d]
+            return w.reshape(shape)
+        w_qkv = padded_heads(m.to_qkv.weight.detach(), 0)
+        self.w_out = padded_heads(m.combine_heads.weight.detach(), 1).contiguous() if d != d0 else None
 
         # q, k, v and the strategy-gate logits come out of one GEMM: the gate projection's rows are appended to the qkv
         # weight (a copy: the session does not follow later changes of the module's parameters), its bias is added where the
@@ -91,11 +107,11 @@ class DecodeSession:
         self.fused_gate = isinstance(gate, torch.nn.Linear) and gate.in_features == m.to_qkv.in_features and gate.out_features == 3 * m.heads
         if self.fused_gate:
             pad = -3 * m.heads % 8                                  # rows of the GEMM output stay 16-byte aligned
-            self.w_cat = torch.cat((m.to_qkv.weight.detach(), gate.weight.detach().to(_BF16),
+            self.w_cat = torch.cat((w_qkv, gate.weight.detach().to(_BF16),
                                     torch.zeros((pad, m.to_qkv.in_features), dtype=_BF16, device=dev)), dim=0).contiguous()
             self.gate_bias = gate.bias.detach().to(_BF16).contiguous() if gate.bias is not None else None
         else:                                                       # a caller-supplied strategy network runs as it is
-            self.w_cat, self.gate_bias = m.to_qkv.weight.detach(), None
+            self.w_cat, self.gate_bias = w_qkv.contiguous(), None
         self.x_buf = torch.zeros((b, 1, m.to_qkv.in_features), dtype=_BF16, device=dev)
         self._desc, self._ws = self._make_desc(dev)
         self.graphs = None
@@ -128,7 +144,7 @@ class DecodeSession:
         dsc.pos, dsc.num_compressed = self.max_len - 1, self.max_nc
         dsc.per_block, dsc.block = m.selection_block_size // self.st, m.selection_block_size
         dsc.num_sel, dsc.share = m.num_selected_blocks, int(bool(m.query_heads_share_selected_kv))
-        dsc.window, dsc.scale = m.sliding_window_size, self.d ** -0.5
+        dsc.window, dsc.scale = m.sliding_window_size, self.d0 ** -0.5
         dsc.num_mem = self.mem_k.shape[-2]
         dsc.kc_stride[:] = self.K.stride()[:3]
         dsc.vc_stride[:] = self.V.stride()[:3]
@@ -166,6 +182,8 @@ class DecodeSession:
             gate_ptr, gate_row, self.gate_bias.data_ptr() if self.gate_bias is not None else None,
             self._ws.data_ptr(), self._ws.numel(), merged.data_ptr(), int(advance),
             torch.cuda.current_stream(x.device).cuda_stream), "nsa_decode_step_dyn")
+        if self.w_out is not None:
+            return torch.nn.functional.linear(merged, self.w_out, m.combine_heads.bias)
         return m.combine_heads(merged)
 
     def compress_window(self, count: bool = True):
@@ -173,11 +191,11 @@ class DecodeSession:
         to the compressed caches (NSA.py:422-441); every index comes from device memory."""
         m = self.module
         rows = ring_rows(self.state[0] - self.cbs, self._ar, self.ring)
-        wk = self.ring_k.index_select(2, rows)
-        wv = self.ring_v.index_select(2, rows)
+        wk = self.ring_k.index_select(2, rows)[..., :self.d0]
+        wv = self.ring_v.index_select(2, rows)[..., :self.d0]
         at = self.state[1:2].long()
-        self.CK.index_copy_(2, at, m.k_compress((wk + m.k_intrablock_positions)[:, :, None]).to(_BF16))
-        self.CV.index_copy_(2, at, m.v_compress((wv + m.v_intrablock_positions)[:, :, None]).to(_BF16))
+        self.CK.index_copy_(2, at, _pad_dim(m.k_compress((wk + m.k_intrablock_positions)[:, :, None]).to(_BF16), self.d))
+        self.CV.index_copy_(2, at, _pad_dim(m.v_compress((wv + m.v_intrablock_positions)[:, :, None]).to(_BF16), self.d))
         if count:
             self.state[1:2].add_(1)
 
@@ -208,12 +226,13 @@ class DecodeSession:
         t, st, cbs = self.pos, self.st, self.cbs
         first = (t // st) * st - (cbs - st)                          # first position of the open window
         rows = ring_rows(first, torch.arange(t - first, device=self.K.device), self.ring)
+        d0 = self.d0        # as the module's own decode step keeps them: keys / values and window rows padded, compressed keys not
         run_k, run_v = self.ring_k.index_select(2, rows), self.ring_v.index_select(2, rows)
         if first < 0:                                                # positions before the sequence start read as zero
             run_k[:, :, :-first] = 0
             run_v[:, :, :-first] = 0
         return ((self.K[:, :, :t].clone(), self.V[:, :, :t].clone()),
-                ((self.CK[:, :, :self.nc].clone(), self.CV[:, :, :self.nc].clone()), (run_k, run_v)))
+                ((self.CK[:, :, :self.nc, :d0].clone(), self.CV[:, :, :self.nc, :d0].clone()), (run_k, run_v)))
 
 
 class TransformerDecodeSession:

@@ -16,6 +16,8 @@ CONFIGS = [
     (192, 64, 6, 2, 16, 8, 4, 8, 2, True, 30, 30),        # group of 3 query heads per kv head
     (128, 64, 4, 2, 16, 32, 16, 128, 2, True, 300, 30),   # 128-token selection blocks
     (128, 64, 2, 1, 4, 5, 4, 20, 2, True, 47, 40),        # compress block 5, selection block 20 (5 compressed keys per block)
+    (128, 32, 4, 2, 16, 8, 4, 8, 2, True, 37, 30),        # head dimensions the kernels are not compiled for: zero-padded buffers
+    (192, 96, 2, 1, 16, 8, 4, 16, 2, True, 40, 30),
 ]
 
 
@@ -67,6 +69,9 @@ def test_graph_decode_matches_eager_decode(cfg):
         a, _ = m(x, cache=sess.cache(), return_cache=True)
         bb, _ = m(x, cache=cache, return_cache=True)
     assert torch.equal(a, bb)
+    # a session can also start from caches that went through the module's decode steps (padded rows for odd head sizes)
+    sess2 = DecodeSession(m, cache, max_len=n0 + steps + 5)
+    assert torch.equal(sess2.step(x), sess.step(x))
 
 
 def test_graph_decode_capacity_is_enforced():
