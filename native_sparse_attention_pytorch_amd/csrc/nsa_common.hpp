@@ -101,6 +101,21 @@ __device__ __forceinline__ bf16x8 lds_row_operand(const __bf16* tile_s, int RS, 
 
 // s_waitcnt vmcnt(0) (expcnt / lgkmcnt left at their maxima): all outstanding global loads
 // and stores of this wave have completed.
+// N operand reads feeding N uses, each read issued AH uses ahead of its own.  The compiler keeps an LDS operand
+// read where the source puts it - right before its MFMA it means a full LDS round trip per MFMA - so the distance
+// is spelled out here.  `rd(i)` returns operand i, `use(i, a)` consumes it; both are inlined into a fully unrolled loop.
+template <int N, int AH, class Read, class Use>
+__device__ __forceinline__ void operands_ahead(Read rd, Use use) {
+  bf16x8 ring[AH + 1];
+#pragma unroll
+  for (int i = 0; i < AH && i < N; ++i) ring[i] = rd(i);
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    if (i + AH < N) ring[(i + AH) % (AH + 1)] = rd(i + AH);
+    use(i, ring[i % (AH + 1)]);
+  }
+}
+
 // Wait for every outstanding vector memory operation.  The plain s_waitcnt builtin does not order
 // loads around itself (the compiler moved gathers issued before it to after it), hence the fence.
 __device__ __forceinline__ void wait_all_loads() {

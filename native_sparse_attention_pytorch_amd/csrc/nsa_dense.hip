@@ -451,6 +451,9 @@ __device__ __forceinline__ void chunk_of(const DensePlan& P, int x, int& T, int&
   chunk_range(P, T, c, qlo, qhi, c0, c1);
 }
 
+#ifndef NSA_DKV_AHEAD
+#define NSA_DKV_AHEAD 3
+#endif
 #ifndef NSA_DKV_STAGES
 #define NSA_DKV_STAGES 1      // measured on MI355X (compressed branch, seq 32k, d 128): 1, 2 or 3 tiles ahead all 4.7 ms
 #endif
@@ -571,13 +574,17 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
     }
     const bf16x8 Pf0 = pack8(Sa, 0), Pf1 = pack8(Sa, 8);
     const bf16x8 Sf0 = pack8(dSa, 0), Sf1 = pack8(dSa, 8);
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 0, 32 * dt, lane), Pf0, dVa[dt]);
-      dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 16, 32 * dt, lane), Pf1, dVa[dt]);
-      dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 0, 32 * dt, lane), Sf0, dKa[dt]);
-      dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 16, 32 * dt, lane), Sf1, dKa[dt]);
-    }
+    // dV^T += dO^T P, dK^T += Q^T dS: 4 * DT MFMAs whose LDS operands are read NSA_DKV_AHEAD MFMAs ahead (the
+    // compiler keeps transpose loads in source order; read right before their MFMA, LDS latency paces the phase)
+    operands_ahead<4 * DT, NSA_DKV_AHEAD>(
+        [&](int i) { return lds_transposed_operand((i & 2) ? xq_s : xg_s, RS, 16 * (i & 1), 32 * (i >> 2), lane); },
+        [&](int i, const bf16x8& a) {
+          const int dt = i >> 2, w = i & 3;
+          if (w == 0) dVa[dt] = mfma32(a, Pf0, dVa[dt]);
+          else if (w == 1) dVa[dt] = mfma32(a, Pf1, dVa[dt]);
+          else if (w == 2) dKa[dt] = mfma32(a, Sf0, dKa[dt]);
+          else dKa[dt] = mfma32(a, Sf1, dKa[dt]);
+        });
     };
     {
       // rows of this wave are visible to every query of the tile iff they lie between the largest lower

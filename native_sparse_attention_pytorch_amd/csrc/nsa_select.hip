@@ -800,6 +800,9 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 // [key][row] in LDS; dQ^T = K^T dS^T is then formed with both operands read through the
 // transpose load (K block row-major in LDS, loaded once per unit), each wave taking half of the
 // features, and the finished 32 x D tile leaves through coalesced row stores.
+#ifndef NSA_BWD_AHEAD
+#define NSA_BWD_AHEAD 3       // LDS operand reads issued this many MFMAs ahead in the backward walk
+#endif
 #ifndef NSA_BWD_STAGES
 #define NSA_BWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1 stage 3.8 ms, 2 and 3 stages 3.27 ms
 #endif
@@ -919,12 +922,13 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
     issue(cur, rn);
     __builtin_amdgcn_sched_barrier(0);
 
-    floatx16 Sa = zero_acc(), Pa = zero_acc();
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      Sa = mfma32(lds_row_operand(xq_s, RS, ks, lane), Kf[ks], Sa);   // [row][key]: lane <-> key, registers <-> rows
-      Pa = mfma32(lds_row_operand(xg_s, RS, ks, lane), Vf[ks], Pa);
-    }
+    floatx16 Sa = zero_acc(), Pa = zero_acc();              // [row][key]: lane <-> key, registers <-> rows
+    operands_ahead<2 * KS, NSA_BWD_AHEAD>(
+        [&](int i) { return lds_row_operand((i & 1) ? xg_s : xq_s, RS, i >> 1, lane); },
+        [&](int i, const bf16x8& a) {
+          if (i & 1) Pa = mfma32(a, Vf[i >> 1], Pa);
+          else Sa = mfma32(a, Kf[i >> 1], Sa);
+        });
     floatx16 dSa;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
@@ -951,26 +955,35 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
         *reinterpret_cast<bf16x4*>(ds_s + kl * RST + 8 * a + 4 * h) = t4;
       }
     }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 0, 32 * dt, lane), Pf0, dVa[dt]);
-      dVa[dt] = mfma32(lds_transposed_operand(xg_s, RS, 16, 32 * dt, lane), Pf1, dVa[dt]);
-      dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 0, 32 * dt, lane), Sf0, dKa[dt]);
-      dKa[dt] = mfma32(lds_transposed_operand(xq_s, RS, 16, 32 * dt, lane), Sf1, dKa[dt]);
-    }
+    // dV^T += dO^T P, dK^T += Q^T dS
+    operands_ahead<4 * DT, NSA_BWD_AHEAD>(
+        [&](int i) { return lds_transposed_operand((i & 2) ? xq_s : xg_s, RS, 16 * (i & 1), 32 * (i >> 2), lane); },
+        [&](int i, const bf16x8& a) {
+          const int dt = i >> 2, w = i & 3;
+          if (w == 0) dVa[dt] = mfma32(a, Pf0, dVa[dt]);
+          else if (w == 1) dVa[dt] = mfma32(a, Pf1, dVa[dt]);
+          else if (w == 2) dKa[dt] = mfma32(a, Sf0, dKa[dt]);
+          else dKa[dt] = mfma32(a, Sf1, dKa[dt]);
+        });
     __syncthreads();
     if (FUSE_DQ) {
       // dQ^T[feature][row] = sum_key K^T[feature][key] dS^T[key][row]; this wave: features 32*DTW*kt ...
       floatx16 Qa[DTW];
 #pragma unroll
       for (int w = 0; w < DTW; ++w) Qa[w] = zero_acc();
-#pragma unroll
-      for (int k0 = 0; k0 < 32 * KT; k0 += 16) {
-        const bf16x8 Sf = lds_transposed_operand(ds_s, RST, k0, 0, lane);          // lane <-> row, k <-> keys k0 ..
-#pragma unroll
-        for (int w = 0; w < DTW; ++w)
-          Qa[w] = mfma32(lds_transposed_operand(kb_s, RSK, k0, 32 * (DTW * kt + w), lane), Sf, Qa[w]);
-      }
+      // per 16 keys: the dS^T operand (lane <-> row, k <-> keys k0 ..), then the DTW K^T operands it multiplies
+      bf16x8 Sf = zero_frag();
+      operands_ahead<2 * KT * (DTW + 1), NSA_BWD_AHEAD>(
+          [&](int i) {
+            const int k0 = 16 * (i / (DTW + 1)), w = i % (DTW + 1);
+            return w == 0 ? lds_transposed_operand(ds_s, RST, k0, 0, lane)
+                          : lds_transposed_operand(kb_s, RSK, k0, 32 * (DTW * kt + w - 1), lane);
+          },
+          [&](int i, const bf16x8& a) {
+            const int w = i % (DTW + 1);
+            if (w == 0) Sf = a;
+            else Qa[w - 1] = mfma32(a, Sf, Qa[w - 1]);
+          });
       // Qa[w][4a + bb] = dQ[row n_][feature 32(DTW kt + w) + 8a + 4h + bb]
 #pragma unroll
       for (int w = 0; w < DTW; ++w)
