@@ -310,11 +310,14 @@ __device__ __forceinline__ void issue_tile_loads(bf16x8 (&raw)[D / 16], const __
                                                  int gmask, int lane) {
   constexpr int CPR = D / 8, RPI = 64 / CPR, NT = 32 / RPI;
   static_assert(NT == D / 16, "tile load count");
+  // all lane exchanges first, then all loads: taken in turn, every load would wait for its own exchange
+  int qi[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) qi[t] = __shfl(my_i, t * RPI + lane / CPR, 64);
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const int rr = t * RPI + lane / CPR, c = lane % CPR;
-    const int i = __shfl(my_i, rr, 64);
-    raw[t] = load8(base + (long)(rr & gmask) * s_head + (long)i * s_tok + 8 * c);
+    raw[t] = load8(base + (long)(rr & gmask) * s_head + (long)qi[t] * s_tok + 8 * c);
   }
 }
 
@@ -352,12 +355,18 @@ __device__ __forceinline__ void store_tile_rows(const floatx16 (&acc)[D / 32], f
     }
   if (h == 0) row_s[n_] = row;
   __syncthreads();
+  // all LDS reads first, then all stores: taken in turn, every store would wait for its own read
+  bf16x8 v[32 / RPI];
+  size_t rw[32 / RPI];
 #pragma unroll
   for (int t = 0; t < 32 / RPI; ++t) {
     const int rr = t * RPI + lane / CPR, c = lane % CPR;
-    const bf16x8 v = *reinterpret_cast<const bf16x8*>(tile_s + rr * RS + 8 * c);
-    __builtin_nontemporal_store(v, reinterpret_cast<bf16x8*>(dst + row_s[rr] * D + 8 * c));
+    v[t] = *reinterpret_cast<const bf16x8*>(tile_s + rr * RS + 8 * c);
+    rw[t] = row_s[rr];
   }
+#pragma unroll
+  for (int t = 0; t < 32 / RPI; ++t)
+    __builtin_nontemporal_store(v[t], reinterpret_cast<bf16x8*>(dst + rw[t] * D + 8 * (lane % CPR)));
   __syncthreads();
 }
 
@@ -996,12 +1005,17 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
         }
       __syncthreads();
       constexpr int CPR = D / 8, RPI = (64 * KT) / CPR;
+      bf16x8 vv[32 / RPI];
+      size_t rw[32 / RPI];
 #pragma unroll
-      for (int t = 0; t < 32 / RPI; ++t) {
+      for (int t = 0; t < 32 / RPI; ++t) {          // all LDS reads first, then all stores
         const int rr = t * RPI + (int)threadIdx.x / CPR, c = threadIdx.x % CPR;
-        const bf16x8 vv = *reinterpret_cast<const bf16x8*>(dq_s + rr * RS + 8 * c);
-        __builtin_nontemporal_store(vv, reinterpret_cast<bf16x8*>(dqpart + row_s[rr] * D + 8 * c));
+        vv[t] = *reinterpret_cast<const bf16x8*>(dq_s + rr * RS + 8 * c);
+        rw[t] = row_s[rr];
       }
+#pragma unroll
+      for (int t = 0; t < 32 / RPI; ++t)
+        __builtin_nontemporal_store(vv[t], reinterpret_cast<bf16x8*>(dqpart + rw[t] * D + 8 * (threadIdx.x % CPR)));
       __syncthreads();
     }
   };
