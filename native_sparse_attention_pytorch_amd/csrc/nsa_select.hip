@@ -373,7 +373,7 @@ __device__ __forceinline__ void store_tile_rows(const floatx16 (&acc)[D / 32], f
 // ------------------------------------------------------------------------------- forward
 
 #ifndef NSA_FWD_STAGES
-#define NSA_FWD_STAGES 1      // measured on MI355X (seq 32k, d 128): 1 stage 1.56 ms, 2 stages 1.60 ms
+#define NSA_FWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1 stage 1.47 ms, 2 stages 1.445 ms
 #endif
 template <int D, int KT>
 __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
@@ -813,7 +813,7 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 #define NSA_BWD_AHEAD 3       // LDS operand reads issued this many MFMAs ahead in the backward walk
 #endif
 #ifndef NSA_BWD_STAGES
-#define NSA_BWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1 stage 3.8 ms, 2 and 3 stages 3.27 ms
+#define NSA_BWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1, 2 and 3 stages all 2.68-2.70 ms once the LDS operand reads run ahead
 #endif
 template <int D, int KT, bool FUSE_DQ>
 __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1))) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
