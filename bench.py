@@ -31,8 +31,8 @@ CFG = dict(batch=1, seq=32768, heads=32, kv_heads=8, dim_head=128, block=64, num
 
 # HBM bytes per launch on this workload, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
 # scaled by streaming kernels of known size (profiles/select_fwd_bwd_seq32k_hbm_traffic.txt)
-MEASURED_TRAFFIC_BYTES = {"fwd_block_walk": 6.416e9, "fwd_merge": 4.850e9, "bwd_dq_merge": 4.546e9,
-                          "bwd_dkv_walk": 13.422e9, "bwd_dkv_reduce": 0.547e9, "bwd_delta": 0.541e9}
+MEASURED_TRAFFIC_BYTES = {"fwd_block_walk": 6.405e9, "fwd_merge": 4.851e9, "bwd_dq_merge": 4.546e9,
+                          "bwd_dkv_walk": 13.398e9, "bwd_dkv_reduce": 0.547e9, "bwd_delta": 0.541e9}
 
 
 def selection(b, h, n, B, S, seed, device):
