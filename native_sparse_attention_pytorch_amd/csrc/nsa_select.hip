@@ -480,28 +480,42 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) Sa[kt] = mfma32(Kf[kt][ks], Qf[ks], Sa[kt]);
     }
-    // local softmax over the block's keys; this lane holds 16*KT keys of row n_, lane^32 the rest
+    // local softmax over the block's keys; this lane holds 16*KT keys of row n_, lane^32 the rest.  The maximum is
+    // taken over the raw scores (the scale is positive) and the scale folded into the exponent's multiply-add; a tile
+    // whose rows all see the whole block (every tile but the own-block ones) skips the key mask (wave-uniform)
+    const bool whole = __all(r.lim >= 32 * KT - 1);
     float mx = -INFINITY;
+    if (!whole) {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i2 = 0; i2 < 16; ++i2) {
+          const int kl = 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
+          if (kl > r.lim) Sa[kt][i2] = -INFINITY;
+        }
+    }
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-      for (int i2 = 0; i2 < 16; ++i2) {
-        const int kl = 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
-        const float s = (kl <= r.lim) ? Sa[kt][i2] * sc : -INFINITY;
-        Sa[kt][i2] = s;
-        mx = fmaxf(mx, s);
-      }
+      for (int i2 = 0; i2 < 16; ++i2) mx = fmaxf(mx, Sa[kt][i2]);
     mx = fmaxf(mx, xor32(mx));
+    const float mxs = mx * sc;                       // the row maximum in the exponent's units (log2)
     float l = 0.f;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int i2 = 0; i2 < 16; ++i2) {
-        const float p = fast_exp2(Sa[kt][i2] - mx);
+        const float p = fast_exp2(__builtin_fmaf(Sa[kt][i2], sc, -mxs));
         Sa[kt][i2] = p;
         l += p;
       }
     l += xor32(l);
+    // normalise the probabilities (32 values) rather than the output tile (64)
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int i2 = 0; i2 < 16; ++i2) Sa[kt][i2] *= inv;
 
     floatx16 Oa[DT];
 #pragma unroll
@@ -518,10 +532,9 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
     {
       // padding rows write to a spare row at the end of the buffers: the stores stay
       // unconditional, so the wait for the next tile's loads never has to cover them
-      const float inv = 1.0f / l;
       const size_t row = r.valid ? (((size_t)bh * P.n + r.i) * P.SP + r.slot) * P.g + r.g : P.prow;
-      store_tile_rows<D>(Oa, inv, row, opart, tile_s, row_s, lane);
-      if (h == 0) lsepart[row] = (mx + fast_log2(l)) * kLn2;
+      store_tile_rows<D>(Oa, 1.0f, row, opart, tile_s, row_s, lane);
+      if (h == 0) lsepart[row] = (mxs + fast_log2(l)) * kLn2;
     }
   };
   // whole rounds of NS tiles first: their steps are unconditional, so each wait counts exactly the
