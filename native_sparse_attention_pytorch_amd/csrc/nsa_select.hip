@@ -314,10 +314,13 @@ __device__ __forceinline__ void issue_tile_loads(bf16x8 (&raw)[D / 16], const __
   int qi[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) qi[t] = __shfl(my_i, t * RPI + lane / CPR, 64);
+  // the head and token strides are below 2^32 (checked when the plan is made): 32 x 32 -> 64-bit multiply-adds
+  const unsigned sh32 = (unsigned)s_head, st32 = (unsigned)s_tok;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const int rr = t * RPI + lane / CPR, c = lane % CPR;
-    raw[t] = load8(base + (long)(rr & gmask) * s_head + (long)qi[t] * s_tok + 8 * c);
+    const unsigned long off = (unsigned long)(unsigned)(rr & gmask) * sh32 + (unsigned long)(unsigned)qi[t] * st32;
+    raw[t] = load8(base + off + 8 * c);
   }
 }
 

@@ -60,6 +60,8 @@ static inline int make_plan(const nsa_select_desc* d, SelPlan& P) {
   for (int t = 0; t < 3; ++t) { P.sq[t] = d->q_stride[t]; P.sk[t] = d->k_stride[t]; P.sv[t] = d->v_stride[t]; P.so[t] = d->o_stride[t]; }
   for (int t = 0; t < 3; ++t)
     if ((P.sq[t] | P.sk[t] | P.sv[t] | P.so[t]) & 7) return NSA_E_ARG;      // rows must start 16-byte aligned
+  for (int t = 1; t < 3; ++t)                                               // head and token strides: 32-bit arithmetic in the gathers
+    if ((P.sq[t] | P.so[t]) < 0 || ((P.sq[t] | P.so[t]) >> 32)) return NSA_E_UNSUPPORTED;
   const long pairs = (long)P.n * (P.S + P.causal);
   // phase length: the Q rows (forward) / Q and dO rows (dQ walk) of one phase are about the size
   // of one XCD's 4 MB L2 (measured best on MI355X among 0.5 .. 64 MB; shorter phases make the
