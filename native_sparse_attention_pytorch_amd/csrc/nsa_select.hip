@@ -955,17 +955,34 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
           else Sa = mfma32(a, Kf[i >> 1], Sa);
         });
     floatx16 dSa;
+    // a tile whose rows all see the whole block (every tile but the own-block ones) skips the key mask (uniform)
+    const bool whole = r.lim >= 32 * KT - 1;
+    if (__all(whole)) {
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      const floatx4 l4 = *reinterpret_cast<const floatx4*>(&lse_s[8 * a + 4 * h]);
-      const floatx4 d4 = *reinterpret_cast<const floatx4*>(&del_s[8 * a + 4 * h]);
-      const int* m4 = &lim_s[8 * a + 4 * h];
+      for (int a = 0; a < 4; ++a) {
+        const floatx4 l4 = *reinterpret_cast<const floatx4*>(&lse_s[8 * a + 4 * h]);
+        const floatx4 d4 = *reinterpret_cast<const floatx4*>(&del_s[8 * a + 4 * h]);
 #pragma unroll
-      for (int bb = 0; bb < 4; ++bb) {
-        const int i2 = 4 * a + bb;
-        const float p = (kl <= m4[bb]) ? fast_exp2(Sa[i2] * sc - l4[bb]) : 0.f;
-        Sa[i2] = p;
-        dSa[i2] = p * (Pa[i2] - d4[bb]);
+        for (int bb = 0; bb < 4; ++bb) {
+          const int i2 = 4 * a + bb;
+          const float p = fast_exp2(__builtin_fmaf(Sa[i2], sc, -l4[bb]));
+          Sa[i2] = p;
+          dSa[i2] = p * (Pa[i2] - d4[bb]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const floatx4 l4 = *reinterpret_cast<const floatx4*>(&lse_s[8 * a + 4 * h]);
+        const floatx4 d4 = *reinterpret_cast<const floatx4*>(&del_s[8 * a + 4 * h]);
+        const int* m4 = &lim_s[8 * a + 4 * h];
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) {
+          const int i2 = 4 * a + bb;
+          const float p = (kl <= m4[bb]) ? fast_exp2(__builtin_fmaf(Sa[i2], sc, -l4[bb])) : 0.f;
+          Sa[i2] = p;
+          dSa[i2] = p * (Pa[i2] - d4[bb]);
+        }
       }
     }
     const bf16x8 Pf0 = pack8(Sa, 0), Pf1 = pack8(Sa, 8);
