@@ -825,6 +825,12 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 // [key][row] in LDS; dQ^T = K^T dS^T is then formed with both operands read through the
 // transpose load (K block row-major in LDS, loaded once per unit), each wave taking half of the
 // features, and the finished 32 x D tile leaves through coalesced row stores.
+#ifndef NSA_BWD_D64_WAVES
+#define NSA_BWD_D64_WAVES 2
+#endif
+#ifndef NSA_BWD_AHEAD_D64
+#define NSA_BWD_AHEAD_D64 3
+#endif
 #ifndef NSA_BWD_AHEAD
 #define NSA_BWD_AHEAD 3       // LDS operand reads issued this many MFMAs ahead in the backward walk
 #endif
@@ -832,7 +838,7 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 #define NSA_BWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1, 2 and 3 stages all 2.68-2.70 ms once the LDS operand reads run ahead
 #endif
 template <int D, int KT, bool FUSE_DQ>
-__global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1))) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+__global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64 ? NSA_BWD_D64_WAVES : 1))) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                               const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
                                                               const float* __restrict__ lse, const float* __restrict__ delta,
                                                               const char* __restrict__ iws, char* __restrict__ bws) {
@@ -840,6 +846,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
   constexpr int RST = 32 + 16;                 // row stride of the [key][row] dS tile (transpose loads only: 8 banks mod 32 per row)
   constexpr int RSK = D + 16;                  // row stride of the K block copy (transpose loads only)
   constexpr int DTW = DT / KT;                 // feature tiles of dQ per wave
+  constexpr int AHD = D == 64 ? NSA_BWD_AHEAD_D64 : NSA_BWD_AHEAD;      // LDS operand look-ahead
   __shared__ __align__(16) float lse_s[32];
   __shared__ __align__(16) float del_s[32];
   __shared__ __align__(16) int lim_s[32];
@@ -948,7 +955,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
     __builtin_amdgcn_sched_barrier(0);
 
     floatx16 Sa = zero_acc(), Pa = zero_acc();              // [row][key]: lane <-> key, registers <-> rows
-    operands_ahead<2 * KS, NSA_BWD_AHEAD>(
+    operands_ahead<2 * KS, AHD>(
         [&](int i) { return lds_row_operand((i & 1) ? xg_s : xq_s, RS, i >> 1, lane); },
         [&](int i, const bf16x8& a) {
           if (i & 1) Pa = mfma32(a, Vf[i >> 1], Pa);
@@ -998,7 +1005,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
       }
     }
     // dV^T += dO^T P, dK^T += Q^T dS
-    operands_ahead<4 * DT, NSA_BWD_AHEAD>(
+    operands_ahead<4 * DT, AHD>(
         [&](int i) { return lds_transposed_operand((i & 2) ? xq_s : xg_s, RS, 16 * (i & 1), 32 * (i >> 2), lane); },
         [&](int i, const bf16x8& a) {
           const int dt = i >> 2, w = i & 3;
@@ -1015,7 +1022,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
       for (int w = 0; w < DTW; ++w) Qa[w] = zero_acc();
       // per 16 keys: the dS^T operand (lane <-> row, k <-> keys k0 ..), then the DTW K^T operands it multiplies
       bf16x8 Sf = zero_frag();
-      operands_ahead<2 * KT * (DTW + 1), NSA_BWD_AHEAD>(
+      operands_ahead<2 * KT * (DTW + 1), AHD>(
           [&](int i) {
             const int k0 = 16 * (i / (DTW + 1)), w = i % (DTW + 1);
             return w == 0 ? lds_transposed_operand(ds_s, RST, k0, 0, lane)
