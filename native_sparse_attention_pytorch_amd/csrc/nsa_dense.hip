@@ -270,11 +270,18 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
     const int jstart = min(P.nb, (kBK * (last_visited + 1)) / (POOL ? NPF : 1));
     const int cntj = P.nb - jstart;
     const int rows_here = max(0, min(ppt, P.n - i0)) * (P.share ? 1 : P.g);
-    for (int e = lane; e < rows_here * cntj; e += 64) {
-      const int rr = e / cntj, jj = jstart + e % cntj;
-      const int qi = i0 + (P.share ? rr : rr / P.g);
-      const long prow = P.share ? ((long)bh * P.n + qi) : (((long)b * P.hkv * P.g + hk * P.g + rr % P.g) * P.n + qi);
-      pooled[prow * P.nb + jj] = -INFINITY;
+    // row by row (no division by the run-time count), 16 bytes per lane where the rows allow it
+    const bool vec = cntj > 0 && !(P.nb & 3) && !(jstart & 3);
+    for (int rr = 0; rr < rows_here; ++rr) {
+      const int qi = i0 + (P.share ? rr : (rr >> P.lg));
+      const long prow = P.share ? ((long)bh * P.n + qi) : (((long)b * P.hkv * P.g + hk * P.g + (rr & (P.g - 1))) * P.n + qi);
+      float* dst = pooled + prow * P.nb;
+      if (vec) {
+        const floatx4 ninf = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+        for (int jj = jstart + 4 * lane; jj < P.nb; jj += 256) *reinterpret_cast<floatx4*>(dst + jj) = ninf;
+      } else {
+        for (int jj = jstart + lane; jj < P.nb; jj += 64) dst[jj] = -INFINITY;
+      }
     }
   }
 
