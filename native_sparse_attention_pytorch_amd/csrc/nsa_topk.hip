@@ -164,6 +164,149 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in,
   }
 }
 
+// Four rows per wave, 16 lanes per row: for rows of up to 512 entries and k <= 16.  A round of the kernel above costs
+// the same ~60 instructions whether a wave serves one row or four, and most of them are the winning lane's re-scan of
+// its VPL entries, which every lane of the wave pays for.  Here a lane's entries live in LDS (its own segment: no
+// lane ever reads another's), cut into groups of eight whose maxima stay in registers; the winner marks its entry
+// taken, re-reads that one group and refreshes one maximum.  Row maxima are DPP butterflies inside a row of 16 lanes
+// (no readlane), the winner is the lowest set bit of the row's 16 bits of the ballot.  Order of equal values: lower
+// lane first, inside a lane lower group first, inside a group lower entry first - lower block index, as above.
+__device__ __forceinline__ float row16_max(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xF, 0xF, false));
+  };
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0xB1>{}));
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x4E>{}));
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x141>{}));
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x140>{}));
+  return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xF, 0xF, false));
+  };
+  v += dpp(v, std::integral_constant<int, 0xB1>{});
+  v += dpp(v, std::integral_constant<int, 0x4E>{});
+  v += dpp(v, std::integral_constant<int, 0x141>{});
+  v += dpp(v, std::integral_constant<int, 0x140>{});
+  return v;
+}
+
+template <int VPL>
+__global__ __launch_bounds__(256) void topk_rows4_kernel(const float* __restrict__ in, long rows, int nb, int k, int softmax, int vec4,
+                                                         int* __restrict__ idx, float* __restrict__ vals, uint8_t* __restrict__ fmask) {
+  constexpr int GS = VPL < 8 ? VPL : 8, NG = VPL / GS;
+  constexpr int SEG = VPL + 4;                            // a lane's segment, padded: 16-byte reads of 16 lanes hit 64 distinct banks
+  __shared__ __align__(16) float xs[16][16 * SEG];        // [row of the work-group][lane `sub`][entries sub*VPL ..]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane & 15, rs = lane >> 4;
+  const long row = (long)blockIdx.x * 16 + wave * 4 + rs;
+  const bool live = row < rows;                             // a dead row group works on the last row and stores nothing
+  const float* src = in + (live ? row : rows - 1) * nb;
+  float* row_s = xs[wave * 4 + rs];
+  float* mine_s = row_s + sub * SEG;
+  float x[VPL];
+  // with 16-byte aligned rows the loads are coalesced (consecutive lanes, consecutive 16 bytes) and the entries reach
+  // their owners through LDS after the softmax, which does not care about the order; otherwise a lane loads its own
+  const bool spread = vec4 != 0;
+  if (spread) {
+#pragma unroll
+    for (int r4 = 0; r4 < VPL / 4; ++r4) {
+      const int j = 4 * (sub + 16 * r4);
+      floatx4 t = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      if (j < nb) t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(src + j));      // read once
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[4 * r4 + e] = t[e];
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+      const int j = sub * VPL + r;
+      x[r] = j < nb ? src[j] : -INFINITY;
+    }
+  }
+  if (softmax) {
+    float mx = -1e3f;
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) mx = fmaxf(mx, x[r]);
+    mx = row16_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) { x[r] = __expf(x[r] - mx); sum += x[r]; }
+    sum = row16_sum(sum) + __expf(-1e3f - mx);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) x[r] *= inv;
+  }
+  if (spread) {
+#pragma unroll
+    for (int r4 = 0; r4 < VPL / 4; ++r4) {
+      const int j = 4 * (sub + 16 * r4);                    // entries j .. j+3 belong to lane j / VPL
+      *reinterpret_cast<floatx4*>(row_s + (j / VPL) * SEG + j % VPL) = floatx4{x[4 * r4], x[4 * r4 + 1], x[4 * r4 + 2], x[4 * r4 + 3]};
+    }
+    __builtin_amdgcn_wave_barrier();                        // LDS operations of one wave execute in order
+#pragma unroll
+    for (int r4 = 0; r4 < VPL / 4; ++r4) {
+      const floatx4 t = *reinterpret_cast<const floatx4*>(mine_s + 4 * r4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[4 * r4 + e] = t[e];
+    }
+  }
+  float gm[NG];
+  int ga[NG];
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+#pragma unroll
+    for (int t = 0; t < GS; ++t) {
+      const int r = g * GS + t;
+      if (sub * VPL + r >= nb) x[r] = -1.0f;                // padding loses against every real entry
+      if (t == 0 || x[r] > gm[g]) { gm[g] = x[r]; ga[g] = r; }      // strict: ties keep the lower index
+    }
+  }
+#pragma unroll
+  for (int r4 = 0; r4 < VPL / 4; ++r4)
+    *reinterpret_cast<floatx4*>(mine_s + 4 * r4) = floatx4{x[4 * r4], x[4 * r4 + 1], x[4 * r4 + 2], x[4 * r4 + 3]};
+
+  float res_v = 0.f;
+  int res_j = 0;
+  for (int s = 0; s < k; ++s) {
+    float bv = gm[0];
+    int ba = ga[0];
+#pragma unroll
+    for (int g = 1; g < NG; ++g)
+      if (gm[g] > bv) { bv = gm[g]; ba = ga[g]; }
+    const float m = row16_max(bv);
+    const unsigned long long holders = __ballot(bv == m);
+    const unsigned row_bits = (unsigned)(holders >> (lane & 48)) & 0xffffu;       // never 0: one of the row's lanes holds m
+    const int w = __builtin_ctz(row_bits);                                        // lowest lane = lowest index among equals
+    const int jw = __shfl(sub * VPL + ba, (lane & 48) + w, 64);
+    if (sub == s) { res_v = m; res_j = jw; }
+    if (sub == w) {
+      mine_s[ba] = -2.0f;                                   // taken
+      const int g0 = ba & ~(GS - 1);                        // first entry of the group that held it
+      float y[GS];
+#pragma unroll
+      for (int t4 = 0; t4 < GS / 4; ++t4) {
+        const floatx4 t = *reinterpret_cast<const floatx4*>(mine_s + g0 + 4 * t4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[4 * t4 + e] = t[e];
+      }
+      float ngm = y[0];
+      int nga = g0;
+#pragma unroll
+      for (int t = 1; t < GS; ++t)
+        if (y[t] > ngm) { ngm = y[t]; nga = g0 + t; }
+#pragma unroll
+      for (int g = 0; g < NG; ++g)
+        if (g * GS == g0) { gm[g] = ngm; ga[g] = nga; }
+    }
+  }
+  if (live && sub < k) {
+    idx[row * k + sub] = res_j;
+    vals[row * k + sub] = res_v;
+    fmask[row * k + sub] = res_v > 1e-10f ? 1 : 0;
+  }
+}
+
 }  // namespace nsa
 
 #define NSA_TOPK_POOL false
@@ -176,6 +319,17 @@ extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   const int vpl = (nb + 63) / 64;
   const int vec4 = (nb % 4 == 0) && ((reinterpret_cast<uintptr_t>(scores) & 15) == 0);
+  if (k <= 16 && nb <= 512) {          // four rows per wave
+    const dim3 grid4((unsigned)((rows + 15) / 16));
+#define NSA_TOPK4(V) hipLaunchKernelGGL((topk_rows4_kernel<V>), grid4, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, idx, vals, fmask)
+    if (nb <= 64) NSA_TOPK4(4);
+    else if (nb <= 128) NSA_TOPK4(8);
+    else if (nb <= 256) NSA_TOPK4(16);
+    else NSA_TOPK4(32);
+#undef NSA_TOPK4
+    hipError_t e4 = hipGetLastError();
+    return e4 == hipSuccess ? 0 : (int)e4;
+  }
   const PoolArgs pool{0, 1, 0, 1};
   const TopkDyn dyn{nullptr, 1};
 #define NSA_TOPK(V) hipLaunchKernelGGL((topk_kernel<V, NSA_TOPK_POOL>), grid, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, pool, idx, vals, fmask, k, dyn)
