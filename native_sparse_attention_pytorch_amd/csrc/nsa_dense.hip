@@ -523,7 +523,9 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
     for (int t = 0; t < NT; ++t) {
       const int rr = t * RPI + lane / CPR;
       const int qi = min(i0 + (rr >> P.lg), P.n - 1);
-      st.raw[t] = load8(base + (long)(rr & (P.g - 1)) * sh + (long)qi * sn + 8 * (lane % CPR));
+      // head and token strides are below 2^32 (checked when the plan is made): 32 x 32 -> 64-bit multiply-adds
+      const unsigned long off = (unsigned long)(unsigned)(rr & (P.g - 1)) * (unsigned)sh + (unsigned long)(unsigned)qi * (unsigned)sn;
+      st.raw[t] = load8(base + off + 8 * (lane % CPR));
     }
     const int qi = min(i0 + pq, P.n - 1);
     const long srow = ((long)b * P.hkv * P.g + hq) * P.n + qi;

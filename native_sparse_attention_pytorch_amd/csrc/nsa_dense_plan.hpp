@@ -52,6 +52,7 @@ static inline int make_dense_plan(const nsa_dense_desc* d, DensePlan& P) {
   for (int t = 0; t < 3; ++t) {
     P.sq[t] = d->q_stride[t]; P.sk[t] = d->k_stride[t]; P.sv[t] = d->v_stride[t]; P.so[t] = d->o_stride[t]; P.sdo[t] = d->do_stride[t];
     if ((P.sq[t] | P.sk[t] | P.sv[t] | P.so[t] | P.sdo[t]) & 7) return NSA_E_ARG;
+    if (t > 0 && ((P.sq[t] | P.sdo[t]) < 0 || ((P.sq[t] | P.sdo[t]) >> 32))) return NSA_E_UNSUPPORTED;      // 32-bit stride arithmetic in the dK/dV gathers
   }
   // dK/dV walk: 64-row tiles of k/v (memory slots included), the queries that can see a tile
   // are cut into chunks of chunk_q; smaller chunks when there would be too few work-groups
