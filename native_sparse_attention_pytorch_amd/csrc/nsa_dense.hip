@@ -31,7 +31,7 @@ __device__ __forceinline__ Interval visible_range(const DensePlan& P, int i) {
     r.hi = min(P.nkeys - 1, i + P.wf);
   } else {
     r.lo = 0;
-    r.hi = P.causal ? min(P.nkeys - 1, i / P.st - 1) : P.nkeys - 1;
+    r.hi = P.causal ? min(P.nkeys - 1, (P.st_sh >= 0 ? (i >> P.st_sh) : i / P.st) - 1) : P.nkeys - 1;
   }
   return r;
 }

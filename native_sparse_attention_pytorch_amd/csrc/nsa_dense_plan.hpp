@@ -9,6 +9,7 @@ namespace nsa {
 struct DensePlan {
   int b, hkv, g, lg, n, nkeys, mem, krows, D, bh;
   int mode, causal, wb, wf, st;
+  int st_sh;                 // log2(st) when the stride is a power of two (the division becomes a shift), else -1
   int pool, npf, nb, B, share, mask_own;
   float scale;
   int key_tiles, chunks, chunk_q;
@@ -49,6 +50,8 @@ static inline int make_dense_plan(const nsa_dense_desc* d, DensePlan& P) {
       if (P.nb == 0) P.pool = 0;
     }
   }
+  P.st_sh = -1;
+  if (P.st > 0 && !(P.st & (P.st - 1))) { P.st_sh = 0; while ((1 << P.st_sh) < P.st) ++P.st_sh; }
   for (int t = 0; t < 3; ++t) {
     P.sq[t] = d->q_stride[t]; P.sk[t] = d->k_stride[t]; P.sv[t] = d->v_stride[t]; P.so[t] = d->o_stride[t]; P.sdo[t] = d->do_stride[t];
     if ((P.sq[t] | P.sk[t] | P.sv[t] | P.so[t] | P.sdo[t]) & 7) return NSA_E_ARG;
