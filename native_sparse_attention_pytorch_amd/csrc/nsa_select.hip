@@ -825,6 +825,9 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 // [key][row] in LDS; dQ^T = K^T dS^T is then formed with both operands read through the
 // transpose load (K block row-major in LDS, loaded once per unit), each wave taking half of the
 // features, and the finished 32 x D tile leaves through coalesced row stores.
+#ifndef NSA_BWD_STAGES_D64
+#define NSA_BWD_STAGES_D64 1
+#endif
 #ifndef NSA_BWD_D64_WAVES
 #define NSA_BWD_D64_WAVES 2
 #endif
@@ -867,7 +870,9 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
 
   // the first list entries, then the block's K / V rows: all requested before anything waits
   const int ppt = 32 >> P.lg;
-  constexpr int NS = KT == 1 ? 1 : NSA_BWD_STAGES;      // a single wave gathers both tiles: no registers for a second stage
+  // a single wave gathers both tiles: no registers for a second stage; at d = 64 the kernel runs two waves per SIMD in 256
+  // registers, where a second stage only adds spills (measured at b4 n4096: 375 us with one stage, 460 us with two)
+  constexpr int NS = KT == 1 ? 1 : (D == 64 ? NSA_BWD_STAGES_D64 : NSA_BWD_STAGES);
   RawEntry e0[NS];
 #pragma unroll
   for (int s2 = 0; s2 < NS; ++s2) e0[s2] = fetch_entry(P, list, ui, ui.v0 + s2 * ppt, n_);
