@@ -44,7 +44,7 @@ int nsa_selftest_mfma(const void* A, const void* B, float* C, const void* X, flo
  * the keys j <= i of its own block (TRI.py include_block_causal).  The `group` query heads
  * h*group .. h*group+group-1 share kv head h and its selection.
  * Limits (NSA_E_UNSUPPORTED otherwise): dim_head 64 or 128, 1 <= block <= 64, group a power of two <= 32,
- * num_sel <= 62, at most 16384 blocks.
+ * num_sel <= 62, at most 16384 blocks, head and token strides of q / out below 2^32 elements.
  * ------------------------------------------------------------------------------------------ */
 typedef struct nsa_select_desc {
   int32_t batch, kv_heads, group, seq, num_sel, block, dim_head, causal;
@@ -103,7 +103,8 @@ int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const
  *                     sel_block / stride must be a power of two <= 32 (with sel_block == stride the
  *                     output holds one logit per compressed key, which serves every other ratio).
  * out/lse as for nsa_select_fwd; dq contiguous [batch, heads, seq, d]; dk, dv contiguous
- * [batch, kv_heads, num_mem + num_keys, d].  bf16 in, fp32 accumulate, bf16 out.
+ * [batch, kv_heads, num_mem + num_keys, d].  bf16 in, fp32 accumulate, bf16 out.  Head and token strides of
+ * q / d_out below 2^32 elements (NSA_E_UNSUPPORTED otherwise).
  * ------------------------------------------------------------------------------------------ */
 typedef struct nsa_dense_desc {
   int32_t batch, kv_heads, group, seq, num_keys, num_mem, dim_head;
