@@ -603,6 +603,52 @@ def _rope_backward(ctx, dout):
 rope_op.register_autograd(_rope_backward, setup_context=_rope_setup)
 
 
+# q and k of a layer in one operator call: at small shapes a layer's step is bound by the host-side cost of its
+# operator calls (~70 us each through torch.library), not by the kernels
+@torch.library.custom_op("nsa_amd::rope_pair", mutates_args=())
+def rope_pair_op(q: Tensor, k: Tensor, freqs: Tensor, offset: int, inverse: bool) -> tuple[Tensor, Tensor]:
+    freqs = freqs.detach().to(torch.float32).contiguous()
+    outs = []
+    for x in (q, k):
+        x = _prep(x)
+        b, h, n, d = x.shape
+        out = torch.empty((b, h, n, d), dtype=_BF16, device=x.device)
+        _lib.check(_lib.lib().nsa_rope(_ptr(x), _s3(x), b, h, n, d, _ptr(freqs), int(offset), int(inverse), _ptr(out), None, _stream()), "nsa_rope")
+        outs.append(out)
+    return outs[0], outs[1]
+
+
+@rope_pair_op.register_fake
+def _(q, k, freqs, offset, inverse):
+    return q.new_empty(q.shape), k.new_empty(k.shape)
+
+
+def _rope_pair_setup(ctx, inputs, output):
+    _, _, freqs, offset, inverse = inputs
+    ctx.save_for_backward(freqs)
+    ctx.args = (offset, inverse)
+
+
+def _rope_pair_backward(ctx, dq, dk):
+    (freqs,) = ctx.saved_tensors
+    offset, inverse = ctx.args
+    dq, dk = rope_pair_op(dq if dq.dtype == _BF16 else dq.to(_BF16), dk if dk.dtype == _BF16 else dk.to(_BF16), freqs, offset, not inverse)
+    return dq, dk, None, None, None
+
+
+rope_pair_op.register_autograd(_rope_pair_backward, setup_context=_rope_pair_setup)
+
+
+def rotary_pair(q: Tensor, k: Tensor, freqs: Tensor, offset: int = 0):
+    """`rotary` of the queries and the keys of a layer in one operator call."""
+    d = q.shape[-1]
+    D = _kernel_dim(d)
+    if D == d:
+        return rope_pair_op(q, k, freqs, int(offset), False)
+    rq, rk = rope_pair_op(_pad_dim(q, D), _pad_dim(k, D), _pad_dim(freqs, D // 2), int(offset), False)
+    return rq[..., :d], rk[..., :d]
+
+
 def rotary(x: Tensor, freqs: Tensor, offset: int = 0) -> Tensor:
     """Rotary embedding of 'b h n d' queries or keys at positions offset .. offset+n-1 (NSA.py:643)."""
     d = x.shape[-1]
@@ -806,6 +852,79 @@ def _windows_backward(ctx, dwin):
 
 
 windows_fwd.register_autograd(_windows_backward, setup_context=_windows_setup)
+
+
+# keys and values of a layer in one operator call (see rope_pair_op)
+@torch.library.custom_op("nsa_amd::windows_pair_fwd", mutates_args=())
+def windows_pair_fwd(k: Tensor, v: Tensor, kpos: Tensor, vpos: Tensor, block: int, stride: int) -> tuple[Tensor, Tensor]:
+    outs = []
+    for x, pos in ((k, kpos), (v, vpos)):
+        x = _prep(x)
+        b, h, n, d = x.shape
+        w = n // stride
+        out = torch.empty((b, h, w, block, d), dtype=_BF16, device=x.device)
+        pos = pos.to(_BF16).contiguous()
+        if pos.shape != (h, block, d):
+            raise RuntimeError("window positions must be 'h block d'")
+        if w > 0:
+            _lib.check(_lib.lib().nsa_windows_fwd(_ptr(x), _s3(x), _ptr(pos), b, h, n, d, int(block), int(stride), _ptr(out), _stream()), "nsa_windows_fwd")
+        outs.append(out)
+    return outs[0], outs[1]
+
+
+@windows_pair_fwd.register_fake
+def _(k, v, kpos, vpos, block, stride):
+    b, h, n, d = k.shape
+    return k.new_empty((b, h, n // stride, block, d)), v.new_empty((b, h, n // stride, block, d))
+
+
+@torch.library.custom_op("nsa_amd::windows_pair_bwd", mutates_args=())
+def windows_pair_bwd(dkw: Tensor, dvw: Tensor, n: int, stride: int) -> tuple[Tensor, Tensor]:
+    outs = []
+    for dwin in (dkw, dvw):
+        dwin = dwin.contiguous()
+        if dwin.dtype != _BF16:
+            raise RuntimeError("window gradients must be bfloat16")
+        b, h, w, block, d = dwin.shape
+        dx = torch.empty((b, h, n, d), dtype=_BF16, device=dwin.device)
+        if w == 0:
+            dx.zero_()
+        else:
+            _lib.check(_lib.lib().nsa_windows_bwd(_ptr(dwin), b, h, n, d, block, int(stride), _ptr(dx), _stream()), "nsa_windows_bwd")
+        outs.append(dx)
+    return outs[0], outs[1]
+
+
+@windows_pair_bwd.register_fake
+def _(dkw, dvw, n, stride):
+    b, h, w, block, d = dkw.shape
+    return dkw.new_empty((b, h, n, d)), dvw.new_empty((b, h, n, d))
+
+
+def _windows_pair_setup(ctx, inputs, output):
+    k, v, kpos, vpos, block, stride = inputs
+    ctx.n, ctx.stride = k.shape[2], stride
+    ctx.pos_dtypes = (kpos.dtype, vpos.dtype)
+
+
+def _windows_pair_backward(ctx, dkw, dvw):
+    dkw = dkw if dkw.dtype == _BF16 else dkw.to(_BF16)
+    dvw = dvw if dvw.dtype == _BF16 else dvw.to(_BF16)
+    dk, dv = windows_pair_bwd(dkw, dvw, ctx.n, ctx.stride)
+    dkpos = dkw.sum(dim=(0, 2), dtype=torch.float32).to(ctx.pos_dtypes[0])
+    dvpos = dvw.sum(dim=(0, 2), dtype=torch.float32).to(ctx.pos_dtypes[1])
+    return dk, dv, dkpos, dvpos, None, None
+
+
+windows_pair_fwd.register_autograd(_windows_pair_backward, setup_context=_windows_pair_setup)
+
+
+def compress_windows_pair(k: Tensor, v: Tensor, kpos: Tensor, vpos: Tensor, block: int, stride: int):
+    """`compress_windows` of the keys and the values of a layer in one operator call."""
+    d = k.shape[-1]
+    D = _kernel_dim(d)
+    kw, vw = windows_pair_fwd(_pad_dim(k, D), _pad_dim(v, D), _pad_dim(kpos, D), _pad_dim(vpos, D), int(block), int(stride))
+    return kw[..., :d], vw[..., :d]
 
 
 def compress_windows(x: Tensor, pos: Tensor | None, block: int, stride: int) -> Tensor:

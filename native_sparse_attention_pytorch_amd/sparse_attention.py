@@ -251,8 +251,8 @@ class SparseAttention(nn.Module):
         # compressed keys / values from the un-rotated k, v
         L = (n // st) * st
         # window gather + intra-window positions in one HIP kernel per tensor (NSA.py:589-603)
-        kw = ops.compress_windows(k.to(bf16), self.k_intrablock_positions, cbs, st).to(k.dtype)
-        vw = ops.compress_windows(v.to(bf16), self.v_intrablock_positions, cbs, st).to(v.dtype)
+        kw, vw = ops.compress_windows_pair(k.to(bf16), v.to(bf16), self.k_intrablock_positions, self.v_intrablock_positions, cbs, st)
+        kw, vw = kw.to(k.dtype), vw.to(v.dtype)
         ck0, cv0 = self.k_compress(kw), self.v_compress(vw)
         mem_k, mem_v = self.compress_mem_kv[0].to(ck0.dtype), self.compress_mem_kv[1].to(cv0.dtype)
         ck = torch.cat((mem_k[None].expand(b, -1, -1, -1), ck0), dim=-2)
@@ -265,8 +265,7 @@ class SparseAttention(nn.Module):
                                          sel_block=B if want_sel else None, share=share)
 
         # rotary positions for the selection and sliding branches (NSA.py:643), one HIP kernel each
-        rq16 = ops.rotary(q.to(bf16), self.rotary_emb.freqs)
-        rk16 = ops.rotary(k.to(bf16), self.rotary_emb.freqs)
+        rq16, rk16 = ops.rotary_pair(q.to(bf16), k.to(bf16), self.rotary_emb.freqs)
         v16 = v.to(bf16)
 
         num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
