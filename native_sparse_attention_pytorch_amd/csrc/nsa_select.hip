@@ -205,7 +205,7 @@ __global__ __launch_bounds__(64) void sel_fill_kernel(const SelPlan P, const voi
       if (j >= P.W) j = -1;
       entry = (q0 + e / P.S) * P.SP + e % P.S;
     }
-    // lanes of this round that name the same block: intersect, bit by bit of the block index, the ballots of the lanes
+    // lanes of this pass that name the same block: intersect, bit by bit of the block index, the ballots of the lanes
     // that agree with this lane (about 10 ballots instead of 64 lane reads); dead lanes are masked out
     unsigned long long same_m = __ballot(j >= 0);
     for (int bit = 0; bit < nbits; ++bit) {
