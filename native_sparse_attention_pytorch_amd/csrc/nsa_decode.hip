@@ -16,6 +16,10 @@
 #include "nsa_common.hpp"
 #include "../../include/nsa_hip.h"
 
+#ifndef NSA_DECODE_WG_TARGET
+#define NSA_DECODE_WG_TARGET 4096     // work-groups of one attend launch beyond which the key range is not split further (batch 32, 32k context: 2048 -> 197 us per step, 4096 and more -> 187 us)
+#endif
+
 namespace nsa {
 
 struct DecodePlan {
@@ -388,7 +392,7 @@ static int make_decode_plan(const nsa_decode_desc* dsc, DecodePlan& P) {
   if (units > 65535) return NSA_E_UNSUPPORTED;
   // split-K: about two tiles per wave, but no more work-groups than a few per CU
   int ns = (P.tiles + 2 * kDecodeWaves - 1) / (2 * kDecodeWaves);
-  const long cap = units >= 2048 ? 1 : 2048 / units;
+  const long cap = units >= NSA_DECODE_WG_TARGET ? 1 : NSA_DECODE_WG_TARGET / units;
   if (ns > cap) ns = (int)cap;
   if (ns > 64) ns = 64;
   if (ns < 1) ns = 1;
