@@ -16,6 +16,9 @@
 #include "nsa_common.hpp"
 #include "../../include/nsa_hip.h"
 
+#ifndef NSA_DECODE_TILES_PER_WAVE
+#define NSA_DECODE_TILES_PER_WAVE 2     // measured at 32k context: 1 tile per wave 197 us (batch 32), 4 tiles 96 us (batch 1) against 187 / 90 us
+#endif
 #ifndef NSA_DECODE_WG_TARGET
 #define NSA_DECODE_WG_TARGET 4096     // work-groups of one attend launch beyond which the key range is not split further (batch 32, 32k context: 2048 -> 197 us per step, 4096 and more -> 187 us)
 #endif
@@ -391,7 +394,7 @@ static int make_decode_plan(const nsa_decode_desc* dsc, DecodePlan& P) {
   const long units = (long)P.b * P.units;
   if (units > 65535) return NSA_E_UNSUPPORTED;
   // split-K: about two tiles per wave, but no more work-groups than a few per CU
-  int ns = (P.tiles + 2 * kDecodeWaves - 1) / (2 * kDecodeWaves);
+  int ns = (P.tiles + NSA_DECODE_TILES_PER_WAVE * kDecodeWaves - 1) / (NSA_DECODE_TILES_PER_WAVE * kDecodeWaves);
   const long cap = units >= NSA_DECODE_WG_TARGET ? 1 : NSA_DECODE_WG_TARGET / units;
   if (ns > cap) ns = (int)cap;
   if (ns > 64) ns = 64;
