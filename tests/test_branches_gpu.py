@@ -130,7 +130,7 @@ def test_importance_logits_gradient_matches_oracle():
 def test_topk_bit_exact_on_given_scores():
     from native_sparse_attention_pytorch_amd.ops import topk_op
     g = torch.Generator().manual_seed(0)
-    for nb, k in [(5, 2), (64, 16), (100, 16), (512, 16), (700, 9), (33, 33)]:
+    for nb, k in [(5, 2), (64, 16), (100, 16), (512, 16), (700, 9), (33, 33), (128, 16), (256, 7), (300, 12), (510, 16), (64, 1), (17, 16)]:
         s = torch.rand(3, 2, 50, nb, generator=g)
         s = (s * 8).round() / 8 if nb % 2 == 0 else s           # many exact ties on even sizes
         s[0, 0, :5] = 0.0                                        # all-zero rows (early queries)
