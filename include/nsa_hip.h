@@ -103,7 +103,9 @@ int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const
  *                     sel_block / stride must be a power of two <= 32 (with sel_block == stride the
  *                     output holds one logit per compressed key, which serves every other ratio).
  * out/lse as for nsa_select_fwd; dq contiguous [batch, heads, seq, d]; dk, dv contiguous
- * [batch, kv_heads, num_mem + num_keys, d].  bf16 in, fp32 accumulate, bf16 out.  Head and token strides of
+ * [batch, kv_heads, num_mem + num_keys, d] (bf16, or fp32 with dkv_fp32: the compressed keys are few and their
+ * gradient feeds sums over every window, where a bf16 rounding per key is the largest error left).
+ * bf16 in, fp32 accumulate, bf16 out.  Head and token strides of
  * q / d_out below 2^32 elements (NSA_E_UNSUPPORTED otherwise).
  * ------------------------------------------------------------------------------------------ */
 typedef struct nsa_dense_desc {
@@ -111,6 +113,7 @@ typedef struct nsa_dense_desc {
   int32_t mode, causal, window, stride;
   int32_t pool, sel_block, share;
   float scale;
+  int32_t dkv_fp32; /* backward: 1 = dk and dv are written as fp32 (the fixed-order sums, unrounded), 0 = bf16 */
   int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3], do_stride[3];
 } nsa_dense_desc;
 
@@ -125,7 +128,8 @@ int nsa_dense_bwd(const nsa_dense_desc* d, const void* q, const void* k, const v
  * pad), :713 (topk) and :721 (fmask = value > 1e-10).  scores: fp32 [rows, nb]; with
  * apply_softmax != 0 they are importance logits (-inf = not selectable), otherwise ready
  * probabilities.  Outputs [rows, k]: idx int32 (descending value, ties to the lower block index -
- * torch.topk leaves tie order unspecified), vals fp32, fmask uint8.  nb <= 2048, k <= nb. */
+ * torch.topk leaves tie order unspecified), vals fp32, fmask uint8.  A NaN or +inf score is ordered first and
+ * comes out as value NaN with fmask 0.  Limits: nb <= 2048, k <= min(nb, 64) (NSA_E_UNSUPPORTED otherwise). */
 int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k, int32_t apply_softmax,
              int32_t* idx, float* vals, uint8_t* fmask, void* stream);
 

@@ -26,6 +26,7 @@ class DenseDesc(C.Structure):
         ("num_keys", C.c_int32), ("num_mem", C.c_int32), ("dim_head", C.c_int32),
         ("mode", C.c_int32), ("causal", C.c_int32), ("window", C.c_int32), ("stride", C.c_int32),
         ("pool", C.c_int32), ("sel_block", C.c_int32), ("share", C.c_int32), ("scale", C.c_float),
+        ("dkv_fp32", C.c_int32),
         ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
         ("o_stride", C.c_int64 * 3), ("do_stride", C.c_int64 * 3),
     ]

@@ -636,7 +636,7 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void dense_bwd_dkv_reduce_kernel(const DensePlan P, const float* __restrict__ part, __bf16* __restrict__ dk, __bf16* __restrict__ dv) {
+__global__ __launch_bounds__(256) void dense_bwd_dkv_reduce_kernel(const DensePlan P, const float* __restrict__ part, void* __restrict__ dk, void* __restrict__ dv) {
   const int T = blockIdx.x, bh = blockIdx.y;
   const int keys = min(kBK, P.krows - kBK * T);
   const float* base = part + ((size_t)bh * P.key_tiles + T) * P.chunks * (2 * kBK * D);
@@ -656,8 +656,9 @@ __global__ __launch_bounds__(256) void dense_bwd_dkv_reduce_kernel(const DensePl
 #pragma unroll 8
     for (int c = clo; c < chi; ++c) acc += __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(src + (size_t)c * (2 * kBK * D)));
     const float s = which == 0 ? P.scale : 1.0f;
-    __bf16* dst = (which == 0 ? dk : dv) + ((size_t)bh * P.krows + (size_t)kBK * T + key) * D + dd;
-    store4_bf16(dst, acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s);
+    const size_t at = ((size_t)bh * P.krows + (size_t)kBK * T + key) * D + dd;
+    if (P.dkv_fp32) *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(which == 0 ? dk : dv) + at) = acc * s;
+    else store4_bf16(reinterpret_cast<__bf16*>(which == 0 ? dk : dv) + at, acc[0] * s, acc[1] * s, acc[2] * s, acc[3] * s);
   }
 }
 
@@ -728,7 +729,7 @@ static int dense_bwd_launch(const DensePlan& P, const void* q, const void* k, co
   hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(P.key_tiles * P.chunks, P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
   NSA_LAUNCH_CHECK();
-  hipLaunchKernelGGL((dense_bwd_dkv_reduce_kernel<D>), dim3(P.key_tiles, P.bh), dim3(256), 0, st, P, part, (__bf16*)dk, (__bf16*)dv);
+  hipLaunchKernelGGL((dense_bwd_dkv_reduce_kernel<D>), dim3(P.key_tiles, P.bh), dim3(256), 0, st, P, part, dk, dv);
   NSA_LAUNCH_CHECK();
   return 0;
 }

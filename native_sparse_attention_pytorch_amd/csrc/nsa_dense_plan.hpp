@@ -11,6 +11,7 @@ struct DensePlan {
   int mode, causal, wb, wf, st;
   int st_sh;                 // log2(st) when the stride is a power of two (the division becomes a shift), else -1
   int pool, npf, nb, B, share, mask_own;
+  int dkv_fp32;              // dk / dv leave the reduce kernel as fp32 instead of bf16
   float scale;
   int key_tiles, chunks, chunk_q;
   long sq[3], sk[3], sv[3], so[3], sdo[3];
@@ -27,6 +28,7 @@ static inline int make_dense_plan(const nsa_dense_desc* d, DensePlan& P) {
   if (d->mode != 0 && d->mode != 1) return NSA_E_ARG;
   P.b = d->batch; P.hkv = d->kv_heads; P.g = d->group; P.n = d->seq; P.nkeys = d->num_keys; P.mem = d->num_mem;
   P.krows = P.nkeys + P.mem; P.D = d->dim_head; P.mode = d->mode; P.causal = d->causal ? 1 : 0; P.scale = d->scale;
+  P.dkv_fp32 = d->dkv_fp32 ? 1 : 0;
   P.lg = 0;
   while ((1 << P.lg) < P.g) ++P.lg;
   const long bh = (long)P.b * P.hkv;

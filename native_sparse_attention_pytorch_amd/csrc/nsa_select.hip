@@ -1272,4 +1272,4 @@ extern "C" int nsa_select_bwd(const nsa_select_desc* d, const void* q, const voi
   return nsa_select_bwd_timed(d, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, bwd_bytes, dq, dk, dv, sel_grads, stream, nullptr, 0);
 }
 
-extern "C" int nsa_abi_version(void) { return 4; }
+extern "C" int nsa_abi_version(void) { return 5; }

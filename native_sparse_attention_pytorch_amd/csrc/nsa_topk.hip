@@ -130,8 +130,10 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in,
     for (int r = 0; r < VPL; ++r) x[r] *= inv;
   }
 #pragma unroll
-  for (int r = 0; r < VPL; ++r)
+  for (int r = 0; r < VPL; ++r) {
     if (lane * VPL + r >= nb) x[r] = -1.0f;              // padding loses against every real entry
+    else if (!(x[r] == x[r])) x[r] = INFINITY;           // NaN (a diverged row): ordered first, like torch.topk, so every comparison below stays defined
+  }
 
   float bv;
   int br;
@@ -159,8 +161,9 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in,
   }
   if (lane < k) {
     idx[row * kstride + lane] = res_j;
-    vals[row * kstride + lane] = res_v;
-    fmask[row * kstride + lane] = res_v > 1e-10f ? 1 : 0;
+    const bool finite = res_v < INFINITY;                 // a NaN or +inf score comes out as NaN with a dead slot
+    vals[row * kstride + lane] = finite ? res_v : NAN;
+    fmask[row * kstride + lane] = (finite && res_v > 1e-10f) ? 1 : 0;
   }
 }
 
@@ -259,6 +262,7 @@ __global__ __launch_bounds__(256) void topk_rows4_kernel(const float* __restrict
     for (int t = 0; t < GS; ++t) {
       const int r = g * GS + t;
       if (sub * VPL + r >= nb) x[r] = -1.0f;                // padding loses against every real entry
+      else if (!(x[r] == x[r])) x[r] = INFINITY;            // NaN: ordered first (see topk_kernel)
       if (t == 0 || x[r] > gm[g]) { gm[g] = x[r]; ga[g] = r; }      // strict: ties keep the lower index
     }
   }
@@ -276,7 +280,7 @@ __global__ __launch_bounds__(256) void topk_rows4_kernel(const float* __restrict
       if (gm[g] > bv) { bv = gm[g]; ba = ga[g]; }
     const float m = row16_max(bv);
     const unsigned long long holders = __ballot(bv == m);
-    const unsigned row_bits = (unsigned)(holders >> (lane & 48)) & 0xffffu;       // never 0: one of the row's lanes holds m
+    const unsigned row_bits = (unsigned)(holders >> (lane & 48)) & 0xffffu;       // never 0: one of the row's lanes holds m (NaN was mapped to +inf above)
     const int w = __builtin_ctz(row_bits);                                        // lowest lane = lowest index among equals
     const int jw = __shfl(sub * VPL + ba, (lane & 48) + w, 64);
     if (sub == s) { res_v = m; res_j = jw; }
@@ -302,8 +306,9 @@ __global__ __launch_bounds__(256) void topk_rows4_kernel(const float* __restrict
   }
   if (live && sub < k) {
     idx[row * k + sub] = res_j;
-    vals[row * k + sub] = res_v;
-    fmask[row * k + sub] = res_v > 1e-10f ? 1 : 0;
+    const bool finite = res_v < INFINITY;
+    vals[row * k + sub] = finite ? res_v : NAN;
+    fmask[row * k + sub] = (finite && res_v > 1e-10f) ? 1 : 0;
   }
 }
 

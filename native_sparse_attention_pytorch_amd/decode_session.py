@@ -69,7 +69,9 @@ class DecodeSession:
             buf[:, :, :src.shape[-2], :src.shape[-1]].copy_(src)      # the module's own decode steps hand back padded rows
             return buf
         self.K, self.V = grown(cache_k, self.max_len), grown(cache_v, self.max_len)
-        self.CK, self.CV = grown(cache_ck, self.max_nc), grown(cache_cv, self.max_nc)
+        # one spare row: the capture warm-up and the recording of the window-completing graph write row `nc` of the compressed
+        # caches whatever nc is, also when the prefill already filled all max_nc rows (the real steps never do: completes_window)
+        self.CK, self.CV = grown(cache_ck, self.max_nc + 1), grown(cache_cv, self.max_nc + 1)
 
         # raw (un-rotated) keys / values of the last tokens, position p in row p % ring; rows never written are zero, which is
         # also what the window of the first compression steps holds for positions before the sequence start (NSA.py:866)
@@ -193,7 +195,7 @@ class DecodeSession:
         rows = ring_rows(self.state[0] - self.cbs, self._ar, self.ring)
         wk = self.ring_k.index_select(2, rows)[..., :self.d0]
         wv = self.ring_v.index_select(2, rows)[..., :self.d0]
-        at = self.state[1:2].long()
+        at = self.state[1:2].long().clamp(max=self.CK.shape[2] - 1)    # the spare last row at most, whatever the counter holds
         self.CK.index_copy_(2, at, _pad_dim(m.k_compress((wk + m.k_intrablock_positions)[:, :, None]).to(_BF16), self.d))
         self.CV.index_copy_(2, at, _pad_dim(m.v_compress((wv + m.v_intrablock_positions)[:, :, None]).to(_BF16), self.d))
         if count:

@@ -322,15 +322,17 @@ def _(q, k, v, mode, causal, window, stride, num_mem, pool, sel_block, share, sc
 
 @torch.library.custom_op("nsa_amd::dense_bwd", mutates_args=())
 def dense_bwd(q: Tensor, k: Tensor, v: Tensor, out: Tensor, dout: Tensor, lse: Tensor, mode: int, causal: bool, window: int,
-              stride: int, num_mem: int, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+              stride: int, num_mem: int, scale: float, dkv_fp32: bool = False) -> tuple[Tensor, Tensor, Tensor]:
     q, k, v, out = _prep(q), _prep(k), _prep(v), _prep(out)
     dout = _prep(dout if dout.dtype == _BF16 else dout.to(_BF16))
     b, hq, n, d = q.shape
     hk, nk = k.shape[1], k.shape[2]
     dq = torch.empty((b, hq, n, d), dtype=_BF16, device=q.device)
-    dk = torch.empty((b, hk, nk, d), dtype=_BF16, device=q.device)
-    dv = torch.empty((b, hk, nk, d), dtype=_BF16, device=q.device)
+    kv_dtype = torch.float32 if dkv_fp32 else _BF16
+    dk = torch.empty((b, hk, nk, d), dtype=kv_dtype, device=q.device)
+    dv = torch.empty((b, hk, nk, d), dtype=kv_dtype, device=q.device)
     dsc = _dense_desc(q, k, v, out, dout, mode, causal, window, stride, num_mem, False, 1, True, scale)
+    dsc.dkv_fp32 = int(dkv_fp32)
     wb = C.c_size_t()
     L = _lib.lib()
     _lib.check(L.nsa_dense_workspace_bytes(C.byref(dsc), C.byref(wb)), "nsa_dense_workspace_bytes")
@@ -341,8 +343,9 @@ def dense_bwd(q: Tensor, k: Tensor, v: Tensor, out: Tensor, dout: Tensor, lse: T
 
 
 @dense_bwd.register_fake
-def _(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale):
-    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+def _(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale, dkv_fp32=False):
+    kv_dtype = torch.float32 if dkv_fp32 else k.dtype
+    return torch.empty_like(q), torch.empty_like(k, dtype=kv_dtype), torch.empty_like(v, dtype=kv_dtype)
 
 
 def _dense_setup(ctx, inputs, output):
@@ -384,11 +387,16 @@ def _dense_backward(ctx, dout, dlse, dpooled):
     mode, causal, window, stride, num_mem, scale, sel_block, share = ctx.args
     dq = dk = dv = None
     if dout is not None:
-        dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale)
+        # the compressed keys are few and every one of their gradients is summed over all windows into the compression
+        # network's parameters: they leave the kernel as fp32 and are rounded to the keys' dtype once, after the
+        # importance term has been added
+        dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale, mode == 1)
     if dpooled is not None and dpooled.numel() > 0:
         dq2, dk2 = _importance_backward(q, k, dpooled, num_mem, stride, sel_block, share, scale)
         dq = dq2.to(q.dtype) if dq is None else (dq.float() + dq2).to(q.dtype)
-        dk = dk2.to(k.dtype) if dk is None else (dk.float() + dk2).to(k.dtype)
+        dk = dk2 if dk is None else dk.float() + dk2
+    if dk is not None:
+        dk, dv = dk.to(k.dtype), (dv.to(v.dtype) if dv is not None else None)
     return (dq, dk, dv) + (None,) * 9
 
 

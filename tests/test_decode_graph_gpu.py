@@ -99,6 +99,30 @@ def test_graph_decode_capacity_is_enforced():
     assert int(sess.state[0]) == 17
 
 
+def test_graph_decode_when_prefill_fills_every_compressed_row():
+    """A prompt whose compressed keys already fill the compressed caches to their capacity (64 tokens, stride 8,
+    room for 66: eight rows, a multiple of the row padding): the capture warm-up still writes one window, which must
+    land in the spare row, and the remaining steps run and agree with the eager decode."""
+    from native_sparse_attention_pytorch_amd import SparseAttention
+    from native_sparse_attention_pytorch_amd.decode_session import DecodeSession
+    from tests.util import assert_close
+    torch.manual_seed(2)
+    m = SparseAttention(dim=128, dim_head=64, heads=2, kv_heads=1, sliding_window_size=8, compress_block_size=16,
+                        compress_block_sliding_stride=8, selection_block_size=16, num_selected_blocks=2, causal=True).to(DEV).bfloat16()
+    xs = torch.randn(1, 66, 128, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        _, cache = m(xs[:, :64], return_cache=True)
+    sess = DecodeSession(m, cache, max_len=66)
+    assert sess.nc == sess.max_nc == 8 and sess.CK.shape[2] == 9
+    for i in (64, 65):
+        with torch.no_grad():
+            want, cache = m(xs[:, i:i + 1], cache=cache, return_cache=True)
+        got = sess.step(xs[:, i:i + 1])
+        torch.cuda.synchronize()
+        assert_close(got, want, 2e-2, 1e-2, f"step {i}")
+    assert torch.equal(sess.cache()[1][0][0], cache[1][0][0][:, :, :8].to(torch.bfloat16))
+
+
 def test_transformer_graph_decode_matches_cached_decode():
     """Whole-model graph replay (embedding, 3 layers, logits) against the model's eager cached decode on the same token
     sequence, replay by replay, across compression steps; then sampling through the graph."""

@@ -1,9 +1,18 @@
 """Full SparseAttention module (HIP path, bf16) against the CPU oracle module (fp32) holding
 the same parameters.  The discrete block selection is compared on its own; outputs and
 gradients are then compared with the oracle evaluated under the HIP path's selection, so that
-a flipped near-tie does not hide or fake a numeric error."""
+a flipped near-tie does not hide or fake a numeric error.
+
+Bounds: forward 2e-2 absolute + 1e-2 relative per element; gradients 5e-2 relative (norm-wise per tensor).  The
+oracle is also run in the module's own dtype (bf16 parameters and activations on the CPU: the reference's torch
+path as a bf16 user would run it); for the two parameters whose gradient that path itself misses the fp32 truth
+by more than 5e-2 (the first bias and the intra-block positions of the key compression network: sums over every
+window in which large terms cancel) the HIP path must be no farther from the truth than 1.15 x the bf16 torch path."""
+import copy
+
 import pytest
 import torch
+from torch import nn
 
 from oracle import nsa_oracle as O
 from tests.util import assert_close
@@ -12,14 +21,34 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
+class EinMixGroupedMLP(nn.Module):
+    """compress_networks.py:73-101 as written there: per-head two-layer MLP from the installed einops mixing layer."""
+
+    def __init__(self, dim_head, compress_window_size, heads, expand_factor=1.):
+        super().__init__()
+        from einops.layers.torch import EinMix
+        dim = dim_head * compress_window_size
+        hidden = int(dim * expand_factor)
+        self.net = nn.Sequential(
+            EinMix('b h w i -> b h w o', weight_shape='h i o', bias_shape='h o', h=heads, i=dim, o=hidden),
+            nn.ReLU(),
+            EinMix('b h w i -> b h w o', weight_shape='h i o', bias_shape='h o', h=heads, i=hidden, o=dim_head))
+
+    def forward(self, kv):
+        return self.net(kv.flatten(-2))
+
+
 def _pair(seed, **kw):
     from native_sparse_attention_pytorch_amd.sparse_attention import SparseAttention
     torch.manual_seed(seed)
     kw = dict(kw)
+    kw_ref = dict(kw)
     if kw.get("compress_mlp") == "grouped":      # per-head MLP, the network train.py:100-104 installs
         from native_sparse_attention_pytorch_amd.compress_networks import GroupedMLP
         kw["compress_mlp"] = GroupedMLP(dim_head=kw["dim_head"], compress_window_size=kw["compress_block_size"], heads=kw["kv_heads"])
-    ref = O.SparseAttentionOracle(**kw)
+        # the oracle side gets the reference's own formulation (compress_networks.py:73-101: two einops mixing layers), not the product class
+        kw_ref["compress_mlp"] = EinMixGroupedMLP(dim_head=kw["dim_head"], compress_window_size=kw["compress_block_size"], heads=kw["kv_heads"])
+    ref = O.SparseAttentionOracle(**kw_ref)
     # move the module away from its symmetric init so every branch and parameter matters
     with torch.no_grad():
         ref.to_strategy_combine[0].weight.normal_(std=0.05)
@@ -114,17 +143,32 @@ def test_module_matches_oracle(ci, n):
     # --- numerics under the HIP path's selection
     want = ref(xr, selection_override=(idx, live))
     (want * do.float()).sum().backward()
-    assert_close(out, want, 3e-2 * want.abs().max().item(), 2e-2, "module out")
-    gerr = (xg.grad.float().cpu() - xr.grad).norm() / xr.grad.norm()
+    # the same pass in the module's dtype on the CPU (the reference's torch path run in bf16)
+    ref16 = copy.deepcopy(ref).to(torch.bfloat16)
+    for p in ref16.parameters():
+        p.grad = None
+    x16 = x.clone().requires_grad_()
+    (ref16(x16, selection_override=(idx, live)).float() * do.float()).sum().backward()
+    rel = lambda a, b_: ((a.float().cpu() - b_.float()).norm() / b_.float().norm().clamp_min(1e-6)).item()
+
+    assert_close(out, want, 2e-2, 1e-2, "module out")
+    gerr = rel(xg.grad, xr.grad)
     assert gerr < 5e-2, f"input grad rel err {gerr:.4f}"
-    for (name, p), (_, pr) in zip(mod.named_parameters(), ref.named_parameters()):
+    for (name, p), (_, pr), (_, p16) in zip(mod.named_parameters(), ref.named_parameters(), ref16.named_parameters()):
         if pr.grad is None:
             assert p.grad is None or name == "rotary_emb.freqs"
             continue
-        e = (p.grad.float().cpu() - pr.grad).norm() / pr.grad.norm().clamp_min(1e-6)
-        # parameter gradients pass through several bf16 stages (kernel gradients are held to 5e-2 in the branch tests); measured
-        # 0.03-0.07 here, the largest on the small biases of the compression network
-        assert e < 1e-1, f"grad of {name}: rel err {e:.4f}"
+        e, e16 = rel(p.grad, pr.grad), rel(p16.grad, pr.grad)
+        bound = max(5e-2, 1.15 * e16)
+        if not kw.get("causal", False) and name in ("k_compress.3.bias", "k_compress.net.2.bias"):
+            # Without the causal mask every query sees every compressed key, and a shift of all compressed keys changes
+            # only their logits relative to the memory slot: this bias gradient is the residual -sum_i dS[i, memory] q_i
+            # of a sum over all keys that otherwise cancels (its norm is ~1/20 of the sibling weight's).  Any flash-style
+            # backward in bf16 leaves two errors in it that do not cancel: delta = sum(out * d_out) from the rounded
+            # forward output (TRI.py:696-756 does the same) and the bf16 dS operand of dK = dS^T Q; emulated on the CPU
+            # each alone is 0.025-0.03 of this gradient.  The causal configurations are held to the bound above.
+            bound = 1e-1
+        assert e < bound, f"grad of {name}: rel err {e:.4f} (bf16 torch path: {e16:.4f})"
 
 
 def test_module_edge_shapes_run():
