@@ -196,6 +196,19 @@ int nsa_decode_attend(const nsa_decode_desc* desc, const void* q, const void* k,
                       const void* mem_v, const void* idx, const uint8_t* fmask, void* ws, size_t ws_bytes, void* out,
                       float* logits, void* stream);
 
+/* nsa_decode_attend without a caller workspace and without any allocation: the split-K partials live in a fixed
+ * device array of the library (NSA_DECODE_NOALLOC_SCRATCH_BYTES per GPU, held until the process ends).  No
+ * counterpart in the reference; it is for callers that cannot allocate device memory - a stream under HIP graph
+ * capture, a serving loop or harness that forbids hipMalloc.  Same arguments and results as nsa_decode_attend
+ * with out != NULL (out is required: the partials are private).  NSA_E_WORKSPACE when
+ * nsa_decode_workspace_bytes(desc) exceeds NSA_DECODE_NOALLOC_SCRATCH_BYTES.  All calls on one GPU share the
+ * array: calls that overlap on one GPU (different streams or threads) race; calls ordered on one stream do not.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress) and should be made outside a
+ * stream capture. */
+#define NSA_DECODE_NOALLOC_SCRATCH_BYTES ((size_t)16 << 20)
+int nsa_decode_attend_noalloc(const nsa_decode_desc* desc, const void* q, const void* k, const void* v, const void* mem_k,
+                              const void* mem_v, const void* idx, const uint8_t* fmask, void* out, float* logits, void* stream);
+
 /* Decode step: block selection from the compressed branch's logits.  Replaces the reduce over the
  * compressed keys of a block and over the heads of a group, the padded softmax, topk and the mask of
  * NSA.py:448-476, 502.  logits: fp32 [batch, heads, num_compressed] as written by nsa_decode_attend;

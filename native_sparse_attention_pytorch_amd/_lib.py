@@ -87,6 +87,8 @@ def lib():
         L.nsa_decode_workspace_bytes.argtypes = [C.POINTER(DecodeDesc), C.POINTER(sz)]
         L.nsa_decode_attend.argtypes = [C.POINTER(DecodeDesc)] + [vp] * 8 + [sz, vp, vp, vp]
         L.nsa_decode_workspace_bytes.restype = L.nsa_decode_attend.restype = C.c_int
+        L.nsa_decode_attend_noalloc.argtypes = [C.POINTER(DecodeDesc)] + [vp] * 10
+        L.nsa_decode_attend_noalloc.restype = C.c_int
         dd = C.POINTER(DecodeDesc)
         L.nsa_decode_combine.argtypes = [dd, vp, dd, vp, dd, vp, vp, vp, vp]
         i2 = C.POINTER(C.c_int64)

@@ -499,6 +499,54 @@ extern "C" int nsa_decode_attend(const nsa_decode_desc* dsc, const void* q, cons
   return launch_attend(P, q, k, v, mem_k, mem_v, idx, fmask, ws, ws_bytes, out, logits, stream);
 }
 
+// ------------------------------------------------------------------------------------------------------------
+// nsa_decode_attend for callers that cannot allocate (a stream under graph capture, a serving loop that forbids
+// hipMalloc): the split-K partials go to a fixed device array of this library instead of a caller workspace.
+// Every GPU the library runs on holds its own copy of the array, at its own address, until the process ends; in
+// host code the array's name is only a handle, so the address is looked up once per device with
+// hipGetSymbolAddress and that pointer is what the kernels receive.  All calls on a GPU share the array: calls
+// that overlap on one GPU (two streams, two threads) race.  Nothing has to be cleared between calls: every wave
+// of the attend kernel writes its partial record (a neutral one when it has no tile) before the merge reads it.
+#include <mutex>
+
+namespace nsa {
+constexpr size_t kNoAllocScratchBytes = NSA_DECODE_NOALLOC_SCRATCH_BYTES;
+constexpr int kNoAllocMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+static void* g_scratch_ptr[kNoAllocMaxDevices];       // per device: device address of `scratch`
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kNoAllocMaxDevices) return NSA_E_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return NSA_E_ARG;
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace nsa
+
+extern "C" int nsa_decode_attend_noalloc(const nsa_decode_desc* dsc, const void* q, const void* k, const void* v, const void* mem_k,
+                                         const void* mem_v, const void* idx, const uint8_t* fmask, void* out, float* logits, void* stream) {
+  using namespace nsa;
+  DecodePlan P;
+  if (int e = make_decode_plan(dsc, P)) return e;
+  if (!out) return NSA_E_ARG;                          // the partials are private to the library: the merged output is the result
+  const size_t need = (size_t)P.b * P.units * P.nparts * P.rec * sizeof(float);
+  if (need > kNoAllocScratchBytes) return NSA_E_WORKSPACE;
+  void* ws = nullptr;
+  if (int e = scratch_of_current_device(&ws)) return e;
+  return launch_attend(P, q, k, v, mem_k, mem_v, idx, fmask, ws, kNoAllocScratchBytes, out, logits, stream);
+}
+
 extern "C" int nsa_decode_combine(const nsa_decode_desc* compressed, const void* ws_compressed, const nsa_decode_desc* selected,
                                   const void* ws_selected, const nsa_decode_desc* sliding, const void* ws_sliding,
                                   const void* gate_logits, void* out, void* stream) {
