@@ -12,8 +12,10 @@
 // same walk: dK/dV of a block accumulate on chip in the wave that owns the block (no atomics),
 // dQ partials are merged per query like the forward partials.
 //
-// No LDS staging is used for operands: register transposes are done with an MFMA against a
-// constant identity operand (see make_ident in nsa_common.hpp).
+// The resident K/V block lives in registers as MFMA operands (its transposed form made once per
+// work unit with an MFMA against a constant identity operand, make_ident in nsa_common.hpp); the
+// streamed Q / dO rows are gathered with coalesced 16-byte loads, staged in row-major LDS tiles
+// and read back as row operands or through the LDS transpose load.
 #include "nsa_common.hpp"
 #include "nsa_select_plan.hpp"
 

@@ -31,6 +31,20 @@ What pins each function (see tests/test_oracle_*.py):
   forward_inference, caches   : the reference's own criterion (tests/test_sparse_attn.py:50-118):
                                 token-by-token decode == parallel forward to 1e-5; greedy
                                 sampling with and without caches gives the same tokens
+  SparseAttentionOracle.forward (the wiring of the pieces above: which branch sees rotated q / k,
+                                the gate fed by the normed input, memory slots first) and
+  TransformerOracle.forward   : tests/test_oracle_composition.py - the module output rebuilt from
+                                library attention under the three dense masks of NSA.py:46-109 with a
+                                complex-multiplication rotary and python loops, no function of this
+                                file; the transformer from its closed forms (depth 0, silenced
+                                sub-layers, one hand-rolled layer, hand-written shifted cross entropy)
+
+Two modes.  Called with fp32 (or fp64) parameters and inputs this file is the "truth" the HIP path is
+compared with.  Cast to another dtype (`oracle.to(torch.bfloat16)`, bf16 input) it is the
+dtype-faithful mode: every fill value (-finfo.max // 10, -finfo.max), the -1e3 pad, the softmaxes
+and the GEMMs are evaluated in that dtype exactly as the reference's torch path does when its
+module is cast (NSA.py:131-132, 171, 693, 742); tests use it to tell the error of the HIP kernels
+from the error any bf16 run of the reference has (tests/test_module_gpu.py).
 
 PARITY UNPINNED (third-party packages absent from the reference tree and from this
 image, so no fixture can be produced): the numeric convention of

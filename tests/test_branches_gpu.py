@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import nsa_oracle as O
-from tests.util import assert_close
+from tests.util import assert_close, assert_grad_close
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -16,7 +16,7 @@ def _rand(shape, g, scale=1.0):
 
 
 def _grad_close(got, want, name):
-    assert_close(got, want, 2e-2 * want.abs().max().item() + 1e-6, 5e-2, name)
+    assert_grad_close(got, want, name)
 
 
 SLIDING = [

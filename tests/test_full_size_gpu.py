@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import nsa_oracle as O
-from tests.util import assert_close, causal_random_selection
+from tests.util import assert_close, assert_grad_close, causal_random_selection
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -27,7 +27,7 @@ def _rand(shape, g, scale):
 
 
 def _grad_close(got, want, name):
-    assert_close(got, want, 2e-2 * want.abs().max().item() + 1e-6, 5e-2, name)
+    assert_grad_close(got, want, name)
 
 
 def test_selection_32k_forward_and_backward():

@@ -300,3 +300,29 @@ def test_transformer_one_layer_hand_rolled():
     lg2, _ = model(ids[:, :11], cache=cache, return_cache=True)
     full = model(ids[:, :11])
     assert torch.allclose(lg2[:, -1], full[:, -1], atol=1e-5)
+
+
+# ------------------------------------------------------------------------- dtype-faithful mode
+
+def test_oracle_in_bf16_is_the_same_function_at_bf16_precision():
+    """The oracle cast to bf16 (fill values, pad, softmaxes and GEMMs in that dtype, as the reference's torch path runs
+    when its module is cast) stays within the bf16 forward bound of the fp32 oracle under the same block selection, and
+    its masks hold exactly: a fully masked key gets probability 0 in bf16 as well (causality is not a matter of precision)."""
+    import copy
+    torch.manual_seed(4)
+    m = _randomised(O.SparseAttentionOracle(dim=64, dim_head=16, heads=4, kv_heads=2, sliding_window_size=6, compress_block_size=8,
+                                            compress_block_sliding_stride=4, selection_block_size=8, num_selected_blocks=2, causal=True), 3)
+    with torch.no_grad():
+        for p in m.parameters():
+            p.copy_(p.bfloat16().float())
+    x = torch.randn(2, 70, 64).bfloat16()
+    y32, parts = m(x.float(), return_parts=True)
+    sel = (parts["idx"], parts["vals"] > 1e-10)
+    m16 = copy.deepcopy(m).to(torch.bfloat16)
+    y16 = m16(x, selection_override=sel)
+    assert y16.dtype == torch.bfloat16
+    assert ((y16.float() - y32).abs() <= 2e-2 + 1e-2 * y32.abs()).all()
+    x2 = x.clone()
+    x2[:, 40:] += 1.0
+    y16b = m16(x2, selection_override=sel)
+    assert torch.equal(y16[:, :40], y16b[:, :40])

@@ -36,3 +36,13 @@ def assert_close(got, want, atol, rtol, what=""):
         raise AssertionError(f"{what}: {int(bad.sum())}/{bad.numel()} elements out of tolerance; "
                              f"max err {err.max().item():.4g} (ref max {want.abs().max().item():.4g}); first at {i}: "
                              f"got {got[tuple(i)].item():.6g} want {want[tuple(i)].item():.6g}")
+
+
+def assert_grad_close(got, want, what=""):
+    """Gradient bound used by the kernel tests: 5e-2 relative in the norm of the whole tensor (the stated bound), and per
+    element 5e-2 relative with an absolute floor of 2e-2 of the tensor's largest entry (a relative bound alone is
+    meaningless for the entries near zero)."""
+    g, w = got.float().cpu(), want.float().cpu()
+    e = ((g - w).norm() / w.norm().clamp_min(1e-12)).item()
+    assert e < 5e-2, f"{what}: relative error {e:.4f} (norm-wise) exceeds 5e-2"
+    assert_close(got, want, 2e-2 * w.abs().max().item() + 1e-6, 5e-2, what)
