@@ -168,6 +168,36 @@ int nsa_windows_fwd(const void* x, const int64_t* x_stride, const void* pos, int
 int nsa_windows_bwd(const void* d_windows, int32_t batch, int32_t heads, int32_t seq, int32_t dim_head, int32_t block,
                     int32_t stride, void* dx, void* stream);
 
+/* Epilogue of the fused qkv projection.  Replaces, in one pass over the projection's output, the head
+ * split (NSA.py:583-587), split_compress_window + the intra-window position add on k and v
+ * (NSA.py:589-603, 270-275) and the rotation of queries and keys (NSA.py:643); the backward replaces the
+ * backward kernels of all of these plus the gradient sums and the concatenation in front of to_qkv.
+ *   qkv     : [batch, seq, (heads + 2 kv_heads) * d] (q heads, then k heads, then v heads of a token;
+ *             element strides qkv_stride = {batch, token}), fp32 if `fp32` else bf16
+ *   freqs   : fp32 [d/2]; token i is rotated by (i + offset) * freqs[p] on feature pair (2p, 2p+1)
+ *   k_pos, v_pos : intra-window positions [kv_heads, block, d] in the dtype of qkv
+ *   rq, rk  : bf16 [batch, heads | kv_heads, seq, d] contiguous, rotated queries / keys
+ *   q16, v16: bf16 contiguous head-split copies of the un-rotated queries / the values, or NULL (a bf16
+ *             qkv is read in place by the attention kernels through strided views)
+ *   k_windows, v_windows : [batch, kv_heads, seq / stride, block, d] contiguous in the dtype of qkv, window w
+ *             = tokens (w+1)*stride - block .. (w+1)*stride - 1 (zeros left of token 0) + positions;
+ *             not touched when block == 0 or seq < stride
+ * nsa_qkv_prep_bwd: any of the six gradients (same layouts and dtypes as the outputs above) may be
+ * NULL (= zero); d_qkv [batch, seq, (heads + 2 kv_heads) * d] with strides qkv_stride, dtype of qkv.  The
+ * gradients of the positions (sums of the window gradients over batch and windows) are left to the caller.
+ * dim_head 64 or 128 (NSA_E_UNSUPPORTED otherwise). */
+typedef struct nsa_qkv_desc {
+  int32_t batch, seq, heads, kv_heads, dim_head;
+  int32_t block, stride;  /* compression window length and step (compress_block_size, compress_block_sliding_stride); block 0: no windows */
+  int32_t fp32;           /* 1: qkv, positions, windows and d_qkv are fp32; 0: bf16 */
+  int32_t offset;         /* rotary position of token 0 */
+  int64_t qkv_stride[2];
+} nsa_qkv_desc;
+int nsa_qkv_prep_fwd(const nsa_qkv_desc* d, const void* qkv, const float* freqs, const void* k_pos, const void* v_pos,
+                     void* q16, void* rq, void* rk, void* v16, void* k_windows, void* v_windows, void* stream);
+int nsa_qkv_prep_bwd(const nsa_qkv_desc* d, const void* d_q16, const void* d_rq, const void* d_rk, const void* d_v16,
+                     const void* d_k_windows, const void* d_v_windows, const float* freqs, void* d_qkv, void* stream);
+
 /* Single-token decode attention over cached keys / values.  Replaces the three attention
  * computations of SparseAttention.forward_inference (NSA.py:396-420 compressed, :446-515 selected
  * blocks + own block, :519-530 sliding window).

@@ -53,6 +53,14 @@ class DecodeStepDesc(C.Structure):
     ]
 
 
+class QkvDesc(C.Structure):
+    _fields_ = [
+        ("batch", C.c_int32), ("seq", C.c_int32), ("heads", C.c_int32), ("kv_heads", C.c_int32), ("dim_head", C.c_int32),
+        ("block", C.c_int32), ("stride", C.c_int32), ("fp32", C.c_int32), ("offset", C.c_int32),
+        ("qkv_stride", C.c_int64 * 2),
+    ]
+
+
 _ERR = {-1: "invalid argument", -2: "shape not supported by the compiled kernels", -3: "workspace too small"}
 
 
@@ -105,6 +113,9 @@ def lib():
         L.nsa_windows_fwd.argtypes = [vp, i3, vp] + [C.c_int32] * 6 + [vp, vp]
         L.nsa_windows_bwd.argtypes = [vp] + [C.c_int32] * 6 + [vp, vp]
         L.nsa_windows_fwd.restype = L.nsa_windows_bwd.restype = C.c_int
+        L.nsa_qkv_prep_fwd.argtypes = [C.POINTER(QkvDesc)] + [vp] * 11
+        L.nsa_qkv_prep_bwd.argtypes = [C.POINTER(QkvDesc)] + [vp] * 9
+        L.nsa_qkv_prep_fwd.restype = L.nsa_qkv_prep_bwd.restype = C.c_int
         for name in ("nsa_dense_workspace_bytes", "nsa_dense_fwd", "nsa_dense_bwd", "nsa_topk", "nsa_gate_fwd", "nsa_gate_bwd"):
             getattr(L, name).restype = C.c_int
         for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):

@@ -1026,3 +1026,85 @@ def decode_step(q: Tensor, k: Tensor, v: Tensor, freqs: Tensor, pos: int, keys: 
     idx = ws[ioff.value:ioff.value + b * units * kk * 4].view(torch.int32).view(b, units, 1, kk)
     fm = ws[foff.value:foff.value + b * units * kk].view(torch.bool).view(b, units, 1, kk)
     return out, idx, fm
+
+
+# ------------------------------------------------------------- epilogue of the qkv projection
+
+def qkv_prep_supported(qkv: Tensor, dim_head: int) -> bool:
+    """The fused epilogue runs on device projections in bf16 or fp32 with 64 or 128 features per head, outside a compiler
+    trace (it is a plain autograd.Function over the C ABI, not a registered operator)."""
+    return (qkv.is_cuda and qkv.dtype in (_BF16, torch.float32) and dim_head in (64, 128) and qkv.dim() == 3
+            and not torch.compiler.is_compiling())
+
+
+def _qkv_desc(qkv: Tensor, heads: int, kv_heads: int, d: int, block: int, stride: int, offset: int) -> _lib.QkvDesc:
+    dsc = _lib.QkvDesc()
+    dsc.batch, dsc.seq, dsc.heads, dsc.kv_heads, dsc.dim_head = qkv.shape[0], qkv.shape[1], heads, kv_heads, d
+    dsc.block, dsc.stride, dsc.fp32, dsc.offset = block, stride, int(qkv.dtype == torch.float32), offset
+    dsc.qkv_stride[:] = (qkv.stride(0), qkv.stride(1))
+    return dsc
+
+
+class _QkvPrep(torch.autograd.Function):
+    """One kernel over the qkv projection's output in each direction (see nsa_qkv_prep_fwd in include/nsa_hip.h)."""
+
+    @staticmethod
+    def forward(ctx, qkv, freqs, kpos, vpos, heads, kv_heads, d, block, stride, offset):
+        b, n, width = qkv.shape
+        if width != (heads + 2 * kv_heads) * d:
+            raise RuntimeError(f"qkv projection of width {width}: expected (heads + 2 kv_heads) * dim_head = {(heads + 2 * kv_heads) * d}")
+        if qkv.stride(2) != 1 or qkv.stride(1) % 8 or qkv.stride(0) % 8 or qkv.data_ptr() % 16:
+            qkv = qkv.contiguous()
+        fp32 = qkv.dtype == torch.float32
+        dev = qkv.device
+        freqs32 = freqs.detach().to(torch.float32).contiguous()
+        w = n // stride if block > 0 else 0
+        rq = torch.empty((b, heads, n, d), dtype=_BF16, device=dev)
+        rk = torch.empty((b, kv_heads, n, d), dtype=_BF16, device=dev)
+        kw = torch.empty((b, kv_heads, w, block, d), dtype=qkv.dtype, device=dev)
+        vw = torch.empty_like(kw)
+        if fp32:
+            q16 = torch.empty((b, heads, n, d), dtype=_BF16, device=dev)
+            v16 = torch.empty((b, kv_heads, n, d), dtype=_BF16, device=dev)
+        else:
+            # a bf16 projection is read in place: 'b n (h d) -> b h n d' views
+            q16 = qkv[..., :heads * d].view(b, n, heads, d).permute(0, 2, 1, 3)
+            v16 = qkv[..., (heads + kv_heads) * d:].view(b, n, kv_heads, d).permute(0, 2, 1, 3)
+        kp = kpos.detach().to(qkv.dtype).contiguous() if w > 0 else None
+        vp = vpos.detach().to(qkv.dtype).contiguous() if w > 0 else None
+        dsc = _qkv_desc(qkv, heads, kv_heads, d, block, stride, offset)
+        _lib.check(_lib.lib().nsa_qkv_prep_fwd(C.byref(dsc), _ptr(qkv), _ptr(freqs32), _ptr(kp), _ptr(vp), _ptr(q16) if fp32 else None,
+                                               _ptr(rq), _ptr(rk), _ptr(v16) if fp32 else None, _ptr(kw) if w > 0 else None,
+                                               _ptr(vw) if w > 0 else None, _stream()), "nsa_qkv_prep_fwd")
+        ctx.save_for_backward(freqs32)
+        ctx.meta = (tuple(qkv.shape), qkv.dtype, heads, kv_heads, d, block, stride, offset, kpos.dtype, vpos.dtype,
+                    ctx.needs_input_grad[2], ctx.needs_input_grad[3])
+        ctx.set_materialize_grads(False)
+        return q16, rq, rk, v16, kw, vw
+
+    @staticmethod
+    def backward(ctx, dq16, drq, drk, dv16, dkw, dvw):
+        (freqs32,) = ctx.saved_tensors
+        shape, dtype, heads, kv_heads, d, block, stride, offset, kp_dtype, vp_dtype, kp_grad, vp_grad = ctx.meta
+        b, n, _ = shape
+        c16 = lambda t: None if t is None else (t if t.dtype == _BF16 else t.to(_BF16)).contiguous()
+        cw = lambda t: None if t is None or t.numel() == 0 else (t if t.dtype == dtype else t.to(dtype)).contiguous()
+        dq16, drq, drk, dv16, dkw, dvw = c16(dq16), c16(drq), c16(drk), c16(dv16), cw(dkw), cw(dvw)
+        dqkv = torch.empty(shape, dtype=dtype, device=freqs32.device)
+        dsc = _qkv_desc(dqkv, heads, kv_heads, d, block, stride, offset)
+        _lib.check(_lib.lib().nsa_qkv_prep_bwd(C.byref(dsc), _ptr(dq16), _ptr(drq), _ptr(drk), _ptr(dv16), _ptr(dkw), _ptr(dvw),
+                                               _ptr(freqs32), _ptr(dqkv), _stream()), "nsa_qkv_prep_bwd")
+        dkp = dkw.sum(dim=(0, 2), dtype=torch.float32).to(kp_dtype) if kp_grad and dkw is not None else None
+        dvp = dvw.sum(dim=(0, 2), dtype=torch.float32).to(vp_dtype) if vp_grad and dvw is not None else None
+        return dqkv, None, dkp, dvp, None, None, None, None, None, None
+
+
+def qkv_prep(qkv: Tensor, freqs: Tensor, k_positions: Tensor, v_positions: Tensor, heads: int, kv_heads: int, dim_head: int,
+             compress_block_size: int, compress_stride: int, offset: int = 0):
+    """Everything the attention branches read, from the fused projection 'b n ((heads + 2 kv_heads) d)' in one pass
+    (NSA.py:583-614, 643): returns (q, rotated q, rotated k, v) as bf16 'b h n d' and the compression windows of k and v
+    'b h w cbs d' (+ intra-window positions) in the projection's dtype.  For a bf16 projection q and v are views of it."""
+    if not qkv_prep_supported(qkv, dim_head):
+        raise RuntimeError("qkv_prep: needs a bf16 / fp32 device projection 'b n (h d)' with dim_head 64 or 128")
+    return _QkvPrep.apply(qkv, freqs, k_positions, v_positions, int(heads), int(kv_heads), int(dim_head), int(compress_block_size),
+                          int(compress_stride), int(offset))

@@ -245,14 +245,22 @@ class SparseAttention(nn.Module):
         bf16 = torch.bfloat16
 
         x = self.norm(inp)
-        q, k, v = self.to_qkv(x).split(self.qkv_split, dim=-1)
-        q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
+        qkv = self.to_qkv(x)
+        q, k, v = qkv.split(self.qkv_split, dim=-1)
+        q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)      # views; read below only by the unfused path and the caches
 
         # compressed keys / values from the un-rotated k, v
         L = (n // st) * st
-        # window gather + intra-window positions in one HIP kernel per tensor (NSA.py:589-603)
-        kw, vw = ops.compress_windows_pair(k.to(bf16), v.to(bf16), self.k_intrablock_positions, self.v_intrablock_positions, cbs, st)
-        kw, vw = kw.to(k.dtype), vw.to(v.dtype)
+        fused = ops.qkv_prep_supported(qkv, self.dim_head)
+        if fused:
+            # head split, rotation of q / k (NSA.py:643), window gather + intra-window positions (NSA.py:589-603) and the
+            # bf16 casts as one pass over the projection's output; its backward writes the projection's gradient directly
+            q16, rq16, rk16, v16, kw, vw = ops.qkv_prep(qkv, self.rotary_emb.freqs, self.k_intrablock_positions, self.v_intrablock_positions,
+                                                        self.heads, self.kv_heads, self.dim_head, cbs, st)
+        else:
+            # window gather + intra-window positions in one HIP kernel per tensor (NSA.py:589-603)
+            kw, vw = ops.compress_windows_pair(k.to(bf16), v.to(bf16), self.k_intrablock_positions, self.v_intrablock_positions, cbs, st)
+            kw, vw = kw.to(k.dtype), vw.to(v.dtype)
         ck0, cv0 = self.k_compress(kw), self.v_compress(vw)
         mem_k, mem_v = self.compress_mem_kv[0].to(ck0.dtype), self.compress_mem_kv[1].to(cv0.dtype)
         ck = torch.cat((mem_k[None].expand(b, -1, -1, -1), ck0), dim=-2)
@@ -261,12 +269,13 @@ class SparseAttention(nn.Module):
 
         want_sel = self.num_selected_blocks > 0 and nc > 0
         share = self.query_heads_share_selected_kv
-        c_out, imp = ops.compress_attend(q.to(bf16), ck.to(bf16), cv.to(bf16), M, st, self.causal,
+        c_out, imp = ops.compress_attend(q16 if fused else q.to(bf16), ck.to(bf16), cv.to(bf16), M, st, self.causal,
                                          sel_block=B if want_sel else None, share=share)
 
-        # rotary positions for the selection and sliding branches (NSA.py:643), one HIP kernel each
-        rq16, rk16 = ops.rotary_pair(q.to(bf16), k.to(bf16), self.rotary_emb.freqs)
-        v16 = v.to(bf16)
+        if not fused:
+            # rotary positions for the selection and sliding branches (NSA.py:643), one HIP kernel each
+            rq16, rk16 = ops.rotary_pair(q.to(bf16), k.to(bf16), self.rotary_emb.freqs)
+            v16 = v.to(bf16)
 
         num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
         if num_sel > 0:

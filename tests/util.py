@@ -43,6 +43,9 @@ def assert_grad_close(got, want, what=""):
     element 5e-2 relative with an absolute floor of 2e-2 of the tensor's largest entry (a relative bound alone is
     meaningless for the entries near zero)."""
     g, w = got.float().cpu(), want.float().cpu()
-    e = ((g - w).norm() / w.norm().clamp_min(1e-12)).item()
-    assert e < 5e-2, f"{what}: relative error {e:.4f} (norm-wise) exceeds 5e-2"
+    # a gradient that is zero in exact arithmetic (one visible key: softmax = 1) comes out as rounding noise; 1e-6 per
+    # element is the absolute floor below which the relative figure means nothing
+    err, floor = (g - w).norm().item(), 1e-6 * w.numel() ** 0.5
+    e = err / max(w.norm().item(), 1e-12)
+    assert e < 5e-2 or err <= floor, f"{what}: relative error {e:.4f} (norm-wise) exceeds 5e-2"
     assert_close(got, want, 2e-2 * w.abs().max().item() + 1e-6, 5e-2, what)
