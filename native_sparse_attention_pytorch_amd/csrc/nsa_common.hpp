@@ -99,6 +99,39 @@ __device__ __forceinline__ bf16x8 lds_row_operand(const __bf16* tile_s, int RS, 
   return *reinterpret_cast<const bf16x8*>(tile_s + (lane & 31) * RS + 16 * ks + 8 * (lane >> 5));
 }
 
+// Swizzled row-major LDS tile (D = 64 or 128 bf16 per row, no padding) for tiles that are read both ways: the 16-byte
+// chunk c of row r is stored at chunk position (c & ~7) | ((c ^ swz(r)) & 7), swz(r) = 2 * (r % 4) + (r / 4) % 2.
+// Eight consecutive rows then put the same chunk into eight different bank groups (16-byte row reads, eight lanes per
+// clock: no conflicts), and four consecutive rows put a pair of adjacent chunks into four disjoint pairs (the transpose
+// load, a 16-lane group reading 4 rows x 32 bytes per clock: no conflicts).  A plain padded stride can give one or the
+// other.  swz depends on the lane only (not on the k-step or the feature tile), so a kernel pays a few address registers.
+__device__ __forceinline__ int lds_swz(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
+
+template <int D>
+__device__ __forceinline__ int lds_swz_off(int row, int chunk) {
+  return row * D + 8 * ((chunk & ~7) | ((chunk ^ lds_swz(row)) & 7));
+}
+
+template <int D>
+__device__ __forceinline__ bf16x8 lds_row_operand_swz(const __bf16* tile_s, int ks, int lane) {
+  return *reinterpret_cast<const bf16x8*>(tile_s + lds_swz_off<D>(lane & 31, 2 * ks + (lane >> 5)));
+}
+
+// as lds_transposed_operand, from a swizzled tile; row0 must be a multiple of 8 and col0 of 16
+template <int D>
+__device__ __forceinline__ bf16x8 lds_transposed_operand_swz(const __bf16* X, int row0, int col0, int lane) {
+  const int ll = lane & 15, e = ll >> 2, qq = ll & 3, mh = (lane >> 4) & 1, h = lane >> 5;
+  const __bf16* p0 = X + lds_swz_off<D>(row0 + 4 * h + e, (col0 >> 3) + 2 * mh + (qq >> 1)) + 4 * (qq & 1);
+  typedef shortx4 __attribute__((address_space(3))) * lds_ptr;
+  const shortx4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
+  const shortx4 b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + 8 * D));      // rows + 8: same swizzle
+  typedef __attribute__((__vector_size__(8 * sizeof(short)))) short shortx8;
+  shortx8 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { r[i] = a[i]; r[4 + i] = b[i]; }
+  return __builtin_bit_cast(bf16x8, r);
+}
+
 // s_waitcnt vmcnt(0) (expcnt / lgkmcnt left at their maxima): all outstanding global loads
 // and stores of this wave have completed.
 // N operand reads feeding N uses, each read issued AH uses ahead of its own.  The compiler keeps an LDS operand
