@@ -29,10 +29,25 @@ HBM_PEAK_GBS = 8000.0
 
 CFG = dict(batch=1, seq=32768, heads=32, kv_heads=8, dim_head=128, block=64, num_sel=15)
 
-# HBM bytes per launch on this workload, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
-# scaled by streaming kernels of known size (profiles/select_fwd_bwd_seq32k_hbm_traffic.txt)
-MEASURED_TRAFFIC_BYTES = {"fwd_block_walk": 6.405e9, "fwd_merge": 4.851e9, "bwd_dq_merge": 4.546e9,
-                          "bwd_dkv_walk": 13.398e9, "bwd_dkv_reduce": 0.547e9, "bwd_delta": 0.541e9}
+# HBM bytes per launch on this workload come from the tracked rocprofv3 summary (FETCH_SIZE / WRITE_SIZE per dispatch,
+# scaled by streaming kernels of known size; the file states the commands), not from literals kept here
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "select_fwd_bwd_seq32k_hbm_traffic.txt")
+TRAFFIC_KERNELS = {"sel_fwd_kernel": "fwd_block_walk", "sel_fwd_combine_kernel": "fwd_merge", "sel_bwd_dq_combine_kernel": "bwd_dq_merge",
+                   "sel_bwd_dkv_kernel": "bwd_dkv_walk", "sel_bwd_dkv_reduce_kernel": "bwd_dkv_reduce", "sel_delta_kernel": "bwd_delta"}
+
+
+def measured_traffic_bytes():
+    """{bench kernel name: HBM bytes per launch} from the summary's table (columns: kernel, raw counters, fetch_GB, write_GB,
+    total_GB); empty when the file is missing."""
+    out = {}
+    try:
+        for line in open(TRAFFIC_SUMMARY):
+            f = line.split()
+            if len(f) == 6 and f[0] in TRAFFIC_KERNELS:
+                out[TRAFFIC_KERNELS[f[0]]] = float(f[5]) * 1e9
+    except OSError:
+        pass
+    return out
 
 
 def selection(b, h, n, B, S, seed, device):
@@ -78,22 +93,22 @@ class HipEvents:
         return out.value
 
 
-def cpu_baseline(cfg, q, k, v, do, idx, msk, nq=8192):
-    """The CPU oracle (fp32 restatement of the reference's pure-torch path) on a bounded sample:
+def cpu_baseline(cfg, q, k, v, do, idx, msk, nq=8192, dtype=torch.float32):
+    """The CPU oracle (restatement of the reference's pure-torch path, in `dtype`) on a bounded sample:
     the last `nq` queries of the same workload against the full-length K/V, forward+backward."""
     from oracle import nsa_oracle as O
     n = cfg["seq"]
     sl = slice(n - nq, n)
-    qc = q[:, :, sl].float().cpu().requires_grad_()
-    kc, vc = k.float().cpu().requires_grad_(), v.float().cpu().requires_grad_()
-    doc = do[:, :, sl].float().cpu()
+    qc = q[:, :, sl].to(dtype).cpu().requires_grad_()
+    kc, vc = k.to(dtype).cpu().requires_grad_(), v.to(dtype).cpu().requires_grad_()
+    doc = do[:, :, sl].to(dtype).cpu()
     ic, mc = idx[:, :, sl].cpu(), msk[:, :, sl].cpu()
     t0 = time.perf_counter()
     out = O.select_attend(qc, kc, vc, ic, mc, cfg["block"], causal=True, q_offset=n - nq, chunk=128)
     (out * doc).sum().backward()
     dt = time.perf_counter() - t0
     return dict(value=nq * cfg["batch"] / dt, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
-                sample=f"last {nq} of {n} queries (each attends 16 blocks), full-length K/V, fp32 fwd+bwd, {dt:.1f} s; "
+                sample=f"last {nq} of {n} queries (each attends 16 blocks), full-length K/V, {str(dtype).split('.')[-1]} fwd+bwd, {dt:.1f} s; "
                        f"host has {os.cpu_count()} logical CPUs"), out.detach()
 
 
@@ -186,13 +201,15 @@ def main():
     kflop = {"fwd_block_walk": 2 * flop_unit, "bwd_dkv_walk": 5 * flop_unit}
     dom = max(kflop, key=lambda nm: kern[nm])
     achieved = kflop[dom] / (kern[dom] * 1e-3) / 1e12
-    traffic = MEASURED_TRAFFIC_BYTES.get(dom)
+    traffic_all = measured_traffic_bytes()
+    traffic = traffic_all.get(dom)
     roofline = dict(bound="mfma", kernel=dom, achieved=round(achieved, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
                     frac=round(achieved / MFMA_PEAK_TFLOPS, 4), traffic=traffic,
                     step_frac=round(value / MFMA_PEAK_TFLOPS, 4),
                     # the kernels are HBM-bound in practice: measured bytes / measured time against 8 TB/s
-                    hbm_GBs={nm: round(MEASURED_TRAFFIC_BYTES[nm] / (kern[nm] * 1e-3) / 1e9, 1) for nm in MEASURED_TRAFFIC_BYTES},
-                    hbm_frac_step=round(sum(MEASURED_TRAFFIC_BYTES.values()) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4))
+                    hbm_GBs={nm: round(traffic_all[nm] / (kern[nm] * 1e-3) / 1e9, 1) for nm in traffic_all},
+                    hbm_frac_step=round(sum(traffic_all.values()) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if traffic_all else None,
+                    traffic_source=os.path.relpath(TRAFFIC_SUMMARY, ROOT))
 
     res = dict(metric="NSA selection-attention fwd+bwd TFLOP/s at seq 32k (bf16)", value=round(value, 2), unit="TFLOP/s",
                n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_step, 4), higher_is_better=True,
@@ -225,8 +242,18 @@ def main():
             tms.append((e0.elapsed_time(e1), e1.elapsed_time(e2), e2.elapsed_time(e3)))
         p_cmp = b * hq * sum(i // 16 + 1 for i in range(n))
         best = min(tms[1:], key=sum)
+        cf, cb = 4 * d * p_cmp / (best[0] * 1e-3) / 1e12, 10 * d * p_cmp / (best[2] * 1e-3) / 1e12
         res["compressed_branch"] = dict(fwd_with_importance_ms=round(best[0], 4), topk_ms=round(best[1], 4), bwd_ms=round(best[2], 4),
-                                        attended_pairs=p_cmp, fwd_bwd_tflops=round(14 * d * p_cmp / (sum(best) * 1e-3) / 1e12, 2))
+                                        attended_pairs=p_cmp, fwd_bwd_tflops=round(14 * d * p_cmp / (sum(best) * 1e-3) / 1e12, 2),
+                                        # its own roofline: algorithmic 4dP forward (with the importance logits) / 10dP backward
+                                        # (delta + dQ + dK/dV + reduce kernels together) over the HIP-event time of each call
+                                        roofline=dict(bound="mfma", peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                                                      fwd=dict(kernel="dense_fwd_kernel<128,4>", achieved=round(cf, 2), frac=round(cf / MFMA_PEAK_TFLOPS, 4)),
+                                                      bwd=dict(kernel="dense_bwd_dq_kernel<128> + dense_bwd_dkv_pipe_kernel<128>", achieved=round(cb, 2),
+                                                               frac=round(cb / MFMA_PEAK_TFLOPS, 4)),
+                                                      topk=dict(bound="hbm", bytes=int(imp.numel() * 4 + idx_.numel() * 9),
+                                                                achieved_GBs=round((imp.numel() * 4 + idx_.numel() * 9) / (best[1] * 1e-3) / 1e9, 1),
+                                                                peak_GBs=HBM_PEAK_GBS)))
     except _Skip:
         pass
     except Exception as ex:  # the headline must still be printed
@@ -370,6 +397,9 @@ def main():
         torch.set_num_threads(min(16, os.cpu_count() or 1))
         base, ref = cpu_baseline(cfg, q, k, v, do, idx, msk)
         res["cpu_baseline"] = base
+        # the same path with the module cast to bf16, as the reference's torch path runs then (smaller sample: bf16 CPU GEMMs are slow)
+        base16, _ = cpu_baseline(cfg, q, k, v, do, idx, msk, nq=1024, dtype=torch.bfloat16)
+        res["cpu_baseline_bf16"] = base16
         err = (out[:, :, n - ref.shape[2]:].float().cpu() - ref).abs().max().item()
         res["config"]["max_abs_err_vs_oracle_sample"] = round(err, 5)
         res["config"]["gpu_over_cpu"] = round(res["config"]["tokens_per_s"] / base["value"], 1)

@@ -189,7 +189,8 @@ int nsa_windows_bwd(const void* d_windows, int32_t batch, int32_t heads, int32_t
 typedef struct nsa_qkv_desc {
   int32_t batch, seq, heads, kv_heads, dim_head;
   int32_t block, stride;  /* compression window length and step (compress_block_size, compress_block_sliding_stride); block 0: no windows */
-  int32_t fp32;           /* 1: qkv, positions, windows and d_qkv are fp32; 0: bf16 */
+  int32_t fp32;           /* 1: qkv, positions, windows and d_qkv are fp32; 0: bf16; 2 (forward only): as 1, and rq / rk are
+                             written as fp32 too, q16 / v16 are not written (inputs of the fp32 forward kernels below) */
   int32_t offset;         /* rotary position of token 0 */
   int64_t qkv_stride[2];
 } nsa_qkv_desc;
@@ -197,6 +198,22 @@ int nsa_qkv_prep_fwd(const nsa_qkv_desc* d, const void* qkv, const float* freqs,
                      void* q16, void* rq, void* rk, void* v16, void* k_windows, void* v_windows, void* stream);
 int nsa_qkv_prep_bwd(const nsa_qkv_desc* d, const void* d_q16, const void* d_rq, const void* d_rk, const void* d_v16,
                      const void* d_k_windows, const void* d_v_windows, const float* freqs, void* d_qkv, void* stream);
+
+/* fp32 forward of the attention branches, for fp32 modules run for inference: products, softmax and
+ * accumulation in fp32 on the vector ALUs, so that the result agrees with the reference's fp32 torch path
+ * to its own test tolerance (1e-5, tests/test_sparse_attn.py:86), which the bf16 MFMA kernels cannot.
+ * Same contracts and descriptors as nsa_dense_fwd (without the importance logits, which are linear in q and
+ * the compressed keys and cost one small fp32 GEMM) and nsa_select_fwd (no workspaces, no inverse index);
+ * q, k, v: fp32 with element strides {batch, head, token}, key / value rows 16-byte aligned; out: fp32
+ * contiguous [batch, heads, seq, d]; lse: fp32 [batch, heads, seq] or NULL.  `seq` of the descriptor is the number
+ * of query rows; query row i sits at sequence position i + q_offset (0 for the parallel forward; the cached length
+ * for a decode step with seq = 1, NSA.py:338-547), and k / v hold num_mem + num_keys rows (dense) or num_keys rows
+ * (selection; idx / fmask are [batch, kv_heads, seq, num_sel]).  Any dim_head <= 128 that is a multiple of 4,
+ * any group size, any block size; no backward. */
+int nsa_dense_fwd_f32(const nsa_dense_desc* d, const float* q, const float* k, const float* v, float* out, float* lse,
+                      int32_t q_offset, void* stream);
+int nsa_select_fwd_f32(const nsa_select_desc* d, const float* q, const float* k, const float* v, const void* idx,
+                       const uint8_t* fmask, float* out, float* lse, int32_t num_keys, int32_t q_offset, void* stream);
 
 /* Single-token decode attention over cached keys / values.  Replaces the three attention
  * computations of SparseAttention.forward_inference (NSA.py:396-420 compressed, :446-515 selected

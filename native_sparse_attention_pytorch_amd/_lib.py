@@ -116,6 +116,9 @@ def lib():
         L.nsa_qkv_prep_fwd.argtypes = [C.POINTER(QkvDesc)] + [vp] * 11
         L.nsa_qkv_prep_bwd.argtypes = [C.POINTER(QkvDesc)] + [vp] * 9
         L.nsa_qkv_prep_fwd.restype = L.nsa_qkv_prep_bwd.restype = C.c_int
+        L.nsa_dense_fwd_f32.argtypes = [C.POINTER(DenseDesc)] + [vp] * 5 + [C.c_int32, vp]
+        L.nsa_select_fwd_f32.argtypes = [C.POINTER(SelectDesc)] + [vp] * 7 + [C.c_int32, C.c_int32, vp]
+        L.nsa_dense_fwd_f32.restype = L.nsa_select_fwd_f32.restype = C.c_int
         for name in ("nsa_dense_workspace_bytes", "nsa_dense_fwd", "nsa_dense_bwd", "nsa_topk", "nsa_gate_fwd", "nsa_gate_bwd"):
             getattr(L, name).restype = C.c_int
         for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):

@@ -635,9 +635,6 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
     }
 }
 
-#ifndef NSA_DKV_PIPE_B
-#define NSA_DKV_PIPE_B 1
-#endif
 #ifndef NSA_DKV_PIPE
 #define NSA_DKV_PIPE 1        // 1: the software-pipelined dK/dV kernel below, 0: the plain one above
 #endif
@@ -833,16 +830,6 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_pipe_kernel(const DensePlan
     accumulate(bc, Pf, Sf);
     commit(st, i0 + 2 * ppt, bnn);
     issue(st, i0 + 3 * ppt);
-#if NSA_DKV_PIPE_B
-#pragma unroll
-    for (int i = 0; i < 4 * DT; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);          // the transposed operand (two LDS reads)
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);          // its MFMA
-      __builtin_amdgcn_sched_group_barrier(0x200, i < NT ? 1 : 0, 0);      // first the commit's LDS writes ...
-      __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-      __builtin_amdgcn_sched_group_barrier(0x020, i >= 4 * DT - NT ? 1 : 0, 0);      // ... then the gathers of the tile after
-    }
-#endif
     __builtin_amdgcn_sched_barrier(0);
     bc = bn;
   };

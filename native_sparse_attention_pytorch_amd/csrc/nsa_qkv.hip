@@ -74,10 +74,10 @@ __device__ __forceinline__ void window_range(const QkvArgs& A, int tok, int& a, 
   w_lo = (a - A.cbs + 1 <= 0) ? 0 : (a - A.cbs + A.st) / A.st;       // ceil((a - cbs + 1) / st)
 }
 
-template <int D, typename T>
+template <int D, typename T, typename TR>
 __global__ __launch_bounds__(256) void qkv_prep_fwd_kernel(const QkvArgs A, const T* __restrict__ qkv, const float* __restrict__ freqs,
                                                            const T* __restrict__ kpos, const T* __restrict__ vpos,
-                                                           __bf16* __restrict__ q16, __bf16* __restrict__ rq, __bf16* __restrict__ rk,
+                                                           __bf16* __restrict__ q16, TR* __restrict__ rq, TR* __restrict__ rk,
                                                            __bf16* __restrict__ v16, T* __restrict__ kw, T* __restrict__ vw) {
   constexpr int CPR = D / 8, TPB = 256 / CPR;
   const int lead = A.cbs > 0 ? A.cbs - A.st : 0;
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void qkv_prep_fwd_kernel(const QkvArgs A, cons
       const long at = (((long)bb * A.hq + h) * A.n + tok) * D + 8 * c;
       if (q16 != nullptr) store_f8<__bf16>(q16 + at, x);
       rotate8(x, sn, cs, r);
-      store_f8<__bf16>(rq + at, r);
+      store_f8<TR>(rq + at, r);
     }
   }
   int a = 0, w_lo = 0, w_hi = -1;
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void qkv_prep_fwd_kernel(const QkvArgs A, cons
       const long at = (((long)bb * A.hk + h) * A.n + tok) * D + 8 * c;
       float r[8];
       rotate8(xk, sn, cs, r);
-      store_f8<__bf16>(rk + at, r);
+      store_f8<TR>(rk + at, r);
       if (v16 != nullptr) store_f8<__bf16>(v16 + at, xv);
     } else {
 #pragma unroll
@@ -230,13 +230,13 @@ static int qkv_args(const nsa_qkv_desc* d, QkvArgs& A) {
 
 using namespace nsa;
 
-template <int D, typename T>
+template <int D, typename T, typename TR = __bf16>
 static int qkv_fwd_launch(const QkvArgs& A, const void* qkv, const float* freqs, const void* kpos, const void* vpos, void* q16, void* rq,
                           void* rk, void* v16, void* kw, void* vw, hipStream_t st) {
   constexpr int TPB = 256 / (D / 8);
   const int lead = A.cbs > 0 ? A.cbs - A.st : 0;
-  hipLaunchKernelGGL((qkv_prep_fwd_kernel<D, T>), dim3((unsigned)((A.n + lead + TPB - 1) / TPB), A.b), dim3(256), 0, st, A, (const T*)qkv, freqs,
-                     (const T*)kpos, (const T*)vpos, (__bf16*)q16, (__bf16*)rq, (__bf16*)rk, (__bf16*)v16, (T*)kw, (T*)vw);
+  hipLaunchKernelGGL((qkv_prep_fwd_kernel<D, T, TR>), dim3((unsigned)((A.n + lead + TPB - 1) / TPB), A.b), dim3(256), 0, st, A, (const T*)qkv, freqs,
+                     (const T*)kpos, (const T*)vpos, (__bf16*)q16, (TR*)rq, (TR*)rk, (__bf16*)v16, (T*)kw, (T*)vw);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
 }
@@ -259,6 +259,10 @@ extern "C" int nsa_qkv_prep_fwd(const nsa_qkv_desc* d, const void* qkv, const fl
   if (!qkv || !freqs || !rq || !rk) return NSA_E_ARG;
   if (A.w > 0 && (!k_pos || !v_pos || !k_windows || !v_windows)) return NSA_E_ARG;
   hipStream_t st = (hipStream_t)stream;
+  if (d->fp32 == 2) {      // fp32 in, fp32 rotated outputs (the fp32 forward kernels read q and v from the projection itself)
+    if (d->dim_head == 64) return qkv_fwd_launch<64, float, float>(A, qkv, freqs, k_pos, v_pos, nullptr, rq, rk, nullptr, k_windows, v_windows, st);
+    return qkv_fwd_launch<128, float, float>(A, qkv, freqs, k_pos, v_pos, nullptr, rq, rk, nullptr, k_windows, v_windows, st);
+  }
   if (d->fp32) {
     if (d->dim_head == 64) return qkv_fwd_launch<64, float>(A, qkv, freqs, k_pos, v_pos, q16, rq, rk, v16, k_windows, v_windows, st);
     return qkv_fwd_launch<128, float>(A, qkv, freqs, k_pos, v_pos, q16, rq, rk, v16, k_windows, v_windows, st);

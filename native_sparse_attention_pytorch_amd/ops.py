@@ -207,6 +207,22 @@ def _split_blocks(idx: Tensor, fmask: Tensor, sel_scale: Tensor | None, block: i
     return idx_k.contiguous(), fm_k.contiguous(), sc_k, sub
 
 
+def _dead_rows_uniform(out: Tensor, fv: Tensor, selected_block_indices: Tensor, fmask: Tensor, block_size: int, q_heads: int, d: int) -> Tensor:
+    """A query whose slots are all dead attends nothing in the kernels.  The reference's torch path (NSA.py:809-815)
+    fills every logit of such a row with the same value, i.e. it attends uniformly over the keys of the (dead) slots'
+    blocks, zero padding included; reproduce that corner with a few elementwise ops (no sync, differentiable in v)."""
+    b, hs, n, S = selected_block_indices.shape
+    hk2 = fv.shape[1]
+    W = (n + block_size - 1) // block_size
+    vpad = torch.nn.functional.pad(fv, (0, 0, 0, W * block_size - n)).reshape(b, hk2, W, block_size, d)
+    vmean = vpad.float().mean(dim=3)                                                  # [b,hk,W,d]
+    gi = selected_block_indices.long().clamp(0, W - 1).reshape(b, hs, n * S, 1).expand(-1, -1, -1, d)
+    avg = vmean.gather(2, gi).reshape(b, hs, n, S, d).mean(dim=3)                     # [b,hk,n,d]
+    dead = ~fmask.bool().any(dim=-1)                                                  # [b,hk,n]
+    g = q_heads // hs
+    return torch.where(dead.repeat_interleave(g, dim=1)[..., None], avg.repeat_interleave(g, dim=1).to(out.dtype), out)
+
+
 def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, selected_block_indices: Tensor, fmask: Tensor,
                          sel_scale: Tensor | None = None, include_block_causal: bool = True, return_lse: bool = False,
                          block_dk_dv_use_dot=None, return_sliding_window_out: bool = False):
@@ -255,20 +271,7 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
     out, lse = _unpad_groups(out, fk.shape[1], g0, gp0)[:, :, :n, :d_head], _unpad_groups(lse, fk.shape[1], g0, gp0)[:, :, :n]
     fv = fv_given if kv_heads == sel_heads else fv_given.repeat_interleave(q_heads // kv_heads, dim=1)
     if not include_block_causal and selected_block_indices.shape[-1] > 0:
-        # A query whose slots are all dead attends nothing in the kernel.  The reference's torch
-        # path (NSA.py:809-815) fills every logit of such a row with the same value, i.e. it
-        # attends uniformly over the keys of the (dead) slots' blocks, zero padding included;
-        # reproduce that corner with a few elementwise ops (no sync, differentiable in v).
-        b, hs, n, S = selected_block_indices.shape
-        hk2, d = fk.shape[1], d_head
-        W = (n + block_size - 1) // block_size
-        vpad = torch.nn.functional.pad(fv, (0, 0, 0, W * block_size - n)).reshape(b, hk2, W, block_size, d)
-        vmean = vpad.float().mean(dim=3)                                                  # [b,hk,W,d]
-        gi = selected_block_indices.long().clamp(0, W - 1).reshape(b, hs, n * S, 1).expand(-1, -1, -1, d)
-        avg = vmean.gather(2, gi).reshape(b, hs, n, S, d).mean(dim=3)                     # [b,hk,n,d]
-        dead = ~fmask.bool().any(dim=-1)                                                  # [b,hk,n]
-        g = q_heads // hs
-        out = torch.where(dead.repeat_interleave(g, dim=1)[..., None], avg.repeat_interleave(g, dim=1).to(out.dtype), out)
+        out = _dead_rows_uniform(out, fv, selected_block_indices, fmask, block_size, q_heads, d_head)
     out = out.to(dtype)
     if return_sliding_window_out:
         out, lse = (out, sliding_out), (lse, sliding_lse)
@@ -1108,3 +1111,119 @@ def qkv_prep(qkv: Tensor, freqs: Tensor, k_positions: Tensor, v_positions: Tenso
         raise RuntimeError("qkv_prep: needs a bf16 / fp32 device projection 'b n (h d)' with dim_head 64 or 128")
     return _QkvPrep.apply(qkv, freqs, k_positions, v_positions, int(heads), int(kv_heads), int(dim_head), int(compress_block_size),
                           int(compress_stride), int(offset))
+
+
+# ------------------------------------------------------------------ fp32 forward (inference)
+
+def _f32(t: Tensor) -> Tensor:
+    if t.dtype != torch.float32 or not t.is_cuda:
+        raise RuntimeError("the fp32 forward kernels take fp32 device tensors")
+    ok = t.stride(-1) == 1 and all(st % 4 == 0 for st in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+    return t if ok else t.contiguous()
+
+
+def _check_f32_dim(d: int):
+    if d > 128 or d % 4:
+        raise RuntimeError(f"dim_head {d}: the fp32 forward kernels take head dimensions <= 128 that are multiples of 4")
+
+
+@torch.no_grad()
+def dense_attend_f32(q: Tensor, k: Tensor, v: Tensor, mode: int, causal: bool, window: int = 0, stride: int = 1, num_mem: int = 0,
+                     q_offset: int = 0):
+    """Sliding-window (mode 0) or compressed (mode 1: k / v = [memory rows; compressed keys]) attention evaluated in fp32
+    (NSA.py:841-850 / 621-639).  q 'b hq n d', k / v 'b hk rows d', any group size; query row i sits at position
+    i + q_offset (a decode step: one row at the cached length).  Returns (out 'b hq n d', lse)."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    b, hq, n, d = q.shape
+    _check_f32_dim(d)
+    out = torch.empty((b, hq, n, d), dtype=torch.float32, device=q.device)
+    lse = torch.empty((b, hq, n), dtype=torch.float32, device=q.device)
+    dsc = _dense_desc(q, k, v, out, out, int(mode), bool(causal), int(window), int(stride), int(num_mem), False, 1, True, float(d ** -0.5))
+    _lib.check(_lib.lib().nsa_dense_fwd_f32(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), int(q_offset), _stream()),
+               "nsa_dense_fwd_f32")
+    return out, lse
+
+
+@torch.no_grad()
+def native_sparse_attend_f32(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, selected_block_indices: Tensor, fmask: Tensor,
+                             include_block_causal: bool = True, return_lse: bool = False, q_offset: int = 0):
+    """`native_sparse_attend` evaluated in fp32 (forward only): same arguments and contract (TRI.py:1938-1987, NSA.py:741-819),
+    any block size, any group size.  fq may hold fewer rows than fk / fv: row i is the query at position i + q_offset."""
+    q_heads, kv_heads, sel_heads = fq.shape[1], fk.shape[1], selected_block_indices.shape[1]
+    assert q_heads % kv_heads == 0 and sel_heads in (q_heads, kv_heads)
+    d = fq.shape[-1]
+    _check_f32_dim(d)
+    if kv_heads != sel_heads:
+        fk, fv = fk.repeat_interleave(q_heads // kv_heads, dim=1), fv.repeat_interleave(q_heads // kv_heads, dim=1)
+    q, k, v = _f32(fq), _f32(fk), _f32(fv)
+    b, hq, n, _ = q.shape
+    idx = selected_block_indices.contiguous()
+    if idx.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError("selected_block_indices must be int64 or int32")
+    fm = fmask.contiguous().view(torch.uint8) if fmask.dtype == torch.bool else fmask.contiguous().to(torch.uint8)
+    out = torch.empty((b, hq, n, d), dtype=torch.float32, device=q.device)
+    lse = torch.empty((b, hq, n), dtype=torch.float32, device=q.device)
+    dsc = _select_desc(q, k, v, out, idx.shape[-1], int(block_size), bool(include_block_causal), float(d ** -0.5), idx.dtype == torch.int64)
+    _lib.check(_lib.lib().nsa_select_fwd_f32(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(idx) if idx.numel() else None,
+                                             _ptr(fm) if fm.numel() else None, _ptr(out), _ptr(lse), k.shape[2], int(q_offset), _stream()),
+               "nsa_select_fwd_f32")
+    if not include_block_causal and idx.shape[-1] > 0 and q_offset == 0 and k.shape[2] == n:
+        out = _dead_rows_uniform(out, fv, selected_block_indices, fmask, int(block_size), q_heads, d)
+    return (out, lse) if return_lse else out
+
+
+@torch.no_grad()
+def importance_logits_f32(q: Tensor, ck: Tensor, stride: int, sel_block: int, share: bool, causal: bool, mask_own: bool = True):
+    """Block-importance logits of NSA.py:652-691 in fp32.  They are the mean, over a fine block's compressed keys and (if
+    shared) the group's heads, of scale * q . ck - linear in both, so one fp32 GEMM against the block means of the
+    compressed keys `ck` 'b hk nc d' (memory slots excluded); -inf where the reference's fill values remove the block from
+    the softmax (a block not entirely before the query; the query's own block when stride != sel_block).  None when no
+    full fine block exists."""
+    b, hq, n, d = q.shape
+    hk = ck.shape[1]
+    g = hq // hk
+    npf = sel_block // stride
+    nb = ck.shape[2] // npf
+    if nb == 0:
+        return None
+    cbar = ck[:, :, :nb * npf].float().reshape(b, hk, nb, npf, d).mean(dim=3)
+    qq = q.float().reshape(b, hk, g, n, d).mean(dim=2) if share else q.float()
+    if not share:
+        cbar = cbar.repeat_interleave(g, dim=1)
+    imp = torch.matmul(qq, cbar.transpose(-1, -2)) * (d ** -0.5)
+    i = torch.arange(n, device=q.device)[:, None]
+    j = torch.arange(nb, device=q.device)[None, :]
+    dead = torch.zeros((n, nb), dtype=torch.bool, device=q.device)
+    if causal:
+        dead |= (j + 1) * sel_block > i
+    if stride != sel_block and mask_own:      # decode steps (mask_own False): every cached block lies before the query
+        dead |= (i // sel_block) == j
+    return imp.masked_fill(dead, float("-inf"))
+
+
+@torch.no_grad()
+def qkv_prep_f32(qkv: Tensor, freqs: Tensor, k_positions: Tensor, v_positions: Tensor, heads: int, kv_heads: int, dim_head: int,
+                 compress_block_size: int, compress_stride: int, offset: int = 0):
+    """`qkv_prep` for the fp32 forward: (q, rotated q, rotated k, v, k windows, v windows), all fp32; q and v are views of
+    the projection.  dim_head 64 or 128."""
+    if qkv.dtype != torch.float32 or dim_head not in (64, 128) or not qkv.is_cuda:
+        raise RuntimeError("qkv_prep_f32: needs an fp32 device projection with dim_head 64 or 128")
+    b, n, width = qkv.shape
+    heads, kv_heads, d, block, stride = int(heads), int(kv_heads), int(dim_head), int(compress_block_size), int(compress_stride)
+    if qkv.stride(2) != 1 or qkv.stride(1) % 8 or qkv.stride(0) % 8 or qkv.data_ptr() % 16:
+        qkv = qkv.contiguous()
+    w = n // stride if block > 0 else 0
+    rq = torch.empty((b, heads, n, d), dtype=torch.float32, device=qkv.device)
+    rk = torch.empty((b, kv_heads, n, d), dtype=torch.float32, device=qkv.device)
+    kw = torch.empty((b, kv_heads, w, block, d), dtype=torch.float32, device=qkv.device)
+    vw = torch.empty_like(kw)
+    freqs32 = freqs.detach().to(torch.float32).contiguous()
+    kp = k_positions.detach().to(torch.float32).contiguous() if w > 0 else None
+    vp = v_positions.detach().to(torch.float32).contiguous() if w > 0 else None
+    dsc = _qkv_desc(qkv, heads, kv_heads, d, block, stride, int(offset))
+    dsc.fp32 = 2
+    _lib.check(_lib.lib().nsa_qkv_prep_fwd(C.byref(dsc), _ptr(qkv), _ptr(freqs32), _ptr(kp), _ptr(vp), None, _ptr(rq), _ptr(rk), None,
+                                           _ptr(kw) if w > 0 else None, _ptr(vw) if w > 0 else None, _stream()), "nsa_qkv_prep_fwd")
+    q = qkv[..., :heads * d].view(b, n, heads, d).permute(0, 2, 1, 3)
+    v = qkv[..., (heads + kv_heads) * d:].view(b, n, kv_heads, d).permute(0, 2, 1, 3)
+    return q, rq, rk, v, kw, vw

@@ -147,6 +147,9 @@ class SparseAttention(nn.Module):
             print('`num_selected_blocks` should be set greater than 0, unless if you are ablating it for experimental purposes')
         self.num_selected_blocks = num_selected_blocks
         self.use_triton_kernel = use_triton_kernel      # kept for call-site compatibility; the HIP kernels always run
+        # an fp32 module that is run without gradients takes the fp32 forward kernels (agreement with the reference's fp32
+        # path to 1e-5); with gradients, or with this switched off, its attention runs in bf16 like any other module's
+        self.fp32_inference_kernels = True
 
         if strategy_combine_mlp is None:
             strategy_combine_mlp = nn.Linear(dim, 3 * heads)
@@ -177,6 +180,9 @@ class SparseAttention(nn.Module):
         x = self.norm(inp)
         q, k, v = self.to_qkv(x).split(self.qkv_split, dim=-1)
         q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
+        if (self.fp32_inference_kernels and q.dtype == torch.float32 and self.dim_head <= 128 and self.dim_head % 4 == 0
+                and all(t.dtype == torch.float32 for t in (cache_k, cache_v, cache_ck, cache_cv, run_k, run_v))):
+            return self._forward_inference_fp32(x, q, k, v, cache, return_cache)
         # head dimensions other than the kernels' 64 / 128 run zero-padded: caches and window rows are then kept D wide
         # (the padding features stay zero), the projections and the compression network see the first d features
         d, D = self.dim_head, ops._kernel_dim(self.dim_head)
@@ -227,6 +233,112 @@ class SparseAttention(nn.Module):
             return out
         return out, ((keys, vals), ((ck, cv), (run_k, run_v)))
 
+    def _forward_inference_fp32(self, x, q, k, v, cache, return_cache):
+        """One decode step of an fp32 module over fp32 caches (as `_forward_fp32` hands them back), every attention branch
+        through the fp32 kernels: the reference's own criterion - token-by-token decoding equals the parallel forward to 1e-5
+        (tests/test_sparse_attn.py:50-91) - then holds for this module too.  Same steps as `forward_inference`."""
+        (cache_k, cache_v), ((cache_ck, cache_cv), (run_k, run_v)) = cache
+        b, t = x.shape[0], cache_k.shape[-2]
+        st, cbs, B = self.compress_block_sliding_stride, self.compress_block_size, self.selection_block_size
+        M, d, f32 = self.num_mem_compress_kv, self.dim_head, torch.float32
+        rq, rk = self.rotary_emb.rotate(q, offset=t), self.rotary_emb.rotate(k, offset=t)
+        run_k, rk_row = _append_rows(run_k, dtype=f32, min_capacity=cbs)
+        run_v, rv_row = _append_rows(run_v, dtype=f32, min_capacity=cbs)
+        rk_row.copy_(k)
+        rv_row.copy_(v)
+        keys, k_row = _append_rows(cache_k, dtype=f32)
+        vals, v_row = _append_rows(cache_v, dtype=f32)
+        k_row.copy_(rk)
+        v_row.copy_(v)
+
+        # compressed branch over every cached compressed key (NSA.py:396-420); none cached: the branch is zero
+        nc = cache_ck.shape[-2]
+        if nc > 0:
+            ak = torch.cat((self.compress_mem_kv[0][None].expand(b, -1, -1, -1), cache_ck), dim=-2)
+            av = torch.cat((self.compress_mem_kv[1][None].expand(b, -1, -1, -1), cache_cv), dim=-2)
+            c_out, _ = ops.dense_attend_f32(q, ak, av, 1, False, 0, st, M)
+        else:
+            c_out = torch.zeros_like(q)
+
+        # selected blocks + own block up to the token (NSA.py:446-515)
+        imp = None
+        if self.num_selected_blocks > 0 and nc > 0:
+            imp = ops.importance_logits_f32(q, cache_ck, st, B, self.query_heads_share_selected_kv, False, mask_own=False)
+        num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
+        if num_sel > 0:
+            _, idx, fmask = ops.importance_topk(imp.contiguous(), num_sel)
+        else:
+            idx = torch.zeros((b, self.kv_heads, 1, 0), dtype=torch.int32, device=x.device)
+            fmask = idx.bool()
+        f_out = ops.native_sparse_attend_f32(rq, keys, vals, B, idx, fmask, include_block_causal=True, q_offset=t)
+        # last window + 1 keys (NSA.py:519-530)
+        s_out, _ = ops.dense_attend_f32(rq, keys, vals, 0, True, self.sliding_window_size, q_offset=t)
+
+        # a compression window is complete: compress it, keep the overlap (NSA.py:422-441)
+        ck, cv = cache_ck, cache_cv
+        if run_k.shape[-2] % cbs == 0:
+            next_ck = self.k_compress((run_k + self.k_intrablock_positions)[:, :, None])
+            next_cv = self.v_compress((run_v + self.v_intrablock_positions)[:, :, None])
+            run_k, run_v = run_k[..., st:, :], run_v[..., st:, :]
+            ck, ck_row = _append_rows(cache_ck, dtype=f32)
+            cv, cv_row = _append_rows(cache_cv, dtype=f32)
+            ck_row.copy_(next_ck)
+            cv_row.copy_(next_cv)
+
+        gates = self.to_strategy_combine(x)                                   # 'b h 1 3' after the sigmoid
+        merged = gates[..., 0:1] * c_out + gates[..., 1:2] * f_out + gates[..., 2:3] * s_out
+        out = self.combine_heads(merged.permute(0, 2, 1, 3).reshape(b, 1, self.heads * d))
+        if not return_cache:
+            return out
+        return out, ((keys, vals), ((ck, cv), (run_k, run_v)))
+
+    @torch.no_grad()
+    def _forward_fp32(self, x, qkv, return_cache):
+        """The parallel forward of an fp32 module without gradients: every attention branch through the fp32 kernels
+        (ops.*_f32), the gate and the merge in fp32 torch - the same steps as `forward` (NSA.py:579-862)."""
+        b, n, _ = x.shape
+        st, cbs, B = self.compress_block_sliding_stride, self.compress_block_size, self.selection_block_size
+        M, d = self.num_mem_compress_kv, self.dim_head
+        q, k, v = qkv.split(self.qkv_split, dim=-1)
+        q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
+        L = (n // st) * st
+        if d in (64, 128):
+            _, rq, rk, _, kw, vw = ops.qkv_prep_f32(qkv, self.rotary_emb.freqs, self.k_intrablock_positions, self.v_intrablock_positions,
+                                                    self.heads, self.kv_heads, d, cbs, st)
+        else:
+            rq, rk = self.rotary_emb.rotate(q), self.rotary_emb.rotate(k)
+            win = lambda t, pos: F.pad(t[..., :L, :], (0, 0, cbs - st, 0)).unfold(2, cbs, st).permute(0, 1, 2, 4, 3) + pos[None, :, None]
+            kw, vw = win(k, self.k_intrablock_positions), win(v, self.v_intrablock_positions)
+        ck0, cv0 = self.k_compress(kw), self.v_compress(vw)
+        ck = torch.cat((self.compress_mem_kv[0][None].expand(b, -1, -1, -1), ck0), dim=-2)
+        cv = torch.cat((self.compress_mem_kv[1][None].expand(b, -1, -1, -1), cv0), dim=-2)
+        nc = ck0.shape[-2]
+        c_out, _ = ops.dense_attend_f32(q, ck, cv, 1, self.causal, 0, st, M)
+        imp = None
+        if self.num_selected_blocks > 0 and nc > 0:
+            imp = ops.importance_logits_f32(q, ck0, st, B, self.query_heads_share_selected_kv, self.causal)
+        num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
+        if num_sel > 0:
+            _, idx, fmask = ops.importance_topk(imp.contiguous(), num_sel)
+            f_out = ops.native_sparse_attend_f32(rq, rk, v, B, idx, fmask, include_block_causal=self.causal)
+        elif self.causal:
+            idx = torch.zeros((b, self.kv_heads, n, 0), dtype=torch.int32, device=x.device)
+            f_out = ops.native_sparse_attend_f32(rq, rk, v, B, idx, idx.bool(), include_block_causal=True)
+        else:
+            own = (torch.arange(n, device=x.device, dtype=torch.int32) // B)[None, None, :, None].expand(b, self.kv_heads, n, 1).contiguous()
+            f_out = ops.native_sparse_attend_f32(rq, rk, v, B, own, torch.ones_like(own, dtype=torch.bool), include_block_causal=False)
+        s_out, _ = ops.dense_attend_f32(rq, rk, v, 0, self.causal, self.sliding_window_size)
+        gates = self.to_strategy_combine(x)                                   # 'b h n 3' after the sigmoid
+        merged = gates[..., 0:1] * c_out + gates[..., 1:2] * f_out + gates[..., 2:3] * s_out
+        out = self.combine_heads(merged.permute(0, 2, 1, 3).reshape(b, n, self.heads * d))
+        if not return_cache:
+            return out
+        co = cbs - st
+        run_k, run_v = k, v
+        if co > 0:
+            run_k, run_v = F.pad(run_k, (0, 0, co, 0)), F.pad(run_v, (0, 0, co, 0))
+        return out, ((rk, v), ((ck0, cv0), (run_k[..., L:, :], run_v[..., L:, :])))
+
     def forward(self, inp, cache=None, disable_triton_kernel=False, sliding_window_flex_mask=None,
                 fine_selection_flex_mask=None, return_cache=False):
         if cache is not None:
@@ -246,6 +358,9 @@ class SparseAttention(nn.Module):
 
         x = self.norm(inp)
         qkv = self.to_qkv(x)
+        if (self.fp32_inference_kernels and qkv.dtype == torch.float32 and not (torch.is_grad_enabled() and qkv.requires_grad)
+                and self.dim_head <= 128 and self.dim_head % 4 == 0 and not torch.compiler.is_compiling()):
+            return self._forward_fp32(x, qkv, return_cache)
         q, k, v = qkv.split(self.qkv_split, dim=-1)
         q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)      # views; read below only by the unfused path and the caches
 

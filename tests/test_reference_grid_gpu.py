@@ -1,7 +1,7 @@
 """The reference's own inference tests (tests/test_sparse_attn.py:46-118) run against the HIP module: token-by-token
 decoding from an empty cache equals the parallel forward, for compress block 5 and selection blocks 8 / 16 / 20, and
-greedy sampling with and without the caches gives the same tokens for selection blocks 4 and 8.  The reference asserts
-1e-5 in fp32; the modules here hold fp32 parameters but compute in bf16, so the bound is the bf16 one."""
+greedy sampling with and without the caches gives the same tokens for selection blocks 4 and 8.  The modules are fp32 and
+run without gradients, so they take the fp32 kernels and the reference's own bound, 1e-5, applies unchanged."""
 import pytest
 import torch
 
@@ -28,8 +28,29 @@ def test_inference(seq_len, num_selected_blocks, compress_block_sliding_stride, 
             sequential_out.append(one_out)
     sequential_out = torch.cat(sequential_out, dim=1)
     assert parallel_out.shape == tokens.shape
-    # bf16 bound; the parallel and the decode kernels round the importance scores differently, so a near-tie may select
-    # another block at an isolated position - such positions stay within the looser bound and are few
+    assert parallel_out.dtype == torch.float32
+    assert torch.allclose(parallel_out, sequential_out, atol=1e-5), (parallel_out - sequential_out).abs().max().item()
+
+
+@pytest.mark.parametrize('seq_len', (16, 70))
+@pytest.mark.parametrize('selection_block_size', (8, 20))
+def test_inference_bf16_kernels(seq_len, selection_block_size):
+    """The same comparison through the bf16 MFMA kernels (fp32 kernels switched off): bf16 bound; the parallel and the decode
+    kernels round the importance scores differently, so a near-tie may select another block at an isolated position - such
+    positions stay within the looser bound and are few."""
+    from native_sparse_attention_pytorch_amd import SparseAttention
+    torch.manual_seed(seq_len * 100 + selection_block_size)
+    attn = SparseAttention(dim=512, dim_head=64, heads=8, causal=True, sliding_window_size=2, compress_block_size=5,
+                           selection_block_size=selection_block_size, num_selected_blocks=2, compress_block_sliding_stride=2).to(DEV)
+    attn.fp32_inference_kernels = False
+    tokens = torch.randn(2, seq_len, 512, device=DEV)
+    with torch.no_grad():
+        parallel_out = attn(tokens)
+        cache, sequential_out = None, []
+        for i in range(seq_len):
+            one_out, cache = attn(tokens[:, i:(i + 1)], cache=cache, return_cache=True)
+            sequential_out.append(one_out)
+    sequential_out = torch.cat(sequential_out, dim=1)
     err = (parallel_out - sequential_out).abs()
     assert err.max().item() < 5e-2 and (err > 5e-3).float().mean().item() < 0.02, (err.max().item(), (err > 5e-3).float().mean().item())
 
@@ -45,10 +66,8 @@ def test_transformer_inference(selection_block_size):
     sampled = model.sample(prompt, 128, temperature=0., use_cache_kv=False)
     sampled_cached = model.sample(prompt, 128, temperature=0., use_cache_kv=True)
     assert sampled.shape == sampled_cached.shape == (1, 127)
-    # bf16 arithmetic: a near-tie between two logits may flip one token, after which the sequences differ
-    same = (sampled == sampled_cached)[0]
-    first_diff = int((~same).float().argmax()) if not bool(same.all()) else same.numel()
-    assert first_diff >= 32, f"cached and uncached greedy sampling part ways after {first_diff} tokens"
+    # fp32 model, fp32 kernels: the reference's assertion unchanged
+    assert torch.allclose(sampled, sampled_cached)
 
 
 def test_readme_configuration():
