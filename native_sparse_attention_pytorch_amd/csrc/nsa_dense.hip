@@ -38,6 +38,17 @@ __device__ __forceinline__ Interval visible_range(const DensePlan& P, int i) {
 
 constexpr int kBK = 64;          // keys per K/V tile
 
+// Work-group ids go round-robin over the 8 XCDs, each with its own L2.  Work items that re-read each other's rows
+// (neighbouring query tiles of a sliding window, neighbouring key tiles of its backward, the key tiles of one query
+// chunk) must therefore not be neighbours in work-group id: item v = (x % 8) * ceil(count / 8) + x / 8 gives every
+// XCD one contiguous range of items, walked in order.  Measured on the sliding-window kernels at seq 32k (window 512):
+// with ids taken as they come every tile fetched its rows from HBM (forward 2.6 GB for 0.4 GB of operands).
+__device__ __forceinline__ int xcd_contiguous(int x, int count) {
+  const int per = (count + 7) >> 3;
+  return (x & 7) * per + (x >> 3);
+}
+static inline unsigned xcd_grid_for(int count) { return 8u * (unsigned)((count + 7) >> 3); }
+
 // One thread's share of a cooperative, coalesced load of `nrows` rows of D bf16 (row index ->
 // memory row through `first_row`, rows >= limit read as zero) by a work-group of NT threads.
 template <int D, int NT>
@@ -89,7 +100,12 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
   const int ppt = 32 >> P.lg;                       // queries per wave tile
-  const int q0 = blockIdx.x * 4 * ppt;              // first query of the work-group
+  // band mode: equal work per tile, neighbouring tiles share most of their window -> one XCD per contiguous range of tiles;
+  // stride mode keeps the round-robin order (causal: work grows with the position, and the compressed keys fit every L2)
+  const int qtiles = (P.n + 4 * ppt - 1) / (4 * ppt);
+  const int xt = P.mode == 0 ? xcd_contiguous(blockIdx.x, qtiles) : (int)blockIdx.x;
+  if (xt >= qtiles) return;
+  const int q0 = xt * 4 * ppt;                      // first query of the work-group
   const int i0 = q0 + wave * ppt;
   const int pq = n_ >> P.lg, g = n_ & (P.g - 1);
   const bool valid = i0 + pq < P.n;
@@ -332,7 +348,10 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P,
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
   const int ppt = 32 >> P.lg;
-  const int q0 = blockIdx.x * 4 * ppt;
+  const int qtiles = (P.n + 4 * ppt - 1) / (4 * ppt);
+  const int xt = P.mode == 0 ? xcd_contiguous(blockIdx.x, qtiles) : (int)blockIdx.x;      // see the forward kernel
+  if (xt >= qtiles) return;
+  const int q0 = xt * 4 * ppt;
   const int i0 = q0 + wave * ppt;
   const int pq = n_ >> P.lg, g = n_ & (P.g - 1);
   const bool valid = i0 + pq < P.n;
@@ -452,10 +471,26 @@ __device__ __forceinline__ void chunk_range(const DensePlan& P, int T, int c, in
   }
 }
 
-__device__ __forceinline__ void chunk_of(const DensePlan& P, int x, int& T, int& c, int& qlo, int& qhi, int& c0, int& c1) {
-  if (P.mode == 0) { T = x / P.chunks; c = x % P.chunks; }
-  else { c = x / P.key_tiles; T = x % P.key_tiles; }
+// Work-group x of the dK/dV walk -> (key tile T, query chunk c); false for the padding ids of the grid.  Band mode:
+// tile-major, one contiguous range of key tiles per XCD (neighbouring tiles see almost the same queries).  Stride mode:
+// all key tiles of a query chunk on one XCD (they stream the same Q / dO rows), chunks dealt to the XCDs in a zig-zag
+// (rounds of 8 chunks, every other round reversed) because under the causal mask a later chunk sees more key tiles.
+__device__ __forceinline__ bool chunk_of(const DensePlan& P, int x, int& T, int& c, int& qlo, int& qhi, int& c0, int& c1) {
+  if (P.mode == 0) {
+    const int v = xcd_contiguous(x, P.key_tiles * P.chunks);
+    if (v >= P.key_tiles * P.chunks) return false;
+    T = v / P.chunks; c = v % P.chunks;
+  } else {
+    const int xc = x & 7, idx = x >> 3, round = idx / P.key_tiles;
+    T = idx % P.key_tiles;
+    c = 8 * round + ((round & 1) ? 7 - xc : xc);
+    if (c >= P.chunks) return false;
+  }
   chunk_range(P, T, c, qlo, qhi, c0, c1);
+  return true;
+}
+static inline unsigned dkv_grid(const DensePlan& P) {
+  return P.mode == 0 ? xcd_grid_for(P.key_tiles * P.chunks) : 8u * (unsigned)(((P.chunks + 7) / 8) * P.key_tiles);
 }
 
 #ifndef NSA_DKV_AHEAD
@@ -486,7 +521,7 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
   // chunk-major order, so that work-groups running together read the same Q/dO chunk (L2 reuse
   // across the key tiles) instead of each streaming its own.
   int T, c, qlo, qhi, c0, c1;
-  chunk_of(P, blockIdx.x, T, c, qlo, qhi, c0, c1);
+  if (!chunk_of(P, blockIdx.x, T, c, qlo, qhi, c0, c1)) return;
   if (c0 >= c1) return;
 
   const int kr_ = kBK * T + 32 * kt + n_;                // this lane's row of k/v
@@ -663,7 +698,7 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_pipe_kernel(const DensePlan
   const int kt = threadIdx.x >> 6, lane = threadIdx.x & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
   int T, c, qlo, qhi, c0, c1;
-  chunk_of(P, blockIdx.x, T, c, qlo, qhi, c0, c1);
+  if (!chunk_of(P, blockIdx.x, T, c, qlo, qhi, c0, c1)) return;
   if (c0 >= c1) return;
 
   const int kr_ = kBK * T + 32 * kt + n_;                // this lane's row of k/v
@@ -903,7 +938,7 @@ extern "C" int nsa_dense_workspace_bytes(const nsa_dense_desc* d, size_t* bwd_by
 template <int D, int NPF>
 static int dense_fwd_launch2(const DensePlan& P, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, hipStream_t st) {
   const int qpw = 4 * (32 >> P.lg);                 // queries per work-group
-  hipLaunchKernelGGL((dense_fwd_kernel<D, NPF>), dim3((P.n + qpw - 1) / qpw, P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+  hipLaunchKernelGGL((dense_fwd_kernel<D, NPF>), dim3(P.mode == 0 ? xcd_grid_for((P.n + qpw - 1) / qpw) : (unsigned)((P.n + qpw - 1) / qpw), P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (__bf16*)out, lse, pooled);
   NSA_LAUNCH_CHECK();
   return 0;
@@ -943,14 +978,14 @@ static int dense_bwd_launch(const DensePlan& P, const void* q, const void* k, co
   hipLaunchKernelGGL((dense_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, delta);
   NSA_LAUNCH_CHECK();
   const int qpw = 4 * (32 >> P.lg);
-  hipLaunchKernelGGL((dense_bwd_dq_kernel<D>), dim3((P.n + qpw - 1) / qpw, P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+  hipLaunchKernelGGL((dense_bwd_dq_kernel<D>), dim3(P.mode == 0 ? xcd_grid_for((P.n + qpw - 1) / qpw) : (unsigned)((P.n + qpw - 1) / qpw), P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (const __bf16*)dout, lse, delta, (__bf16*)dq);
   NSA_LAUNCH_CHECK();
   if (NSA_DKV_PIPE)
-    hipLaunchKernelGGL((dense_bwd_dkv_pipe_kernel<D>), dim3(P.key_tiles * P.chunks, P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+    hipLaunchKernelGGL((dense_bwd_dkv_pipe_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
   else
-    hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(P.key_tiles * P.chunks, P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+    hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
   NSA_LAUNCH_CHECK();
   hipLaunchKernelGGL((dense_bwd_dkv_reduce_kernel<D>), dim3(P.key_tiles, P.bh), dim3(256), 0, st, P, part, dk, dv);
