@@ -981,7 +981,9 @@ static int dense_bwd_launch(const DensePlan& P, const void* q, const void* k, co
   hipLaunchKernelGGL((dense_bwd_dq_kernel<D>), dim3(P.mode == 0 ? xcd_grid_for((P.n + qpw - 1) / qpw) : (unsigned)((P.n + qpw - 1) / qpw), P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (const __bf16*)dout, lse, delta, (__bf16*)dq);
   NSA_LAUNCH_CHECK();
-  if (NSA_DKV_PIPE)
+  // d = 64 fits two waves per SIMD in the plain kernel (219 registers), which overlap each other's phases; the pipelined
+  // kernel needs the whole register file of a SIMD for one wave and is slower there (config-3 module: 280 against 200 us)
+  if (NSA_DKV_PIPE && D == 128)
     hipLaunchKernelGGL((dense_bwd_dkv_pipe_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
   else
