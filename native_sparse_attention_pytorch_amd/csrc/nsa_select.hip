@@ -594,17 +594,33 @@ __global__ __launch_bounds__(256) void sel_fwd_combine_kernel(const SelPlan P, c
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    for (unsigned long long m = live; m; m &= m - 1) {
-      const int s = __builtin_ctzll(m);
-      const size_t row = row0 + (size_t)s * P.g;
-      const float ls = __builtin_nontemporal_load(lsepart + row);
-      const bf16x8 o = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(opart + row * D + dd));
-      const float mn = fmaxf(mx, ls);
-      const float a = __expf(mx - mn), w = __expf(ls - mn);      // first slot: mx = -inf -> a = 0
-      sum = sum * a + w;
+    // the slots are merged in order, but their loads are requested eight slots at a time: taken one by one every slot
+    // costs a memory round trip, which is all a short sequence has to hide behind
+    for (unsigned long long m = live; m;) {
+      int sl[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * a + w * (float)o[e];
-      mx = mn;
+      for (int u = 0; u < 8; ++u) {
+        sl[u] = m ? __builtin_ctzll(m) : -1;
+        m &= m - 1;                                          // 0 stays 0
+      }
+      float ls[8];
+      bf16x8 o[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const size_t row = row0 + (size_t)max(sl[u], 0) * P.g;
+        ls[u] = __builtin_nontemporal_load(lsepart + row);
+        o[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(opart + row * D + dd));
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (sl[u] < 0) continue;
+        const float mn = fmaxf(mx, ls[u]);
+        const float a = __expf(mx - mn), w = __expf(ls[u] - mn);      // first slot: mx = -inf -> a = 0
+        sum = sum * a + w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = acc[e] * a + w * (float)o[u][e];
+        mx = mn;
+      }
     }
     const float L = live ? mx + __logf(sum) : -INFINITY;
     const float inv = live ? 1.0f / sum : 0.f;
@@ -800,11 +816,23 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    for (unsigned long long m = live; m; m &= m - 1) {
-      const int s = __builtin_ctzll(m);
-      const bf16x8 o = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(dqpart + (row0 + (size_t)s * P.g) * D + dd));
+    for (unsigned long long m = live; m;) {                 // eight slots' loads in flight at a time, summed in slot order
+      int sl[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += (float)o[e];
+      for (int u = 0; u < 8; ++u) {
+        sl[u] = m ? __builtin_ctzll(m) : -1;
+        m &= m - 1;
+      }
+      bf16x8 o[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        o[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(dqpart + (row0 + (size_t)max(sl[u], 0) * P.g) * D + dd));
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (sl[u] < 0) continue;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += (float)o[u][e];
+      }
     }
     bf16x8 r;
 #pragma unroll
