@@ -336,6 +336,14 @@ __device__ __forceinline__ void commit_tile(const bf16x8 (&raw)[D / 16], __bf16*
   }
 }
 
+// the same into a swizzled tile (lds_swz_off: conflict-free for row reads and for the transpose load)
+template <int D>
+__device__ __forceinline__ void commit_tile_swz(const bf16x8 (&raw)[D / 16], __bf16* tile_s, int lane) {
+  constexpr int CPR = D / 8, RPI = 64 / CPR, NT = 32 / RPI;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) *reinterpret_cast<bf16x8*>(tile_s + lds_swz_off<D>(t * RPI + lane / CPR, lane % CPR)) = raw[t];
+}
+
 // Write a wave's 32-row x D accumulator tile (transposed MFMA layout: lane <-> row n_,
 // register (dt, a, b) <-> feature 32dt + 8a + 4h + b) as bf16 rows through LDS, so that every
 // global store instruction covers whole 2*D-byte rows (16 bytes per lane, consecutive lanes
@@ -594,33 +602,17 @@ __global__ __launch_bounds__(256) void sel_fwd_combine_kernel(const SelPlan P, c
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    // the slots are merged in order, but their loads are requested eight slots at a time: taken one by one every slot
-    // costs a memory round trip, which is all a short sequence has to hide behind
-    for (unsigned long long m = live; m;) {
-      int sl[8];
+    for (unsigned long long m = live; m; m &= m - 1) {
+      const int s = __builtin_ctzll(m);
+      const size_t row = row0 + (size_t)s * P.g;
+      const float ls = __builtin_nontemporal_load(lsepart + row);
+      const bf16x8 o = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(opart + row * D + dd));
+      const float mn = fmaxf(mx, ls);
+      const float a = __expf(mx - mn), w = __expf(ls - mn);      // first slot: mx = -inf -> a = 0
+      sum = sum * a + w;
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        sl[u] = m ? __builtin_ctzll(m) : -1;
-        m &= m - 1;                                          // 0 stays 0
-      }
-      float ls[8];
-      bf16x8 o[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const size_t row = row0 + (size_t)max(sl[u], 0) * P.g;
-        ls[u] = __builtin_nontemporal_load(lsepart + row);
-        o[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(opart + row * D + dd));
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        if (sl[u] < 0) continue;
-        const float mn = fmaxf(mx, ls[u]);
-        const float a = __expf(mx - mn), w = __expf(ls[u] - mn);      // first slot: mx = -inf -> a = 0
-        sum = sum * a + w;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] = acc[e] * a + w * (float)o[u][e];
-        mx = mn;
-      }
+      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * a + w * (float)o[e];
+      mx = mn;
     }
     const float L = live ? mx + __logf(sum) : -INFINITY;
     const float inv = live ? 1.0f / sum : 0.f;
@@ -816,23 +808,11 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    for (unsigned long long m = live; m;) {                 // eight slots' loads in flight at a time, summed in slot order
-      int sl[8];
+    for (unsigned long long m = live; m; m &= m - 1) {
+      const int s = __builtin_ctzll(m);
+      const bf16x8 o = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(dqpart + (row0 + (size_t)s * P.g) * D + dd));
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        sl[u] = m ? __builtin_ctzll(m) : -1;
-        m &= m - 1;
-      }
-      bf16x8 o[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        o[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(dqpart + (row0 + (size_t)max(sl[u], 0) * P.g) * D + dd));
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        if (sl[u] < 0) continue;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] += (float)o[u][e];
-      }
+      for (int e = 0; e < 8; ++e) acc[e] += (float)o[e];
     }
     bf16x8 r;
 #pragma unroll
@@ -855,6 +835,9 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 // [key][row] in LDS; dQ^T = K^T dS^T is then formed with both operands read through the
 // transpose load (K block row-major in LDS, loaded once per unit), each wave taking half of the
 // features, and the finished 32 x D tile leaves through coalesced row stores.
+#ifndef NSA_SEL_SWZ
+#define NSA_SEL_SWZ 1      // Q / dO tiles of the backward walk in the swizzled layout (read as rows and through the transpose load)
+#endif
 #ifndef NSA_BWD_STAGES_D64
 #define NSA_BWD_STAGES_D64 1
 #endif
@@ -968,10 +951,10 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
     const RowInfo r = cur.r;
     // commit the current tile to LDS
     if (KT == 1) {
-      commit_tile<D>(cur.raw[0], xq_s, RS, lane);
-      commit_tile<D>(cur.raw[NR - 1], xg_s, RS, lane);
+      NSA_SEL_SWZ ? commit_tile_swz<D>(cur.raw[0], xq_s, lane) : commit_tile<D>(cur.raw[0], xq_s, RS, lane);
+      NSA_SEL_SWZ ? commit_tile_swz<D>(cur.raw[NR - 1], xg_s, lane) : commit_tile<D>(cur.raw[NR - 1], xg_s, RS, lane);
     } else {
-      commit_tile<D>(cur.raw[0], load_q ? xq_s : xg_s, RS, lane);
+      NSA_SEL_SWZ ? commit_tile_swz<D>(cur.raw[0], load_q ? xq_s : xg_s, lane) : commit_tile<D>(cur.raw[0], load_q ? xq_s : xg_s, RS, lane);
     }
     if (kt == 0 && h == 0) {
       lse_s[n_] = r.valid ? cur.lse_r * kLog2e : INFINITY; // +inf: a padding row gets p = 0
@@ -991,7 +974,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
 
     floatx16 Sa = zero_acc(), Pa = zero_acc();              // [row][key]: lane <-> key, registers <-> rows
     operands_ahead<2 * KS, AHD>(
-        [&](int i) { return lds_row_operand((i & 1) ? xg_s : xq_s, RS, i >> 1, lane); },
+        [&](int i) { return NSA_SEL_SWZ ? lds_row_operand_swz<D>((i & 1) ? xg_s : xq_s, i >> 1, lane) : lds_row_operand((i & 1) ? xg_s : xq_s, RS, i >> 1, lane); },
         [&](int i, const bf16x8& a) {
           if (i & 1) Pa = mfma32(a, Vf[i >> 1], Pa);
           else Sa = mfma32(a, Kf[i >> 1], Sa);
@@ -1041,7 +1024,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
     }
     // dV^T += dO^T P, dK^T += Q^T dS
     operands_ahead<4 * DT, AHD>(
-        [&](int i) { return lds_transposed_operand((i & 2) ? xq_s : xg_s, RS, 16 * (i & 1), 32 * (i >> 2), lane); },
+        [&](int i) { return NSA_SEL_SWZ ? lds_transposed_operand_swz<D>((i & 2) ? xq_s : xg_s, 16 * (i & 1), 32 * (i >> 2), lane) : lds_transposed_operand((i & 2) ? xq_s : xg_s, RS, 16 * (i & 1), 32 * (i >> 2), lane); },
         [&](int i, const bf16x8& a) {
           const int dt = i >> 2, w = i & 3;
           if (w == 0) dVa[dt] = mfma32(a, Pf0, dVa[dt]);
