@@ -414,7 +414,11 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P,
 #pragma unroll
         for (int i2 = 0; i2 < 16; ++i2) {
           const int key = kb0 + 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
-          const float p = (!decltype(masked)::value || (key >= klo && key <= khi)) ? fast_exp2(Sa[kt][i2] * sc - lse_r) : 0.f;
+          // the mask goes into the exponent (exp2(-inf) = 0, '&' instead of '&&'): a select around the exponential is compiled
+          // as a branch per element
+          float x = __builtin_fmaf(Sa[kt][i2], sc, -lse_r);
+          if (decltype(masked)::value) x = ((key >= klo) & (key <= khi)) ? x : -INFINITY;
+          const float p = fast_exp2(x);
           Sa[kt][i2] = p * (Pa[kt][i2] - del_r);
         }
 #pragma unroll
@@ -610,7 +614,9 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
 #pragma unroll
         for (int bb = 0; bb < 4; ++bb) {
           const int i2 = 4 * a + bb;
-          const float p = (!decltype(masked)::value || (kr_ >= lo4[bb] && kr_ <= hi4[bb])) ? fast_exp2(Sa[i2] * sc - l4[bb]) : 0.f;
+          float x = __builtin_fmaf(Sa[i2], sc, -l4[bb]);      // mask in the exponent: see the dQ kernel
+          if (decltype(masked)::value) x = ((kr_ >= lo4[bb]) & (kr_ <= hi4[bb])) ? x : -INFINITY;
+          const float p = fast_exp2(x);
           Sa[i2] = p;
           dSa[i2] = p * (Pa[i2] - d4[bb]);
         }
@@ -655,226 +661,6 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
 #pragma unroll
   for (int s2 = 0; s2 < NS - 1; ++s2)
     if (i0 + s2 * ppt < c1) step(i0 + s2 * ppt, stg[s2]);
-  // partial [bh][tile][chunk][2][64][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][row 32kt + n_]
-  float* pk = part + (((size_t)bh * P.key_tiles + T) * P.chunks + c) * (2 * kBK * D) + (size_t)(32 * kt + n_) * D + 4 * h;
-  float* pv = pk + kBK * D;
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      floatx4 x, y;
-#pragma unroll
-      for (int bb = 0; bb < 4; ++bb) { x[bb] = dKa[dt][4 * a + bb]; y[bb] = dVa[dt][4 * a + bb]; }
-      *reinterpret_cast<floatx4*>(pk + 32 * dt + 8 * a) = x;
-      *reinterpret_cast<floatx4*>(pv + 32 * dt + 8 * a) = y;
-    }
-}
-
-#ifndef NSA_DKV_PIPE
-#define NSA_DKV_PIPE 1        // 1: the software-pipelined dK/dV kernel below, 0: the plain one above
-#endif
-
-// The same dK/dV walk as a software pipeline inside each wave.  At d = 128 a wave's accumulators and
-// K / V operands leave room for one wave per SIMD only, so nothing but the wave itself can fill the
-// MFMA pipe while its softmax runs on the VALU (and the other way round): in the plain kernel a tile
-// costs S / dP products, softmax, dV / dK products and two barriers strictly one after the other.
-// Here the Q / dO tiles live in a ring of three LDS buffers and iteration t runs
-//   phase A: S, dP of tile t+1 (MFMA, operands from buffer t+1)  together with  P, dS of tile t (VALU)
-//   phase B: dV, dK of tile t (MFMA, transposed operands from buffer t)  together with  the commit of
-//            tile t+2's rows (already in registers) to buffer t+2 and the gathers of tile t+3
-// with one barrier per tile: it publishes the commit of the iteration before and retires the buffer
-// the commit of this iteration overwrites (last read in phase B two iterations back).
-template <int D>
-__global__ __launch_bounds__(128) void dense_bwd_dkv_pipe_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
-                                                                 const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
-                                                                 const float* __restrict__ lse, const float* __restrict__ delta, float* __restrict__ part) {
-  constexpr int KS = D / 16, DT = D / 32, RS = D, NB = 3;      // swizzled tiles (lds_swz_off): no row padding
-  __shared__ __align__(16) float lse_s[NB][32];
-  __shared__ __align__(16) float del_s[NB][32];
-  __shared__ __align__(16) int lo_s[NB][32];
-  __shared__ __align__(16) int hi_s[NB][32];
-  __shared__ __align__(16) __bf16 xq_s[NB][32 * RS];
-  __shared__ __align__(16) __bf16 xg_s[NB][32 * RS];
-  const int kt = threadIdx.x >> 6, lane = threadIdx.x & 63, n_ = lane & 31, h = lane >> 5;
-  const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
-  int T, c, qlo, qhi, c0, c1;
-  if (!chunk_of(P, blockIdx.x, T, c, qlo, qhi, c0, c1)) return;
-  if (c0 >= c1) return;
-
-  const int kr_ = kBK * T + 32 * kt + n_;                // this lane's row of k/v
-  const bool kok = kr_ < P.krows;
-  bf16x8 Kf[KS], Vf[KS];
-  {
-    const long krow = kok ? kr_ : 0;
-    const __bf16* kp = k + b * P.sk[0] + hk * P.sk[1] + krow * P.sk[2] + 8 * h;
-    const __bf16* vp = v + b * P.sv[0] + hk * P.sv[1] + krow * P.sv[2] + 8 * h;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      Kf[ks] = kok ? load8(kp + 16 * ks) : zero_frag();
-      Vf[ks] = kok ? load8(vp + 16 * ks) : zero_frag();
-    }
-  }
-  floatx16 dKa[DT], dVa[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt) { dKa[dt] = zero_acc(); dVa[dt] = zero_acc(); }
-  const float sc = P.scale * kLog2e;
-  const int ppt = 32 >> P.lg;
-  const int pq = n_ >> P.lg, g = n_ & (P.g - 1);
-  const int hq = hk * P.g + g;
-  const __bf16* qbase = q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1];
-  const __bf16* gbase = dout + b * P.sdo[0] + (long)(hk * P.g) * P.sdo[1];
-  constexpr int CPR = D / 8, RPI = 64 / CPR, NT = 32 / RPI;
-
-  // wave 0 gathers a tile's Q rows, wave 1 its dO rows (coalesced 16-byte loads into registers)
-  struct Stage { bf16x8 raw[NT]; float lse_r, del_r; };
-  auto issue = [&](Stage& st, int i0) {
-    const __bf16* base = kt == 0 ? qbase : gbase;
-    const long sh = kt == 0 ? P.sq[1] : P.sdo[1], sn = kt == 0 ? P.sq[2] : P.sdo[2];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int rr = t * RPI + lane / CPR;
-      const int qi = min(i0 + (rr >> P.lg), P.n - 1);
-      const unsigned long off = (unsigned long)(unsigned)(rr & (P.g - 1)) * (unsigned)sh + (unsigned long)(unsigned)qi * (unsigned)sn;
-      st.raw[t] = load8(base + off + 8 * (lane % CPR));
-    }
-    const int qi = min(i0 + pq, P.n - 1);
-    const long srow = ((long)b * P.hkv * P.g + hq) * P.n + qi;
-    st.lse_r = lse[srow]; st.del_r = delta[srow];
-  };
-  auto commit = [&](const Stage& st, int i0, int buf) {
-    __bf16* dst = kt == 0 ? xq_s[buf] : xg_s[buf];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) *reinterpret_cast<bf16x8*>(dst + lds_swz_off<D>(t * RPI + lane / CPR, lane % CPR)) = st.raw[t];
-    if (kt == 0 && h == 0) {
-      const bool valid = i0 + pq < c1;
-      const int i = min(i0 + pq, P.n - 1);
-      lse_s[buf][n_] = valid ? st.lse_r * kLog2e : INFINITY;   // +inf: a padding row gets p = 0
-      del_s[buf][n_] = st.del_r;
-      const Interval me = visible_range(P, i);
-      lo_s[buf][n_] = P.mode == 0 ? me.lo : 0;
-      hi_s[buf][n_] = P.mode == 0 ? me.hi : me.hi + P.mem;
-    }
-  };
-  // S = Q K^T and dP = dO V^T of the tile in buffer `buf` ([row][key]: lane <-> key, registers <-> rows)
-  auto scores = [&](int buf, floatx16& Sa, floatx16& Pa) {
-    Sa = zero_acc(); Pa = zero_acc();
-    const __bf16* xq = xq_s[buf];
-    const __bf16* xg = xg_s[buf];
-    operands_ahead<2 * KS, NSA_DKV_AHEAD>(
-        [&](int i) { return lds_row_operand_swz<D>((i & 1) ? xg : xq, i >> 1, lane); },
-        [&](int i, const bf16x8& a) {
-          if (i & 1) Pa = mfma32(a, Vf[i >> 1], Pa);
-          else Sa = mfma32(a, Kf[i >> 1], Sa);
-        });
-  };
-  // P = exp2(S * sc - lse), dS = P * (dP - delta) of the tile in buffer `buf`, packed as MFMA operands
-  auto softmax = [&](auto masked, int buf, const floatx16& Sa, const floatx16& Pa, bf16x8 (&Pf)[2], bf16x8 (&Sf)[2]) {
-    floatx16 pa, dSa;
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      const floatx4 l4 = *reinterpret_cast<const floatx4*>(&lse_s[buf][8 * a + 4 * h]);
-      const floatx4 d4 = *reinterpret_cast<const floatx4*>(&del_s[buf][8 * a + 4 * h]);
-      typedef int intx4 __attribute__((ext_vector_type(4)));
-      intx4 lo4 = {0, 0, 0, 0}, hi4 = {0, 0, 0, 0};
-      if (decltype(masked)::value) {
-        lo4 = *reinterpret_cast<const intx4*>(&lo_s[buf][8 * a + 4 * h]);
-        hi4 = *reinterpret_cast<const intx4*>(&hi_s[buf][8 * a + 4 * h]);
-      }
-#pragma unroll
-      for (int bb = 0; bb < 4; ++bb) {
-        const int i2 = 4 * a + bb;
-        // the mask goes into the exponent (exp2(-inf) = 0): a select on the result invites a branch around the exponential
-        float x = __builtin_fmaf(Sa[i2], sc, -l4[bb]);
-        if (decltype(masked)::value) x = ((kr_ >= lo4[bb]) & (kr_ <= hi4[bb])) ? x : -INFINITY;      // '&': no short-circuit branch
-        const float p = fast_exp2(x);
-        pa[i2] = p;
-        dSa[i2] = p * (Pa[i2] - d4[bb]);
-      }
-    }
-    Pf[0] = pack8(pa, 0); Pf[1] = pack8(pa, 8);
-    Sf[0] = pack8(dSa, 0); Sf[1] = pack8(dSa, 8);
-  };
-  // dV^T += dO^T P, dK^T += Q^T dS with the transposed operands of buffer `buf`
-  auto accumulate = [&](int buf, const bf16x8 (&Pf)[2], const bf16x8 (&Sf)[2]) {
-    const __bf16* xq = xq_s[buf];
-    const __bf16* xg = xg_s[buf];
-    operands_ahead<4 * DT, NSA_DKV_AHEAD>(
-        [&](int i) { return lds_transposed_operand_swz<D>((i & 2) ? xq : xg, 16 * (i & 1), 32 * (i >> 2), lane); },
-        [&](int i, const bf16x8& a) {
-          const int dt = i >> 2, w = i & 3;
-          if (w == 0) dVa[dt] = mfma32(a, Pf[0], dVa[dt]);
-          else if (w == 1) dVa[dt] = mfma32(a, Pf[1], dVa[dt]);
-          else if (w == 2) dKa[dt] = mfma32(a, Sf[0], dKa[dt]);
-          else dKa[dt] = mfma32(a, Sf[1], dKa[dt]);
-        });
-  };
-
-  const int ntiles = (c1 - c0 + ppt - 1) / ppt;
-  Stage st;
-  issue(st, c0);
-  wait_all_loads();
-  commit(st, c0, 0);
-  issue(st, c0 + ppt);
-  __syncthreads();
-  floatx16 Sc, Pc;
-  scores(0, Sc, Pc);
-  wait_all_loads();
-  commit(st, c0 + ppt, 1);
-  issue(st, c0 + 2 * ppt);
-  int bc = 0;
-  // one pipeline step; the two register sets for S / dP swap roles from step to step (the loop is unrolled by
-  // two instead of copying 32 registers per tile)
-  auto iter = [&](int ti, floatx16& Sc, floatx16& Pc, floatx16& Sn, floatx16& Pn) {
-    const int bn = bc == NB - 1 ? 0 : bc + 1, bnn = bn == NB - 1 ? 0 : bn + 1;
-    const int i0 = c0 + ti * ppt;
-    __syncthreads();
-    bf16x8 Pf[2], Sf[2];
-    {
-      // rows of this wave are visible to every query of the tile iff they lie between the largest lower
-      // and the smallest upper bound, which consecutive queries take at the tile's ends (wave-uniform)
-      const Interval vf = visible_range(P, min(i0, P.n - 1)), vl = visible_range(P, min(i0 + ppt - 1, P.n - 1));
-      const int all_lo = P.mode == 0 ? vl.lo : 0, all_hi = P.mode == 0 ? vf.hi : vf.hi + P.mem;
-      const int r0 = kBK * T + 32 * kt;
-      // phase A: one straight-line block per variant, the next tile's products in the shadow of this tile's softmax
-      if (r0 >= all_lo && r0 + 31 <= all_hi && i0 + ppt <= c1) {
-        scores(bn, Sn, Pn);
-        softmax(std::false_type{}, bc, Sc, Pc, Pf, Sf);
-        // the order the scheduler is asked for: per MFMA one operand read and its share of the softmax's VALU work
-        // (left alone it emits the sixteen MFMAs first and the softmax after them)
-#pragma unroll
-        for (int i = 0; i < 2 * KS; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 80 / (2 * KS), 0);
-        }
-      } else {
-        scores(bn, Sn, Pn);
-        softmax(std::true_type{}, bc, Sc, Pc, Pf, Sf);
-#pragma unroll
-        for (int i = 0; i < 2 * KS; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 144 / (2 * KS), 0);
-        }
-      }
-    }
-    // phase B: this tile's dV / dK products; the commit of tile ti + 2 and the gathers of tile ti + 3 ride along.
-    // The scheduling fences keep the phases of consecutive steps apart: left free, the scheduler stretches live ranges
-    // across them until the register file overflows.
-    __builtin_amdgcn_sched_barrier(0);
-    accumulate(bc, Pf, Sf);
-    commit(st, i0 + 2 * ppt, bnn);
-    issue(st, i0 + 3 * ppt);
-    __builtin_amdgcn_sched_barrier(0);
-    bc = bn;
-  };
-  floatx16 S1, P1;
-  int ti = 0;
-  for (; ti + 1 < ntiles; ti += 2) {
-    iter(ti, Sc, Pc, S1, P1);
-    iter(ti + 1, S1, P1, Sc, Pc);
-  }
-  if (ti < ntiles) iter(ti, Sc, Pc, S1, P1);
   // partial [bh][tile][chunk][2][64][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][row 32kt + n_]
   float* pk = part + (((size_t)bh * P.key_tiles + T) * P.chunks + c) * (2 * kBK * D) + (size_t)(32 * kt + n_) * D + 4 * h;
   float* pv = pk + kBK * D;
@@ -981,14 +767,8 @@ static int dense_bwd_launch(const DensePlan& P, const void* q, const void* k, co
   hipLaunchKernelGGL((dense_bwd_dq_kernel<D>), dim3(P.mode == 0 ? xcd_grid_for((P.n + qpw - 1) / qpw) : (unsigned)((P.n + qpw - 1) / qpw), P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (const __bf16*)dout, lse, delta, (__bf16*)dq);
   NSA_LAUNCH_CHECK();
-  // d = 64 fits two waves per SIMD in the plain kernel (219 registers), which overlap each other's phases; the pipelined
-  // kernel needs the whole register file of a SIMD for one wave and is slower there (config-3 module: 280 against 200 us)
-  if (NSA_DKV_PIPE && D == 128)
-    hipLaunchKernelGGL((dense_bwd_dkv_pipe_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
-                       (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
-  else
-    hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
-                       (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
+  hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+                     (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
   NSA_LAUNCH_CHECK();
   hipLaunchKernelGGL((dense_bwd_dkv_reduce_kernel<D>), dim3(P.key_tiles, P.bh), dim3(256), 0, st, P, part, dk, dv);
   NSA_LAUNCH_CHECK();

@@ -759,7 +759,7 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
       for (int i2 = 0; i2 < 16; ++i2) {
         const int kl = 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
         const float sraw = Sa[kt][i2];
-        const float p = (kl <= r.lim) ? fast_exp2(sraw * sc - lse_r) : 0.f;
+        const float p = fast_exp2((kl <= r.lim) ? __builtin_fmaf(sraw, sc, -lse_r) : -INFINITY);      // mask in the exponent: no branch around the exponential
         const float ds = p * (Pa[kt][i2] - del_r);
         Sa[kt][i2] = ds;
         if (GATE) gs += ds * sraw;
@@ -1004,7 +1004,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
 #pragma unroll
         for (int bb = 0; bb < 4; ++bb) {
           const int i2 = 4 * a + bb;
-          const float p = (kl <= m4[bb]) ? fast_exp2(__builtin_fmaf(Sa[i2], sc, -l4[bb])) : 0.f;
+          const float p = fast_exp2((kl <= m4[bb]) ? __builtin_fmaf(Sa[i2], sc, -l4[bb]) : -INFINITY);      // mask in the exponent: no branch around the exponential
           Sa[i2] = p;
           dSa[i2] = p * (Pa[i2] - d4[bb]);
         }
