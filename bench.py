@@ -123,9 +123,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="only the headline workload (for profiler runs): no compressed-branch, module or decode legs")
-    ap.add_argument("--skip", default="", help="comma-separated legs to leave out: compressed, module, decode, train, generate")
+    ap.add_argument("--skip", default="", help="comma-separated legs to leave out: rowtraffic, compressed, module, decode, train, generate")
     args = ap.parse_args()
-    skip = set(filter(None, args.skip.split(","))) | ({"compressed", "module", "decode", "train", "generate"} if args.headline_only else set())
+    skip = set(filter(None, args.skip.split(","))) | ({"rowtraffic", "compressed", "module", "decode", "train", "generate"} if args.headline_only else set())
 
     def leg(name):
         """Announce a leg on stderr (a long profiler run must not look hung) or skip it."""
@@ -249,7 +249,7 @@ def main():
                                         # (delta + dQ + dK/dV + reduce kernels together) over the HIP-event time of each call
                                         roofline=dict(bound="mfma", peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
                                                       fwd=dict(kernel="dense_fwd_kernel<128,4>", achieved=round(cf, 2), frac=round(cf / MFMA_PEAK_TFLOPS, 4)),
-                                                      bwd=dict(kernel="dense_bwd_dq_kernel<128> + dense_bwd_dkv_pipe_kernel<128>", achieved=round(cb, 2),
+                                                      bwd=dict(kernel="dense_bwd_dq_kernel<128> + dense_bwd_dkv_kernel<128>", achieved=round(cb, 2),
                                                                frac=round(cb / MFMA_PEAK_TFLOPS, 4)),
                                                       topk=dict(bound="hbm", bytes=int(imp.numel() * 4 + idx_.numel() * 9),
                                                                 achieved_GBs=round((imp.numel() * 4 + idx_.numel() * 9) / (best[1] * 1e-3) / 1e9, 1),
@@ -392,6 +392,35 @@ def main():
         pass
     except Exception as ex:
         res["generate_config5_bf16"] = dict(error=repr(ex))
+
+    # what the memory system gives the walks' access pattern (random 1 KB rows, loads of a round in flight together): the
+    # ceiling to read the hbm_GBs figures against.  2 GB buffers = HBM; a 2 MB source = rows that stay in L2.
+    try:
+        leg("rowtraffic")
+        big = 2 << 30
+        src = torch.zeros(big // 4, dtype=torch.float32, device=dev)
+        dst = torch.zeros(big // 4, dtype=torch.float32, device=dev)
+        rows_big, waves, iters = big // 1024, 8192, 64
+        probe = {}
+        for name, sr, rd, wr in (("gather_hbm", rows_big, 2, 0), ("scatter_hbm", rows_big, 0, 2), ("gather1_scatter1_hbm", rows_big, 1, 1),
+                                 ("gather2_scatter1_hbm", rows_big, 2, 1), ("gather1_scatter2_hbm", rows_big, 1, 2),
+                                 ("gather_l2_scatter_hbm", 2048, 1, 1)):
+            best = None
+            for rep in range(4):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                _lib.check(L.nsa_probe_row_traffic(P(src), sr, P(dst), rows_big, rd, wr, iters, waves, 1, 1000 * rep, stream), "probe")
+                e1.record()
+                torch.cuda.synchronize()
+                t = e0.elapsed_time(e1)
+                best = t if rep > 0 and (best is None or t < best) else best
+            probe[name] = round(waves * iters * 4 * (rd + wr) * 1024 / (best * 1e-3) / 1e9, 1)
+        res["row_traffic_GBs"] = probe
+        del src, dst
+    except _Skip:
+        pass
+    except Exception as ex:
+        res["row_traffic_GBs"] = dict(error=repr(ex))
 
     if not args.no_cpu:
         torch.set_num_threads(min(16, os.cpu_count() or 1))

@@ -33,6 +33,14 @@ int nsa_abi_version(void);
  * identity-operand register transpose.  No reference counterpart (Triton hides layouts). */
 int nsa_selftest_mfma(const void* A, const void* B, float* C, const void* X, float* T, void* stream);
 
+/* Memory-system probe with the access pattern of the block-selection walks (no reference counterpart; used by
+ * bench.py to state the ceiling next to the walks' achieved GB/s).  `waves` wavefronts each repeat `iters` times:
+ * gather `reads` groups of four 1 KB rows from pseudo-random rows of src (src_rows rows of 1 KB), then scatter
+ * `writes` groups of four 1 KB rows to pseudo-random rows of dst (dst_rows rows of 1 KB; ordinary or non-temporal
+ * stores).  reads, writes <= 8.  Moves waves * iters * 4 * (reads + writes) KB. */
+int nsa_probe_row_traffic(const void* src, size_t src_rows, void* dst, size_t dst_rows, int32_t reads, int32_t writes,
+                          int32_t iters, int32_t waves, int32_t nontemporal, uint32_t seed, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Block-selection attention.  Replaces native_sparse_attend / NSA.forward / NSA.backward
  * (TRI.py:1938-1987, 1827-1872, 1875-1925) and the kernels they launch (TRI.py:599-694,

@@ -80,6 +80,8 @@ def lib():
         L.nsa_select_bwd.argtypes = [C.POINTER(SelectDesc)] + [vp] * 10 + [sz] + [vp] * 5
         L.nsa_selftest_mfma.argtypes = [vp] * 6
         L.nsa_selftest_mfma.restype = C.c_int
+        L.nsa_probe_row_traffic.argtypes = [vp, sz, vp, sz, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_uint32, vp]
+        L.nsa_probe_row_traffic.restype = C.c_int
         L.nsa_select_fwd_timed.argtypes = L.nsa_select_fwd.argtypes + [vp, C.c_int]
         L.nsa_select_bwd_timed.argtypes = L.nsa_select_bwd.argtypes + [vp, C.c_int]
         L.nsa_select_fwd_timed.restype = L.nsa_select_bwd_timed.restype = C.c_int
