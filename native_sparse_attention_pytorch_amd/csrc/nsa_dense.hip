@@ -201,32 +201,41 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
             if (npf == 16) { grp[0] += grp[1]; grp[2] += grp[3]; }
             if (npf == 32) { grp[0] = (grp[0] + grp[1]) + (grp[2] + grp[3]); }
           }
+          // the distinct sums of this 32-key half, then the head sums for all of them under one (wave-uniform) decision and
+          // all LDS stores under one predicate: taken value by value, each value carried its own cascade of branches
+          constexpr int NV = npf == 1 ? 16 : npf == 2 ? 8 : npf <= 8 ? 4 : npf == 16 ? 2 : 1;
+          float val[NV];
+          int koff[NV];
 #pragma unroll
-          for (int i2 = 0; i2 < 16; ++i2) {
-            const bool distinct = npf == 1 || (npf == 2 && !(i2 & 1)) || (npf == 4 && !(i2 & 3)) || (npf == 8 && !(i2 & 3)) ||
-                                  (npf == 16 && !(i2 & 7)) || (npf == 32 && i2 == 0);
-            if (!distinct) continue;
-            float val; int koff; bool mine;
-            if (npf == 1) { val = Sraw[kt][i2]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 3); mine = true; }
-            else if (npf == 2) { val = Sraw[kt][i2] + Sraw[kt][i2 | 1]; koff = 8 * (i2 >> 2) + 4 * h + (i2 & 2); mine = true; }
-            else if (npf == 4) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2) + 4 * h; mine = true; }
-            else if (npf == 8) { val = grp[i2 >> 2]; koff = 8 * (i2 >> 2); mine = h == 0; }
-            else if (npf == 16) { val = grp[(i2 >> 3) * 2]; koff = 16 * (i2 >> 3); mine = h == 0; }
-            else { val = grp[0]; koff = 0; mine = h == 0; }
-            int prow_local = n_;                         // row inside the wave tile (per head) ...
-            if (P.share) {
-              if (P.g == 2) {
-                val += dpp_quad_xor1(val);
-              } else if (P.g == 4) {
-                val += dpp_quad_xor1(val);
-                val += dpp_quad_xor2(val);
-              } else {
-                for (int mk = 1; mk < P.g; mk <<= 1) val += __shfl_xor(val, mk, 64);
+          for (int vi = 0; vi < NV; ++vi) {
+            if (npf == 1) { val[vi] = Sraw[kt][vi]; koff[vi] = 8 * (vi >> 2) + 4 * h + (vi & 3); }
+            else if (npf == 2) { val[vi] = Sraw[kt][2 * vi] + Sraw[kt][2 * vi + 1]; koff[vi] = 8 * (vi >> 1) + 4 * h + 2 * (vi & 1); }
+            else if (npf == 4) { val[vi] = grp[vi]; koff[vi] = 8 * vi + 4 * h; }
+            else if (npf == 8) { val[vi] = grp[vi]; koff[vi] = 8 * vi; }
+            else if (npf == 16) { val[vi] = grp[2 * vi]; koff[vi] = 16 * vi; }
+            else { val[vi] = grp[0]; koff[vi] = 0; }
+          }
+          bool mine = npf < 8 || h == 0;
+          int prow_local = n_;                           // row inside the wave tile (per head) ...
+          if (P.share) {
+            if (P.g == 2) {
+#pragma unroll
+              for (int vi = 0; vi < NV; ++vi) val[vi] += dpp_quad_xor1(val[vi]);
+            } else if (P.g == 4) {
+#pragma unroll
+              for (int vi = 0; vi < NV; ++vi) { val[vi] += dpp_quad_xor1(val[vi]); val[vi] += dpp_quad_xor2(val[vi]); }
+            } else {
+              for (int mk = 1; mk < P.g; mk <<= 1) {
+#pragma unroll
+                for (int vi = 0; vi < NV; ++vi) val[vi] += __shfl_xor(val[vi], mk, 64);
               }
-              prow_local = pq;                           // ... or query inside the wave tile (shared)
-              mine = mine && g == 0;
             }
-            if (mine) pw[prow_local * nbt + (32 * kt + koff) / npf] = val;
+            prow_local = pq;                             // ... or query inside the wave tile (shared)
+            mine = mine && g == 0;
+          }
+          if (mine) {
+#pragma unroll
+            for (int vi = 0; vi < NV; ++vi) pw[prow_local * nbt + (32 * kt + koff[vi]) / npf] = val[vi];
           }
         }
         __builtin_amdgcn_wave_barrier();
