@@ -566,35 +566,42 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
     if (vt + s2 * ppt < ui.v1) step(vt + s2 * ppt, stg[s2]);
 }
 
-// live-slot bitmask of query (bh, i): bit s < S = selected slot s, bit S = own block
-__device__ __forceinline__ unsigned long long live_slots(const SelPlan& P, const void* idx, const uint8_t* fmask, int bh, int i, int lane) {
+// live-slot bitmask of query (bh, i): bit s < S = selected slot s, bit S = own block.  `sub` is the lane's index inside the
+// group of lanes that serves the query (the whole wave, or one half of it when two queries share a wave: half = 0 / 1)
+__device__ __forceinline__ unsigned long long live_slots(const SelPlan& P, const void* idx, const uint8_t* fmask, int bh, int i, int sub, int half, bool two) {
   bool ok = false;
-  if (lane < P.S) {
-    const size_t pos = ((size_t)bh * P.n + i) * P.S + lane;
+  if (sub < P.S) {
+    const size_t pos = ((size_t)bh * P.n + i) * P.S + sub;
     if (fmask[pos]) {
       const int j = read_idx(idx, P.idx64, pos);
       ok = j >= 0 && j < P.W;
     }
-  } else if (lane == P.S) {
+  } else if (sub == P.S) {
     ok = P.causal != 0;
   }
-  return __ballot(ok);
+  const unsigned long long bal = __ballot(ok);
+  return two ? ((bal >> (32 * half)) & 0xffffffffull) : bal;
 }
+
+// Queries per wave of the merge kernels: a query's partial row is G * D / 8 chunks of 16 bytes, one per lane; when that is
+// at most half a wave (d = 64 with G <= 4) and the slots fit 32 mask bits, two queries share a wave instead of idling half of it.
+__host__ __device__ __forceinline__ bool merge_two_per_wave(const SelPlan& P, int cpr) { return P.g * cpr <= 32 && P.SP <= 32; }
 
 // merge the per-slot partials of one query: out = sum_s exp(lse_s - LSE) * o_s
 template <int D>
 __global__ __launch_bounds__(256) void sel_fwd_combine_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, const char* __restrict__ fws,
                                                              __bf16* __restrict__ out, float* __restrict__ lse) {
-  const int lane = threadIdx.x & 63;
-  const long qi = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  constexpr int CPR = D / 8;                    // 16-byte chunks per row
+  const bool two = merge_two_per_wave(P, CPR);
+  const int lane = threadIdx.x & 63, half = two ? lane >> 5 : 0, sub = two ? lane & 31 : lane, width = two ? 32 : 64;
+  const long qi = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * (two ? 2 : 1) + half;
   if (qi >= (long)P.bh * P.n) return;
   const int bh = (int)(qi / P.n), i = (int)(qi % P.n);
   const int b = bh / P.hkv, hk = bh % P.hkv;
-  const unsigned long long live = live_slots(P, idx, fmask, bh, i, lane);
+  const unsigned long long live = live_slots(P, idx, fmask, bh, i, sub, half, two);
   const __bf16* opart = reinterpret_cast<const __bf16*>(fws + P.off_opart);
   const float* lsepart = reinterpret_cast<const float*>(fws + P.off_lsepart);
-  constexpr int CPR = D / 8;                    // 16-byte chunks per row
-  for (int c = lane; c < P.g * CPR; c += 64) {
+  for (int c = sub; c < P.g * CPR; c += width) {
     const int g = c / CPR, dd = (c % CPR) * 8;
     const size_t row0 = ((size_t)bh * P.n + i) * P.SP * P.g + g;
     // one pass, streaming log-sum-exp merge: acc = sum_s exp(lse_s - m) * o_s, rescaled as m grows
@@ -792,17 +799,18 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
 template <int D>
 __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, const char* __restrict__ bws,
                                                                 __bf16* __restrict__ dq, float* __restrict__ sel_grads) {
-  const int lane = threadIdx.x & 63;
-  const long qi = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  constexpr int CPR = D / 8;
+  const bool two = merge_two_per_wave(P, CPR);
+  const int lane = threadIdx.x & 63, half = two ? lane >> 5 : 0, sub = two ? lane & 31 : lane, width = two ? 32 : 64;
+  const long qi = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * (two ? 2 : 1) + half;
   if (qi >= (long)P.bh * P.n) return;
   const int bh = (int)(qi / P.n), i = (int)(qi % P.n);
   const int b = bh / P.hkv, hk = bh % P.hkv;
-  const unsigned long long live = live_slots(P, idx, fmask, bh, i, lane);
+  const unsigned long long live = live_slots(P, idx, fmask, bh, i, sub, half, two);
   // slots the walk never visited carry no gradient
-  if (sel_grads && lane < P.S && !((live >> lane) & 1)) sel_grads[((size_t)bh * P.n + i) * P.S + lane] = 0.f;
+  if (sel_grads && sub < P.S && !((live >> sub) & 1)) sel_grads[((size_t)bh * P.n + i) * P.S + sub] = 0.f;
   const __bf16* dqpart = reinterpret_cast<const __bf16*>(bws + P.off_dqpart);
-  constexpr int CPR = D / 8;
-  for (int c = lane; c < P.g * CPR; c += 64) {
+  for (int c = sub; c < P.g * CPR; c += width) {
     const int g = c / CPR, dd = (c % CPR) * 8;
     const size_t row0 = ((size_t)bh * P.n + i) * P.SP * P.g + g;
     float acc[8];
@@ -1195,8 +1203,8 @@ static int launch_fwd(const SelPlan& P, const void* q, const void* k, const void
                      (const char*)iws, (char*)fws);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 1, st);
-  const long nq = (long)P.bh * P.n;
-  hipLaunchKernelGGL((sel_fwd_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)fws, (__bf16*)out, lse);
+  const long nq = (long)P.bh * P.n, qpb = merge_two_per_wave(P, D / 8) ? 8 : 4;      // queries per work-group of the merge
+  hipLaunchKernelGGL((sel_fwd_combine_kernel<D>), dim3((unsigned)((nq + qpb - 1) / qpb)), dim3(256), 0, st, P, idx, fmask, (const char*)fws, (__bf16*)out, lse);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 2, st);
   return 0;
@@ -1252,8 +1260,8 @@ static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void
   }
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 3, st);
-  const long nq = (long)P.bh * P.n;
-  hipLaunchKernelGGL((sel_bwd_dq_combine_kernel<D>), dim3((unsigned)((nq + 3) / 4)), dim3(256), 0, st, P, idx, fmask, (const char*)bws, (__bf16*)dq, sel_grads);
+  const long nq = (long)P.bh * P.n, qpb = merge_two_per_wave(P, D / 8) ? 8 : 4;
+  hipLaunchKernelGGL((sel_bwd_dq_combine_kernel<D>), dim3((unsigned)((nq + qpb - 1) / qpb)), dim3(256), 0, st, P, idx, fmask, (const char*)bws, (__bf16*)dq, sel_grads);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 4, st);
   hipLaunchKernelGGL((sel_bwd_dkv_reduce_kernel<D, KT>), dim3(P.W, P.bh), dim3(256), 0, st, P, (const char*)iws, (const char*)bws, (__bf16*)dk, (__bf16*)dv);
