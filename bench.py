@@ -230,6 +230,7 @@ def main():
         qc = q.clone().requires_grad_()
         tms = []
         for it in range(3):
+            qc.grad = ck.grad = cv.grad = None      # a step's gradients start from None (no accumulation pass in the timing)
             e0, e1, e2, e3 = (torch.cuda.Event(enable_timing=True) for _ in range(4))
             e0.record()
             c_out, imp = ops.compress_attend(qc, ck, cv, 1, 16, True, sel_block=B, share=True)
