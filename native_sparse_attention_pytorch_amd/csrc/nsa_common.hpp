@@ -132,6 +132,59 @@ __device__ __forceinline__ bf16x8 lds_transposed_operand_swz(const __bf16* X, in
   return __builtin_bit_cast(bf16x8, r);
 }
 
+// A 64-row tile (D bf16 per row) copied from global memory straight into a swizzled LDS tile (the layout read by
+// lds_row_operand_swz / lds_transposed_operand_swz) with global_load_lds_dwordx4: no staging registers and no LDS store
+// instructions.  One instruction of a wave fills 1 KB of consecutive LDS (lane l writes bytes 16 l .. 16 l + 15 after the
+// wave-uniform address in M0), i.e. 1024 / (2 D) whole rows, so the swizzle is applied on the global side: the lane that
+// writes chunk position p of row r fetches chunk (p & ~7) | ((p ^ swz(r)) & 7).  NT threads cover the tile in
+// 64 * D / (8 * NT) rounds; a lane's rows in different rounds differ by a multiple of 8, which leaves its swizzle (and
+// source chunk) alone.  A tile whose 64 rows all exist is addressed as scalar base + one per-lane 32-bit offset that never
+// changes: per tile a few scalar additions and no vector arithmetic (per-lane 64-bit row addresses cost more vector
+// instructions per tile than a quarter of the softmax).  In a tile that crosses `limit`, rows at or beyond it re-read row
+// limit - 1 (finite values; callers mask their scores) through per-lane addresses.
+// The copy is asynchronous: it counts in vmcnt, and the tile may be read after s_waitcnt vmcnt(0) by every wave that
+// issued a part of it plus a work-group barrier.  A wave must not end while a copy it issued is in flight.
+// Inline assembly rather than __builtin_amdgcn_global_load_lds: the compiler makes every later LDS read wait for all the
+// copies it knows of (s_waitcnt vmcnt(0) in front of the first operand read of the tile in use), which serialises the
+// copy of the next tile with the work on this one.
+template <int D, int NT>
+struct TileDma {
+  static constexpr int CPR = D / 8, RPS = 64 / CPR, WAVES = NT / 64, ROUNDS = (64 / RPS) / WAVES;
+  static_assert((WAVES * RPS) % 8 == 0 && ROUNDS >= 1, "a lane's rows must keep their swizzle from round to round");
+  int row_in, src_off;
+  unsigned voff;        // byte offset of this lane's 16 bytes from the first row of a round
+  unsigned lds0;        // LDS byte address of this wave's segment in round 0 (wave-uniform)
+  long s_row;
+  // lds_base: the LDS array the tiles live in; a tile is addressed by its byte offset from it
+  __device__ __forceinline__ void init(int tid, long row_stride, const __bf16* lds_base) {
+    typedef __attribute__((address_space(3))) void* lds_p;
+    const int lane = tid & 63, pos = lane % CPR, wave = tid >> 6;
+    s_row = row_stride;
+    row_in = wave * RPS + lane / CPR;
+    src_off = 8 * ((pos & ~7) | ((pos ^ lds_swz(row_in)) & 7));
+    voff = (unsigned)(row_in * row_stride + src_off) * 2u;
+    lds0 = __builtin_amdgcn_readfirstlane((unsigned)(unsigned long)(lds_p)lds_base + wave * 1024);
+  }
+  // base, first_row, limit and tile_off (bytes from lds_base) must be wave-uniform
+  __device__ __forceinline__ void issue(const __bf16* __restrict__ base, long first_row, long limit, unsigned tile_off) const {
+    if (first_row + 64 <= limit) {
+      const __bf16* tb = base + first_row * s_row;
+#pragma unroll
+      for (int r = 0; r < ROUNDS; ++r)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(voff), "s"(tb + r * WAVES * RPS * s_row) : "memory", "m0");
+    } else {
+#pragma unroll
+      for (int r = 0; r < ROUNDS; ++r) {
+        long row = first_row + row_in + r * WAVES * RPS;
+        row = row < limit ? row : limit - 1;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(base + row * s_row + src_off) : "memory", "m0");
+      }
+    }
+  }
+};
+
 // s_waitcnt vmcnt(0) (expcnt / lgkmcnt left at their maxima): all outstanding global loads
 // and stores of this wave have completed.
 // N operand reads feeding N uses, each read issued AH uses ahead of its own.  The compiler keeps an LDS operand

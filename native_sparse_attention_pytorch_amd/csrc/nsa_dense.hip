@@ -84,16 +84,22 @@ __device__ __forceinline__ TileWalk make_walk(const DensePlan& P, int i_first, i
   return w;
 }
 
+#ifndef NSA_FWD_AHK
+#define NSA_FWD_AHK 3
+#endif
+#ifndef NSA_FWD_AHV
+#define NSA_FWD_AHV 2
+#endif
 // ------------------------------------------------------------------------------- forward
 // NPF = selection block / compress stride when the importance logits are wanted, 0 otherwise
 template <int D, int NPF>
 __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                         const __bf16* __restrict__ v, __bf16* __restrict__ out, float* __restrict__ lse,
                                                         float* __restrict__ pooled) {
-  constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
-  constexpr int RSV = D + 16;       // V is only read through the transpose load: 8 banks per row keep it conflict-free
-  __shared__ __align__(16) __bf16 k_s[kBK * RS];
-  __shared__ __align__(16) __bf16 v_s[kBK * RSV];
+  constexpr int KS = D / 16, DT = D / 32, TILE = kBK * D;
+  // two swizzled tiles each for K and V, filled by asynchronous copies: tile t+1 lands while tile t is being used
+  __shared__ __align__(1024) __bf16 k_s[2 * TILE];
+  __shared__ __align__(1024) __bf16 v_s[2 * TILE];
   constexpr bool POOL = NPF > 0;
   constexpr int NBT = POOL ? kBK / (POOL ? NPF : 1) : 1;        // fine blocks per key tile
   __shared__ float pool_s[POOL ? 4 * 32 * NBT : 1];   // per wave: [rows or queries of the tile][fine blocks of the key tile]
@@ -101,9 +107,10 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
   const int ppt = 32 >> P.lg;                       // queries per wave tile
   // band mode: equal work per tile, neighbouring tiles share most of their window -> one XCD per contiguous range of tiles;
-  // stride mode keeps the round-robin order (causal: work grows with the position, and the compressed keys fit every L2)
+  // stride mode keeps the round-robin order (the compressed keys fit every L2), causal from the last tile down: work grows
+  // with the position, and the longest work-groups should not be the last to start
   const int qtiles = (P.n + 4 * ppt - 1) / (4 * ppt);
-  const int xt = P.mode == 0 ? xcd_contiguous(blockIdx.x, qtiles) : (int)blockIdx.x;
+  const int xt = P.mode == 0 ? xcd_contiguous(blockIdx.x, qtiles) : (P.causal ? qtiles - 1 - (int)blockIdx.x : (int)blockIdx.x);
   if (xt >= qtiles) return;
   const int q0 = xt * 4 * ppt;                      // first query of the work-group
   const int i0 = q0 + wave * ppt;
@@ -133,34 +140,37 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
 
   const __bf16* kbase = k + b * P.sk[0] + hk * P.sk[1];
   const __bf16* vbase = v + b * P.sv[0] + hk * P.sv[1];
-  TileRegs<D, 256> kr, vr;
-  auto load_tile = [&](int t) {
+  TileDma<D, 256> kdma, vdma;
+  kdma.init(tid, P.sk[2], k_s);
+  vdma.init(tid, P.sv[2], v_s);
+  auto load_tile = [&](int t, int into) {
     const long first = t < 0 ? 0 : (long)P.mem + (long)t * kBK;
     const long limit = t < 0 ? P.mem : (long)P.mem + P.nkeys;
-    kr.load(kbase, P.sk[2], first, limit, tid);
-    vr.load(vbase, P.sv[2], first, limit, tid);
+    kdma.issue(kbase, first, limit, into * TILE * 2);
+    vdma.issue(vbase, first, limit, into * TILE * 2);
   };
-  int t = walk.t_first;
-  if (t <= walk.t_hi || t < 0) load_tile(t);
+  int t = walk.t_first, buf = 0;
+  if (t <= walk.t_hi || t < 0) load_tile(t, 0);      // (a memory tile is always walked: every copy issued is waited for)
 
-  for (; t <= walk.t_hi; t = walk.next(t)) {
-    kr.commit(k_s, RS, tid);
-    vr.commit(v_s, RSV, tid);
+  for (; t <= walk.t_hi; t = walk.next(t), buf ^= 1) {
+    // one barrier per tile: behind it this wave's and every other wave's part of tile t has landed, and all waves are done
+    // with tile t-1, whose buffer the copy of tile t+1 may now overwrite
+    wait_all_loads();
     __syncthreads();
     const int tn = walk.next(t);
-    if (tn <= walk.t_hi) load_tile(tn);
+    if (tn <= walk.t_hi) load_tile(tn, buf ^ 1);
+    const __bf16* kt_s = k_s + buf * TILE;
+    const __bf16* vt_s = v_s + buf * TILE;
     const bool memtile = t < 0;
     const int kb0 = memtile ? 0 : t * kBK;
     // skip tiles outside this wave's reach (the barriers below are still executed)
     const bool active = memtile || (kb0 <= my_hi && kb0 + kBK - 1 >= my_lo);
     if (active) {
       floatx16 Sa[2];
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-        Sa[kt] = zero_acc();
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) Sa[kt] = mfma32(lds_row_operand(k_s + 32 * kt * RS, RS, ks, lane), Qf[ks], Sa[kt]);
-      }
+      Sa[0] = zero_acc();
+      Sa[1] = zero_acc();
+      operands_ahead<2 * KS, NSA_FWD_AHK>([&](int i2) { return lds_row_operand_swz<D>(kt_s + 32 * (i2 / KS) * D, i2 % KS, lane); },
+                                          [&](int i2, bf16x8 a) { Sa[i2 / KS] = mfma32(a, Qf[i2 % KS], Sa[i2 / KS]); });
       const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
       floatx16 Sraw[2];
       if (POOL) { Sraw[0] = Sa[0]; Sraw[1] = Sa[1]; }
@@ -171,7 +181,8 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
 #pragma unroll
           for (int i2 = 0; i2 < 16; ++i2) {
             const int key = kb0 + 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
-            const float s = (!decltype(masked)::value || (key >= klo && key <= khi)) ? Sa[kt][i2] * sc : -INFINITY;
+            // raw scores: the (positive) scale is folded into the exponent's multiply-add below, the maximum is taken raw
+            const float s = (!decltype(masked)::value || ((key >= klo) & (key <= khi))) ? Sa[kt][i2] : -INFINITY;
             Sa[kt][i2] = s;
             tmax = fmaxf(tmax, s);
           }
@@ -258,14 +269,14 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
 
       tmax = fmaxf(tmax, xor32(tmax));
       const float mnew = fmaxf(m, tmax);
-      const float mref = (mnew == -INFINITY) ? 0.f : mnew;
-      const float alpha = fast_exp2(m - mref);
+      const float mref = (mnew == -INFINITY) ? 0.f : mnew * sc;      // m, mnew: raw maxima; mref in the exponent's units
+      const float alpha = fast_exp2(__builtin_fmaf(m, sc, -mref));
       float rs = 0.f;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int i2 = 0; i2 < 16; ++i2) {
-          const float p = fast_exp2(Sa[kt][i2] - mref);
+          const float p = fast_exp2(__builtin_fmaf(Sa[kt][i2], sc, -mref));
           Sa[kt][i2] = p;
           rs += p;
         }
@@ -276,17 +287,12 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) Oa[dt][e] *= alpha;
+      bf16x8 Pf[4];
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int u2 = 0; u2 < 2; ++u2) {
-          const bf16x8 Pf = pack8(Sa[kt], 8 * u2);
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-            Oa[dt] = mfma32(lds_transposed_operand(v_s, RSV, 32 * kt + 16 * u2, 32 * dt, lane), Pf, Oa[dt]);
-        }
+      for (int c = 0; c < 4; ++c) Pf[c] = pack8(Sa[c >> 1], 8 * (c & 1));
+      operands_ahead<4 * DT, NSA_FWD_AHV>([&](int i2) { return lds_transposed_operand_swz<D>(vt_s, 16 * (i2 / DT), 32 * (i2 % DT), lane); },
+                                          [&](int i2, bf16x8 a) { Oa[i2 % DT] = mfma32(a, Pf[i2 / DT], Oa[i2 % DT]); });
     }
-    __syncthreads();
   }
 
   if (POOL) {
@@ -318,7 +324,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
 #pragma unroll
       for (int a = 0; a < 4; ++a)
         store4_bf16(op + 32 * dt + 8 * a, Oa[dt][4 * a] * inv, Oa[dt][4 * a + 1] * inv, Oa[dt][4 * a + 2] * inv, Oa[dt][4 * a + 3] * inv);
-    if (h == 0) lse[((long)b * P.hkv * P.g + hq) * P.n + i] = (m + fast_log2(l)) * kLn2;
+    if (h == 0) lse[((long)b * P.hkv * P.g + hq) * P.n + i] = (m * sc + fast_log2(l)) * kLn2;
   }
 }
 
