@@ -213,7 +213,24 @@ __device__ __forceinline__ void wait_all_loads() {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+// Maximum / sum of a value over the two 32-lane halves of the wave (lane l with lane l ^ 32), left in both halves.
+// v_permlane32_swap exchanges the upper half of one register with the lower half of another inside the VALU; the shuffle
+// it replaces (ds_bpermute) is an LDS round trip on the critical path of every tile's softmax.  Inline assembly: the
+// builtin with the same value for both operands is folded away by the compiler as if the swap did nothing.  The s_nop
+// on either side covers the wait states between a VALU write and the swap's read, and the swap's write and a VALU read.
+__device__ __forceinline__ void swap_halves(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float halves_max(float v) {
+  float a = v, b = v;
+  swap_halves(a, b);      // a = lower half's values in both halves, b = upper half's
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float halves_sum(float v) {
+  float a = v, b = v;
+  swap_halves(a, b);
+  return a + b;
+}
 
 // value of lane ^ 1 / lane ^ 2 (DPP quad permutes: VALU speed, no LDS round trip)
 __device__ __forceinline__ float dpp_quad_xor1(float v) {

@@ -212,7 +212,7 @@ __device__ __forceinline__ void decode_attend_body(const AttendArgs& A, const in
       Sa[i] = s;
       mx = fmaxf(mx, s);
     }
-    mx = fmaxf(mx, xor32(mx));
+    mx = halves_max(mx);
     const float mn = fmaxf(m, mx);
     const float alpha = fast_exp2(m - mn);
     float ls = 0.f;
@@ -235,7 +235,7 @@ __device__ __forceinline__ void decode_attend_body(const AttendArgs& A, const in
     t = tn;
     T = Tn;
   }
-  l += xor32(l);
+  l = halves_sum(l);
 
   // partial record of this wave: [gc][D] O, [gc] max, [gc] sum
   if (n_ < P.gc) {

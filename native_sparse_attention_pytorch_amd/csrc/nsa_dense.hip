@@ -207,7 +207,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
             for (int a = 0; a < 4; ++a) grp[a] = (Sraw[kt][4 * a] + Sraw[kt][4 * a + 1]) + (Sraw[kt][4 * a + 2] + Sraw[kt][4 * a + 3]);
             if (npf >= 8) {
 #pragma unroll
-              for (int a = 0; a < 4; ++a) grp[a] += xor32(grp[a]);
+              for (int a = 0; a < 4; ++a) grp[a] = halves_sum(grp[a]);
             }
             if (npf == 16) { grp[0] += grp[1]; grp[2] += grp[3]; }
             if (npf == 32) { grp[0] = (grp[0] + grp[1]) + (grp[2] + grp[3]); }
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
         __builtin_amdgcn_wave_barrier();
       }
 
-      tmax = fmaxf(tmax, xor32(tmax));
+      tmax = halves_max(tmax);
       const float mnew = fmaxf(m, tmax);
       const float mref = (mnew == -INFINITY) ? 0.f : mnew * sc;      // m, mnew: raw maxima; mref in the exponent's units
       const float alpha = fast_exp2(__builtin_fmaf(m, sc, -mref));
@@ -280,8 +280,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
           Sa[kt][i2] = p;
           rs += p;
         }
-      rs += xor32(rs);
-      l = l * alpha + rs;
+      l = l * alpha + rs;       // this lane's half of the keys: the halves are added once, after the walk
       m = mnew;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
@@ -316,6 +315,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
     }
   }
 
+  l = halves_sum(l);
   if (valid) {
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     __bf16* op = out + b * P.so[0] + (long)hq * P.so[1] + (long)i * P.so[2] + 4 * h;

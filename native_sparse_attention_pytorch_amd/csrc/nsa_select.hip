@@ -511,7 +511,7 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int i2 = 0; i2 < 16; ++i2) mx = fmaxf(mx, Sa[kt][i2]);
-    mx = fmaxf(mx, xor32(mx));
+    mx = halves_max(mx);
     const float mxs = mx * sc;                       // the row maximum in the exponent's units (log2)
     float l = 0.f;
 #pragma unroll
@@ -522,7 +522,7 @@ __global__ __launch_bounds__(64) void sel_fwd_kernel(const SelPlan P, const __bf
         Sa[kt][i2] = p;
         l += p;
       }
-    l += xor32(l);
+    l = halves_sum(l);
     // normalise the probabilities (32 values) rather than the output tile (64)
     const float inv = 1.0f / l;
 #pragma unroll
@@ -772,7 +772,7 @@ __global__ __launch_bounds__(64) void sel_bwd_dq_kernel(const SelPlan P, const _
         if (GATE) gs += ds * sraw;
       }
     if (GATE) {
-      gs += xor32(gs);
+      gs = halves_sum(gs);
       for (int mk = 1; mk < P.g; mk <<= 1) gs += __shfl_xor(gs, mk, 64);      // the G heads of a pair are adjacent lanes
       if (r.valid && r.g == 0 && h == 0 && r.slot < P.S) sel_grads[((size_t)bh * P.n + r.i) * P.S + r.slot] = gs * P.scale;
     }
