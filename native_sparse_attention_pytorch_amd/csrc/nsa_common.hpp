@@ -165,14 +165,18 @@ struct TileDma {
     voff = (unsigned)(row_in * row_stride + src_off) * 2u;
     lds0 = __builtin_amdgcn_readfirstlane((unsigned)(unsigned long)(lds_p)lds_base + wave * 1024);
   }
+  // One round (1 KB per wave) of a tile whose 64 rows all exist; tb = address of the tile's first row.  Issuing a copy
+  // keeps the wave's instruction stream busy for some 60 cycles; callers with MFMAs to issue put the rounds between them.
+  __device__ __forceinline__ void round_full(const __bf16* __restrict__ tb, unsigned tile_off, int r) const {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(voff), "s"(tb + r * WAVES * RPS * s_row) : "memory", "m0");
+  }
   // base, first_row, limit and tile_off (bytes from lds_base) must be wave-uniform
   __device__ __forceinline__ void issue(const __bf16* __restrict__ base, long first_row, long limit, unsigned tile_off) const {
     if (first_row + 64 <= limit) {
       const __bf16* tb = base + first_row * s_row;
 #pragma unroll
-      for (int r = 0; r < ROUNDS; ++r)
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                     :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(voff), "s"(tb + r * WAVES * RPS * s_row) : "memory", "m0");
+      for (int r = 0; r < ROUNDS; ++r) round_full(tb, tile_off, r);
     } else {
 #pragma unroll
       for (int r = 0; r < ROUNDS; ++r) {

@@ -158,19 +158,41 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
     wait_all_loads();
     __syncthreads();
     const int tn = walk.next(t);
-    if (tn <= walk.t_hi) load_tile(tn, buf ^ 1);
+    // The copy of the next tile: between the MFMAs of this tile's scores where it can be (a copy instruction holds the
+    // wave's issue for about as long as two MFMAs run), up front for a tile that needs the clamped path or a wave with no
+    // scores to compute
+    const long nfirst = (long)P.mem + (long)tn * kBK;                    // (the memory tile is never a next tile)
+    const bool more = tn <= walk.t_hi, spread = more && nfirst + kBK <= (long)P.mem + P.nkeys;
+    const __bf16* ktb = kbase + nfirst * P.sk[2];
+    const __bf16* vtb = vbase + nfirst * P.sv[2];
+    const unsigned noff = (buf ^ 1) * TILE * 2;
     const __bf16* kt_s = k_s + buf * TILE;
     const __bf16* vt_s = v_s + buf * TILE;
     const bool memtile = t < 0;
     const int kb0 = memtile ? 0 : t * kBK;
     // skip tiles outside this wave's reach (the barriers below are still executed)
     const bool active = memtile || (kb0 <= my_hi && kb0 + kBK - 1 >= my_lo);
+    if (!active || !spread) {
+      if (more) load_tile(tn, buf ^ 1);
+    }
     if (active) {
       floatx16 Sa[2];
       Sa[0] = zero_acc();
       Sa[1] = zero_acc();
-      operands_ahead<2 * KS, NSA_FWD_AHK>([&](int i2) { return lds_row_operand_swz<D>(kt_s + 32 * (i2 / KS) * D, i2 % KS, lane); },
-                                          [&](int i2, bf16x8 a) { Sa[i2 / KS] = mfma32(a, Qf[i2 % KS], Sa[i2 / KS]); });
+      auto scores = [&](auto copying) {
+        constexpr int RN = TileDma<D, 256>::ROUNDS;
+        static_assert(2 * RN <= KS, "one copy round after every second MFMA");
+        operands_ahead<2 * KS, NSA_FWD_AHK>([&](int i2) { return lds_row_operand_swz<D>(kt_s + 32 * (i2 / KS) * D, i2 % KS, lane); },
+                                            [&](int i2, bf16x8 a) {
+                                              Sa[i2 / KS] = mfma32(a, Qf[i2 % KS], Sa[i2 / KS]);
+                                              if (decltype(copying)::value && (i2 & 1) && (i2 >> 1) < 2 * RN) {
+                                                if ((i2 >> 1) < RN) kdma.round_full(ktb, noff, i2 >> 1);
+                                                else vdma.round_full(vtb, noff, (i2 >> 1) - RN);
+                                              }
+                                            });
+      };
+      if (spread) scores(std::true_type{});
+      else scores(std::false_type{});
       const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
       floatx16 Sraw[2];
       if (POOL) { Sraw[0] = Sa[0]; Sraw[1] = Sa[1]; }
@@ -268,9 +290,24 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
       }
 
       tmax = halves_max(tmax);
-      const float mnew = fmaxf(m, tmax);
-      const float mref = (mnew == -INFINITY) ? 0.f : mnew * sc;      // m, mnew: raw maxima; mref in the exponent's units
-      const float alpha = fast_exp2(__builtin_fmaf(m, sc, -mref));
+      // The reference maximum m of a row (raw units) follows the running maximum only when that has grown by more than
+      // kSlack in the exponent's units: until then the probabilities are taken against the stale reference (at most
+      // 2^kSlack, exact in fp32 and with the same relative rounding in bf16) and nothing needs rescaling.  Softmax is
+      // invariant to the reference, so the result is the same function; what goes away is the multiplication of the
+      // whole accumulator tile by factors that are 1 or close to it in nearly every tile.  One wave-uniform test.
+      // (m = -inf, tmax finite: the difference is +inf and the row moves; both -inf: NaN compares false, nothing to do)
+      constexpr float kSlack = 8.f;
+      if (__any((tmax - m) * sc > kSlack)) {
+        const float mnew = fmaxf(m, tmax);
+        const float alpha = fast_exp2((mnew == -INFINITY) ? 0.f : (m - mnew) * sc);
+        m = mnew;
+        l *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) Oa[dt][e] *= alpha;
+      }
+      const float mref = (m == -INFINITY) ? 0.f : m * sc;
       float rs = 0.f;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
@@ -280,12 +317,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
           Sa[kt][i2] = p;
           rs += p;
         }
-      l = l * alpha + rs;       // this lane's half of the keys: the halves are added once, after the walk
-      m = mnew;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) Oa[dt][e] *= alpha;
+      l += rs;                  // this lane's half of the keys: the halves are added once, after the walk
       bf16x8 Pf[4];
 #pragma unroll
       for (int c = 0; c < 4; ++c) Pf[c] = pack8(Sa[c >> 1], 8 * (c & 1));
