@@ -213,80 +213,88 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
       else scale_scores(std::true_type{});
 
       if (POOL && !memtile) {
-        // Block-importance logits of this 64-key tile: sum the raw scaled logits over the npf keys
-        // of a fine block (in registers / one exchange between the lane halves) and over the G
-        // heads of the group (adjacent lanes: DPP quad permutes for G <= 4), stage the sums in
-        // LDS and write them with coalesced stores; visibility is index arithmetic at store time.
-        constexpr int npf = POOL ? NPF : 1, nbt = NBT;
-        float* pw = pool_s + wave * (32 * nbt);
+        // Block-importance logits of this 64-key tile: sum the raw logits over the npf keys of a fine block (in registers /
+        // one exchange between the lane halves) and over the G heads of the group (adjacent lanes: DPP quad permutes for
+        // G <= 4), stage the sums in LDS and write them with coalesced stores; visibility is index arithmetic at store time.
+        // One straight-line variant per way of summing heads, chosen by one wave-uniform switch per tile: with the choice
+        // made value by value inside, the compiler threaded a dozen scalar branches through every half tile.
+        // HS = 0: one row per head (no sharing, or groups of one head); 2 / 4: shared, group of 2 / 4; 1: shared, any other
+        auto pool = [&](auto hs) {
+          constexpr int HS = decltype(hs)::value;
+          constexpr bool SH = HS != 0;
+          constexpr int npf = POOL ? NPF : 1, nbt = NBT;
+          float* pw = pool_s + wave * (32 * nbt);
+          const int prow_local = SH ? pq : n_;           // query inside the wave tile (shared) or row of the wave tile (per head)
+          const bool mine = (npf < 8 || h == 0) && (!SH || g == 0);
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-          float grp[4];
+          for (int kt = 0; kt < 2; ++kt) {
+            float grp[4];
 #pragma unroll
-          for (int a = 0; a < 4; ++a) grp[a] = 0.f;
-          if (npf >= 4) {
+            for (int a = 0; a < 4; ++a) grp[a] = 0.f;
+            if (npf >= 4) {
 #pragma unroll
-            for (int a = 0; a < 4; ++a) grp[a] = (Sraw[kt][4 * a] + Sraw[kt][4 * a + 1]) + (Sraw[kt][4 * a + 2] + Sraw[kt][4 * a + 3]);
-            if (npf >= 8) {
+              for (int a = 0; a < 4; ++a) grp[a] = (Sraw[kt][4 * a] + Sraw[kt][4 * a + 1]) + (Sraw[kt][4 * a + 2] + Sraw[kt][4 * a + 3]);
+              if (npf >= 8) {
 #pragma unroll
-              for (int a = 0; a < 4; ++a) grp[a] = halves_sum(grp[a]);
+                for (int a = 0; a < 4; ++a) grp[a] = halves_sum(grp[a]);
+              }
+              if (npf == 16) { grp[0] += grp[1]; grp[2] += grp[3]; }
+              if (npf == 32) { grp[0] = (grp[0] + grp[1]) + (grp[2] + grp[3]); }
             }
-            if (npf == 16) { grp[0] += grp[1]; grp[2] += grp[3]; }
-            if (npf == 32) { grp[0] = (grp[0] + grp[1]) + (grp[2] + grp[3]); }
-          }
-          // the distinct sums of this 32-key half, then the head sums for all of them under one (wave-uniform) decision and
-          // all LDS stores under one predicate: taken value by value, each value carried its own cascade of branches
-          constexpr int NV = npf == 1 ? 16 : npf == 2 ? 8 : npf <= 8 ? 4 : npf == 16 ? 2 : 1;
-          float val[NV];
-          int koff[NV];
+            // the distinct sums of this 32-key half
+            constexpr int NV = npf == 1 ? 16 : npf == 2 ? 8 : npf <= 8 ? 4 : npf == 16 ? 2 : 1;
+            float val[NV];
+            int koff[NV];
 #pragma unroll
-          for (int vi = 0; vi < NV; ++vi) {
-            if (npf == 1) { val[vi] = Sraw[kt][vi]; koff[vi] = 8 * (vi >> 2) + 4 * h + (vi & 3); }
-            else if (npf == 2) { val[vi] = Sraw[kt][2 * vi] + Sraw[kt][2 * vi + 1]; koff[vi] = 8 * (vi >> 1) + 4 * h + 2 * (vi & 1); }
-            else if (npf == 4) { val[vi] = grp[vi]; koff[vi] = 8 * vi + 4 * h; }
-            else if (npf == 8) { val[vi] = grp[vi]; koff[vi] = 8 * vi; }
-            else if (npf == 16) { val[vi] = grp[2 * vi]; koff[vi] = 16 * vi; }
-            else { val[vi] = grp[0]; koff[vi] = 0; }
-          }
-          bool mine = npf < 8 || h == 0;
-          int prow_local = n_;                           // row inside the wave tile (per head) ...
-          if (P.share) {
-            if (P.g == 2) {
+            for (int vi = 0; vi < NV; ++vi) {
+              if (npf == 1) { val[vi] = Sraw[kt][vi]; koff[vi] = 8 * (vi >> 2) + 4 * h + (vi & 3); }
+              else if (npf == 2) { val[vi] = Sraw[kt][2 * vi] + Sraw[kt][2 * vi + 1]; koff[vi] = 8 * (vi >> 1) + 4 * h + 2 * (vi & 1); }
+              else if (npf == 4) { val[vi] = grp[vi]; koff[vi] = 8 * vi + 4 * h; }
+              else if (npf == 8) { val[vi] = grp[vi]; koff[vi] = 8 * vi; }
+              else if (npf == 16) { val[vi] = grp[2 * vi]; koff[vi] = 16 * vi; }
+              else { val[vi] = grp[0]; koff[vi] = 0; }
+            }
+            if (HS == 2 || HS == 4) {
 #pragma unroll
               for (int vi = 0; vi < NV; ++vi) val[vi] += dpp_quad_xor1(val[vi]);
-            } else if (P.g == 4) {
+            }
+            if (HS == 4) {
 #pragma unroll
-              for (int vi = 0; vi < NV; ++vi) { val[vi] += dpp_quad_xor1(val[vi]); val[vi] += dpp_quad_xor2(val[vi]); }
-            } else {
+              for (int vi = 0; vi < NV; ++vi) val[vi] += dpp_quad_xor2(val[vi]);
+            }
+            if (HS == 1) {
               for (int mk = 1; mk < P.g; mk <<= 1) {
 #pragma unroll
                 for (int vi = 0; vi < NV; ++vi) val[vi] += __shfl_xor(val[vi], mk, 64);
               }
             }
-            prow_local = pq;                             // ... or query inside the wave tile (shared)
-            mine = mine && g == 0;
-          }
-          if (mine) {
+            if (mine) {
 #pragma unroll
-            for (int vi = 0; vi < NV; ++vi) pw[prow_local * nbt + (32 * kt + koff[vi]) / npf] = val[vi];
+              for (int vi = 0; vi < NV; ++vi) pw[prow_local * nbt + (32 * kt + koff[vi]) / npf] = val[vi];
+            }
           }
-        }
-        __builtin_amdgcn_wave_barrier();
-        const int rows_here = P.share ? ppt : 32;
-        const float norm = P.scale / (float)(npf * (P.share ? P.g : 1));
-        for (int e = lane; e < rows_here * nbt; e += 64) {
-          const int rr = e / nbt, jj = e % nbt;
-          const int qi = i0 + (P.share ? rr : (rr >> P.lg));
-          const int jblk = (kb0 / npf) + jj;
-          if (qi < P.n && jblk < P.nb) {
+          __builtin_amdgcn_wave_barrier();
+          const int rows_here = SH ? ppt : 32;
+          const float norm = P.scale / (float)(npf * (SH ? P.g : 1));
+          const int jb0 = kb0 / npf;
+          for (int e = lane; e < rows_here * nbt; e += 64) {
+            const int rr = e / nbt, jj = e % nbt;
+            const int qi = i0 + (SH ? rr : (rr >> P.lg));
+            const int jblk = jb0 + jj;
+            const float sum = pw[e];
             // all npf keys of the block visible: (jblk+1)*npf - 1 <= qi/st - 1  <=>  (jblk+1)*B <= qi
-            const bool own = (long)jblk * P.B <= qi && qi < (long)(jblk + 1) * P.B;
-            const bool vis = (!P.causal || (long)(jblk + 1) * P.B <= qi) && !(P.mask_own && own);
-            const long prow = P.share ? ((long)bh * P.n + qi) : (((long)b * P.hkv * P.g + hk * P.g + (rr & (P.g - 1))) * P.n + qi);
-            pooled[prow * P.nb + jblk] = vis ? pw[rr * nbt + jj] * norm : -INFINITY;
+            const int blo = jblk * P.B, bhi = blo + P.B;
+            const bool own = (blo <= qi) & (qi < bhi);
+            const bool vis = (!P.causal | (bhi <= qi)) & !(P.mask_own & own);
+            const long head = SH ? (long)bh : (long)bh * P.g + (rr & (P.g - 1));
+            if ((qi < P.n) & (jblk < P.nb)) pooled[(head * P.n + qi) * P.nb + jblk] = vis ? sum * norm : -INFINITY;
           }
-        }
-        __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_wave_barrier();
+        };
+        if (!P.share || P.g == 1) pool(std::integral_constant<int, 0>{});
+        else if (P.g == 4) pool(std::integral_constant<int, 4>{});
+        else if (P.g == 2) pool(std::integral_constant<int, 2>{});
+        else pool(std::integral_constant<int, 1>{});
       }
 
       tmax = halves_max(tmax);
