@@ -171,6 +171,15 @@ struct TileDma {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(voff), "s"(tb + r * WAVES * RPS * s_row) : "memory", "m0");
   }
+  // The same under an execution mask (all ones: copy; zero: no lane takes part, nothing is read or written and tb may point
+  // anywhere): lets a caller keep one straight-line instruction stream whether or not there is a tile to copy.
+  // `lanes` is all ones or zero (32 bits, used for both halves of the mask) and wave-uniform.
+  __device__ __forceinline__ void round_full_if(unsigned lanes, const __bf16* __restrict__ tb, unsigned tile_off, int r) const {
+    asm volatile("s_mov_b32 m0, %0\n\ts_mov_b64 vcc, exec\n\ts_mov_b32 exec_lo, %3\n\ts_mov_b32 exec_hi, %3\n\t"
+                 "global_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, vcc"
+                 :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(voff), "s"(tb + r * WAVES * RPS * s_row),
+                    "s"(__builtin_amdgcn_readfirstlane(lanes)) : "memory", "m0", "vcc");
+  }
   // base, first_row, limit and tile_off (bytes from lds_base) must be wave-uniform
   __device__ __forceinline__ void issue(const __bf16* __restrict__ base, long first_row, long limit, unsigned tile_off) const {
     if (first_row + 64 <= limit) {
@@ -178,9 +187,13 @@ struct TileDma {
 #pragma unroll
       for (int r = 0; r < ROUNDS; ++r) round_full(tb, tile_off, r);
     } else {
+      // (the lane's row passes through an empty volatile statement: this path runs once or twice per work-group, and without
+      // the fence the compiler keeps every round's loop-invariant address terms in registers for the whole walk)
+      int ri = row_in;
+      asm volatile("" : "+v"(ri));
 #pragma unroll
       for (int r = 0; r < ROUNDS; ++r) {
-        long row = first_row + row_in + r * WAVES * RPS;
+        long row = first_row + ri + r * WAVES * RPS;
         row = row < limit ? row : limit - 1;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                      :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(base + row * s_row + src_off) : "memory", "m0");

@@ -84,6 +84,12 @@ __device__ __forceinline__ TileWalk make_walk(const DensePlan& P, int i_first, i
   return w;
 }
 
+#ifndef NSA_DQ_AHK
+#define NSA_DQ_AHK 3
+#endif
+#ifndef NSA_DQ_AHT
+#define NSA_DQ_AHT 1
+#endif
 #ifndef NSA_FWD_AHK
 #define NSA_FWD_AHK 3
 #endif
@@ -191,6 +197,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
                                               }
                                             });
       };
+      // (two copies of the score products rather than copies under an execution mask: measured faster where the registers allow it)
       if (spread) scores(std::true_type{});
       else scores(std::false_type{});
       const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
@@ -397,9 +404,10 @@ template <int D>
 __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                            const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
                                                            const float* __restrict__ lse, const float* __restrict__ delta, __bf16* __restrict__ dq) {
-  constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
-  __shared__ __align__(16) __bf16 k_s[kBK * RS];
-  __shared__ __align__(16) __bf16 v_s[kBK * RS];
+  constexpr int KS = D / 16, DT = D / 32, TILE = kBK * D;
+  // as in the forward kernel: two swizzled tiles each for K and V, filled by asynchronous copies, one barrier per tile
+  __shared__ __align__(1024) __bf16 k_s[2 * TILE];
+  __shared__ __align__(1024) __bf16 v_s[2 * TILE];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
   const int ppt = 32 >> P.lg;
@@ -433,58 +441,74 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P,
 
   const __bf16* kbase = k + b * P.sk[0] + hk * P.sk[1];
   const __bf16* vbase = v + b * P.sv[0] + hk * P.sv[1];
-  TileRegs<D, 256> kr, vr;
-  auto load_tile = [&](int t) {
+  TileDma<D, 256> kdma, vdma;
+  kdma.init(tid, P.sk[2], k_s);
+  vdma.init(tid, P.sv[2], v_s);
+  auto load_tile = [&](int t, int into) {
     const long first = t < 0 ? 0 : (long)P.mem + (long)t * kBK;
     const long limit = t < 0 ? P.mem : (long)P.mem + P.nkeys;
-    kr.load(kbase, P.sk[2], first, limit, tid);
-    vr.load(vbase, P.sv[2], first, limit, tid);
+    kdma.issue(kbase, first, limit, into * TILE * 2);
+    vdma.issue(vbase, first, limit, into * TILE * 2);
   };
-  int t = walk.t_first;
-  if (t <= walk.t_hi || t < 0) load_tile(t);
+  int t = walk.t_first, buf = 0;
+  if (t <= walk.t_hi || t < 0) load_tile(t, 0);
 
-  for (; t <= walk.t_hi; t = walk.next(t)) {
-    kr.commit(k_s, RS, tid);
-    vr.commit(v_s, RS, tid);
+  for (; t <= walk.t_hi; t = walk.next(t), buf ^= 1) {
+    wait_all_loads();
     __syncthreads();
     const int tn = walk.next(t);
-    if (tn <= walk.t_hi) load_tile(tn);
+    // the copy of the next tile goes between the S / dP MFMAs where it can (see the forward kernel)
+    const long nfirst = (long)P.mem + (long)tn * kBK;
+    const bool more = tn <= walk.t_hi, spread = more && nfirst + kBK <= (long)P.mem + P.nkeys;
+    const __bf16* ktb = kbase + nfirst * P.sk[2];
+    const __bf16* vtb = vbase + nfirst * P.sv[2];
+    const unsigned noff = (buf ^ 1) * TILE * 2;
+    const __bf16* kt_s = k_s + buf * TILE;
+    const __bf16* vt_s = v_s + buf * TILE;
     const bool memtile = t < 0;
     const int kb0 = memtile ? 0 : t * kBK;
     const bool active = memtile || (kb0 <= my_hi && kb0 + kBK - 1 >= my_lo);
+    if (!active || !spread) {
+      if (more) load_tile(tn, buf ^ 1);
+    }
+    const unsigned lanes = spread ? ~0u : 0u;
     auto tile_math = [&](auto masked) {
-      floatx16 Sa[2], Pa[2];
+      constexpr int RN = TileDma<D, 256>::ROUNDS;
+      static_assert(2 * RN <= KS, "one copy round after every fourth MFMA");
+      // one 32-key half at a time: S and dP (2 KS MFMAs), then dS of that half on the VALU - independent of the other
+      // half's MFMAs, which the scheduler may run beside it - and 8 registers of packed dS instead of 32 of S and dP
+      const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
+      bf16x8 Sf[4];
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
-        Sa[kt] = zero_acc(); Pa[kt] = zero_acc();
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          Sa[kt] = mfma32(lds_row_operand(k_s + 32 * kt * RS, RS, ks, lane), Qf[ks], Sa[kt]);
-          Pa[kt] = mfma32(lds_row_operand(v_s + 32 * kt * RS, RS, ks, lane), Gf[ks], Pa[kt]);
-        }
-      }
-      const int klo = memtile ? 0 : me.lo, khi = memtile ? P.mem - 1 : me.hi;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+        floatx16 Sa = zero_acc(), Pa = zero_acc();
+        // operand i: k-step i / 2, even i from K (scores), odd i from V (dP)
+        operands_ahead<2 * KS, NSA_DQ_AHK>(
+            [&](int i2) { return lds_row_operand_swz<D>(((i2 & 1) ? vt_s : kt_s) + 32 * kt * D, i2 >> 1, lane); },
+            [&](int i2, bf16x8 a) {
+              if (i2 & 1) Pa = mfma32(a, Gf[i2 >> 1], Pa);
+              else Sa = mfma32(a, Qf[i2 >> 1], Sa);
+              const int c = (kt * 2 * KS + i2) >> 2;      // a copy round after every fourth MFMA of the tile
+              if ((i2 & 3) == 3 && c < 2 * RN) {
+                if (c < RN) kdma.round_full_if(lanes, ktb, noff, c);
+                else vdma.round_full_if(lanes, vtb, noff, c - RN);
+              }
+            });
 #pragma unroll
         for (int i2 = 0; i2 < 16; ++i2) {
           const int key = kb0 + 32 * kt + 8 * (i2 >> 2) + 4 * h + (i2 & 3);
           // the mask goes into the exponent (exp2(-inf) = 0, '&' instead of '&&'): a select around the exponential is compiled
           // as a branch per element
-          float x = __builtin_fmaf(Sa[kt][i2], sc, -lse_r);
+          float x = __builtin_fmaf(Sa[i2], sc, -lse_r);
           if (decltype(masked)::value) x = ((key >= klo) & (key <= khi)) ? x : -INFINITY;
           const float p = fast_exp2(x);
-          Sa[kt][i2] = p * (Pa[kt][i2] - del_r);
+          Sa[i2] = p * (Pa[i2] - del_r);
         }
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int u2 = 0; u2 < 2; ++u2) {
-          const bf16x8 Sf = pack8(Sa[kt], 8 * u2);
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-            Qa[dt] = mfma32(lds_transposed_operand(k_s, RS, 32 * kt + 16 * u2, 32 * dt, lane), Sf, Qa[dt]);
-        }
+        Sf[2 * kt] = pack8(Sa, 0);
+        Sf[2 * kt + 1] = pack8(Sa, 8);
+      }
+      operands_ahead<4 * DT, NSA_DQ_AHT>([&](int i2) { return lds_transposed_operand_swz<D>(kt_s, 16 * (i2 / DT), 32 * (i2 % DT), lane); },
+                                         [&](int i2, bf16x8 a) { Qa[i2 % DT] = mfma32(a, Sf[i2 / DT], Qa[i2 % DT]); });
     };
     if (active) {
       // a tile every row of the wave sees completely needs no per-element mask (wave-uniform); each
@@ -492,7 +516,6 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P,
       if (!memtile && kb0 >= all_lo && kb0 + kBK - 1 <= all_hi) tile_math(std::false_type{});
       else tile_math(std::true_type{});
     }
-    __syncthreads();
   }
   if (valid) {
     __bf16* op = dq + srow * D + 4 * h;
