@@ -29,6 +29,7 @@ SLIDING = [
     (1, 6, 2, 200, 64, 32, True),         # G=3: not a power of two (padded with zero heads)
     (1, 4, 2, 150, 32, 20, True),         # dim_head 32 (zero-padded to 64)
     (1, 2, 1, 150, 96, 20, False),        # dim_head 96 (-> 128)
+    (1, 4, 2, 500, 128, 70, False),       # d 128, window on both sides, several key tiles, the last one partial
 ]
 
 
@@ -69,6 +70,8 @@ COMPRESS = [
     (1, 12, 2, 100, 64, 4, 20, 1, True, True),       # G=6 with npf 5
     (1, 4, 2, 200, 32, 4, 16, 1, True, True),        # dim_head 32
     (1, 4, 2, 200, 96, 8, 16, 2, True, False),       # dim_head 96
+    (1, 8, 2, 2100, 128, 8, 32, 2, True, True),      # d 128, 262 compressed keys + 2 slots: full tiles, a partial last tile, npf 4
+    (1, 4, 2, 1100, 128, 4, 16, 1, False, True),     # d 128, non-causal: every query tile walks all 5 key tiles
 ]
 
 
