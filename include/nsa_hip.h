@@ -114,7 +114,7 @@ int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const
  * [batch, kv_heads, num_mem + num_keys, d] (bf16, or fp32 with dkv_fp32: the compressed keys are few and their
  * gradient feeds sums over every window, where a bf16 rounding per key is the largest error left).
  * bf16 in, fp32 accumulate, bf16 out.  Head and token strides of
- * q / d_out below 2^32 elements (NSA_E_UNSUPPORTED otherwise).
+ * q / d_out below 2^32 elements, token strides of k / v below 2^26 (NSA_E_UNSUPPORTED otherwise).
  * ------------------------------------------------------------------------------------------ */
 typedef struct nsa_dense_desc {
   int32_t batch, kv_heads, group, seq, num_keys, num_mem, dim_head;

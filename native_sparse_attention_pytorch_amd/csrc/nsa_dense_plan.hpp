@@ -59,6 +59,8 @@ static inline int make_dense_plan(const nsa_dense_desc* d, DensePlan& P) {
     if ((P.sq[t] | P.sk[t] | P.sv[t] | P.so[t] | P.sdo[t]) & 7) return NSA_E_ARG;
     if (t > 0 && ((P.sq[t] | P.sdo[t]) < 0 || ((P.sq[t] | P.sdo[t]) >> 32))) return NSA_E_UNSUPPORTED;      // 32-bit stride arithmetic in the dK/dV gathers
   }
+  // the K / V tile copies address a lane's row as a 32-bit byte offset (up to 15 rows) from a scalar base
+  if (P.sk[2] < 0 || P.sv[2] < 0 || (P.sk[2] >> 26) || (P.sv[2] >> 26)) return NSA_E_UNSUPPORTED;
   // dK/dV walk: 64-row tiles of k/v (memory slots included), the queries that can see a tile
   // are cut into chunks of chunk_q; smaller chunks when there would be too few work-groups
   P.key_tiles = (P.krows + 63) / 64;
