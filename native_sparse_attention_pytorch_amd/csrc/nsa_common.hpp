@@ -168,14 +168,16 @@ struct TileDma {
   // One round (1 KB per wave) of a tile whose 64 rows all exist; tb = address of the tile's first row.  Issuing a copy
   // keeps the wave's instruction stream busy for some 60 cycles; callers with MFMAs to issue put the rounds between them.
   __device__ __forceinline__ void round_full(const __bf16* __restrict__ tb, unsigned tile_off, int r) const {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+    // (s_nop 3: five wait states between the last scalar write and the load - enough for M0, and for an address register
+    // the compiler may have produced with v_readfirstlane right before: hazards inside inline assembly are not its business)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(voff), "s"(tb + r * WAVES * RPS * s_row) : "memory", "m0");
   }
   // The same under an execution mask (all ones: copy; zero: no lane takes part, nothing is read or written and tb may point
   // anywhere): lets a caller keep one straight-line instruction stream whether or not there is a tile to copy.
   // `lanes` is all ones or zero (32 bits, used for both halves of the mask) and wave-uniform.
   __device__ __forceinline__ void round_full_if(unsigned lanes, const __bf16* __restrict__ tb, unsigned tile_off, int r) const {
-    asm volatile("s_mov_b32 m0, %0\n\ts_mov_b64 vcc, exec\n\ts_mov_b32 exec_lo, %3\n\ts_mov_b32 exec_hi, %3\n\t"
+    asm volatile("s_mov_b32 m0, %0\n\ts_mov_b64 vcc, exec\n\ts_mov_b32 exec_lo, %3\n\ts_mov_b32 exec_hi, %3\n\ts_nop 0\n\t"
                  "global_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, vcc"
                  :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(voff), "s"(tb + r * WAVES * RPS * s_row),
                     "s"(__builtin_amdgcn_readfirstlane(lanes)) : "memory", "m0", "vcc");
@@ -195,7 +197,7 @@ struct TileDma {
       for (int r = 0; r < ROUNDS; ++r) {
         long row = first_row + ri + r * WAVES * RPS;
         row = row < limit ? row : limit - 1;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, off"
                      :: "s"(lds0 + tile_off + r * WAVES * 1024), "v"(base + row * s_row + src_off) : "memory", "m0");
       }
     }
