@@ -153,7 +153,7 @@ struct TileDma {
   static_assert((WAVES * RPS) % 8 == 0 && ROUNDS >= 1, "a lane's rows must keep their swizzle from round to round");
   int row_in, src_off;
   unsigned voff;        // byte offset of this lane's 16 bytes from the first row of a round
-  unsigned lds0;        // LDS byte address of this wave's segment in round 0 (wave-uniform)
+  unsigned lds0;        // LDS byte address of this wave's segment of the first 1 KB copy of a tile (wave-uniform)
   long s_row;
   // lds_base: the LDS array the tiles live in; a tile is addressed by its byte offset from it
   __device__ __forceinline__ void init(int tid, long row_stride, const __bf16* lds_base) {
