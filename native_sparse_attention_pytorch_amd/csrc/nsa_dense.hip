@@ -216,7 +216,8 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
             tmax = fmaxf(tmax, s);
           }
       };
-      if (!memtile && kb0 >= all_lo && kb0 + kBK - 1 <= all_hi) scale_scores(std::false_type{});      // wave-uniform
+      const bool plain = !memtile && kb0 >= all_lo && kb0 + kBK - 1 <= all_hi;      // wave-uniform
+      if (plain) scale_scores(std::false_type{});
       else scale_scores(std::true_type{});
 
       if (POOL && !memtile) {
@@ -284,6 +285,18 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
           const int rows_here = SH ? ppt : 32;
           const float norm = P.scale / (float)(npf * (SH ? P.g : 1));
           const int jb0 = kb0 / npf;
+          // The bulk of the tiles under a causal mask: every row of the wave sees every key of the tile, so every block of
+          // the tile is complete, visible and not the row's own, and (checked here) rows and blocks all exist.  Then a value's
+          // address is one wave-uniform base per tile plus a per-lane offset that does not depend on the tile.
+          const bool direct = P.causal && plain && i0 + ppt <= P.n && jb0 + nbt <= P.nb && (long)P.g * P.n * P.nb < (1l << 30);
+          if (direct) {
+            float* tbase = pooled + ((long)(SH ? bh : bh * P.g) * P.n + i0) * P.nb + jb0;
+            for (int e = lane; e < rows_here * nbt; e += 64) {
+              const int rr = e / nbt, jj = e % nbt;
+              const unsigned off = SH ? (unsigned)(rr * P.nb + jj) : (unsigned)(((rr & (P.g - 1)) * P.n + (rr >> P.lg)) * P.nb + jj);
+              tbase[off] = pw[e] * norm;
+            }
+          } else
           for (int e = lane; e < rows_here * nbt; e += 64) {
             const int rr = e / nbt, jj = e % nbt;
             const int qi = i0 + (SH ? rr : (rr >> P.lg));
