@@ -101,10 +101,13 @@ __device__ __forceinline__ bf16x8 lds_row_operand(const __bf16* tile_s, int RS, 
 
 // Swizzled row-major LDS tile (D = 64 or 128 bf16 per row, no padding) for tiles that are read both ways: the 16-byte
 // chunk c of row r is stored at chunk position (c & ~7) | ((c ^ swz(r)) & 7), swz(r) = 2 * (r % 4) + (r / 4) % 2.
-// Eight consecutive rows then put the same chunk into eight different bank groups (16-byte row reads, eight lanes per
-// clock: no conflicts), and four consecutive rows put a pair of adjacent chunks into four disjoint pairs (the transpose
-// load, a 16-lane group reading 4 rows x 32 bytes per clock: no conflicts).  A plain padded stride can give one or the
-// other.  swz depends on the lane only (not on the k-step or the feature tile), so a kernel pays a few address registers.
+// Measured with the bank-conflict counters (gfx950: 64 banks of 4 bytes per clock): a 64-lane 16-byte row read takes 8 clocks
+// in this layout (4 is the minimum, reached by a row stride of D + 8), the transpose load 4 clocks at D = 128 and 2 at D = 64
+// (2 is the minimum; stride D + 8 takes 8, D + 16 takes 4) - as good as a padded stride can be for a tile read both ways, and
+// the only choice for tiles filled by global_load_lds, which cannot pad.  A swizzle over all 16 positions of a row reaches
+// both minima but costs an XOR per read (rows r and r + 8 differ, k-steps no longer fold into immediate offsets); it was
+// measured no faster in the dense kernels and slower in the selection backward walk.  swz depends on the lane only (not on
+// the k-step or the feature tile), so a kernel pays a few address registers.
 __device__ __forceinline__ int lds_swz(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
 
 template <int D>
