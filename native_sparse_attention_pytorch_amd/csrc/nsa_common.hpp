@@ -74,13 +74,10 @@ typedef __attribute__((__vector_size__(4 * sizeof(short)))) short shortx4;
 // of X in the same order in which a 32x32 MFMA result holds its rows (registers 8u .. 8u+7).
 // Uses the gfx950 LDS transpose load: in every group of 16 lanes, lane ll receives element
 // ll % 4 of the four 8-byte rows addressed by lanes 4e + ll / 4 (e = 0..3) of its group.
-// Bank conflicts (32 banks of 4 bytes; a 16-lane group reads 4 consecutive rows x 32 bytes): free
-// when the row stride is 8 banks mod 32 (RS*2 bytes = 32 mod 128, i.e. RS = D + 16), two-way at
-// RS = D + 8.  The 16-byte row reads of lds_row_operand are served 8 rows per clock and want 4
-// banks per row instead (RS = D + 8); a tile read both ways cannot have both with a plain stride,
-// and an XOR swizzle that gives both was measured slower in the backward kernels (its chunk index
-// no longer folds into the instructions' immediate offsets: more address registers in kernels that
-// have none to spare).
+// Bank conflicts (measured with the conflict counters, D = 128): this load takes 4 clocks at a row stride of D + 16 and 8 at
+// D + 8 (2 would be conflict-free), the 16-byte row reads of lds_row_operand 4 clocks at D + 8 (their minimum) and 8 at D + 16:
+// a tile read only one way uses the matching stride, a tile read both ways the swizzled layout below or the stride of the
+// read it does more often.
 __device__ __forceinline__ bf16x8 lds_transposed_operand(const __bf16* X, int RS, int row0, int col0, int lane) {
   const int ll = lane & 15, e = ll >> 2, qq = ll & 3, mh = (lane >> 4) & 1, h = lane >> 5;
   const __bf16* p0 = X + (row0 + 4 * h + e) * RS + col0 + 16 * mh + 4 * qq;
