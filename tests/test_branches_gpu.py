@@ -168,6 +168,29 @@ def test_importance_softmax_topk_matches_oracle():
     assert not fm.cpu()[:, :, :B].any()
 
 
+@pytest.mark.parametrize("d", [64, 128])
+def test_dense_strided_views_equal_contiguous(d):
+    """q / k / v as 'b n (h d) -> b h n d' views of one projection output (token stride = the whole row, k and v at
+    offsets that are only 16-byte aligned): the tile copies address rows through the strides they are given, so the
+    results must be bit-equal to those on contiguous copies, forward and backward, causal and two-sided windows."""
+    from native_sparse_attention_pytorch_amd import ops
+    b, hq, hk, n = 2, 8, 2, 777
+    g = torch.Generator().manual_seed(d)
+    big = _rand((b, n, (hq + 2 * hk) * d + 24), g, d ** -0.5).cuda()
+    q = big[..., :hq * d].view(b, n, hq, d).transpose(1, 2)
+    k = big[..., hq * d + 8:hq * d + 8 + hk * d].view(b, n, hk, d).transpose(1, 2)
+    v = big[..., hq * d + 16 + hk * d:hq * d + 16 + 2 * hk * d].view(b, n, hk, d).transpose(1, 2)
+    do = _rand((b, hq, n, d), g).cuda()
+    for causal, win in ((True, 100), (False, 50)):
+        o1, l1, _ = ops.dense_fwd(q, k, v, 0, causal, win, 1, 0, False, 1, True, d ** -0.5)
+        o2, l2, _ = ops.dense_fwd(q.contiguous(), k.contiguous(), v.contiguous(), 0, causal, win, 1, 0, False, 1, True, d ** -0.5)
+        assert torch.equal(o1, o2) and torch.equal(l1, l2)
+        g1 = ops.dense_bwd(q, k, v, o1, do, l1, 0, causal, win, 1, 0, d ** -0.5)
+        g2 = ops.dense_bwd(q.contiguous(), k.contiguous(), v.contiguous(), o2, do, l2, 0, causal, win, 1, 0, d ** -0.5)
+        for a, b_ in zip(g1, g2):
+            assert torch.equal(a, b_)
+
+
 @pytest.mark.parametrize("b,h,n,d", [(2, 4, 100, 64), (1, 8, 333, 128)])
 def test_gate_combine_matches_oracle(b, h, n, d):
     from native_sparse_attention_pytorch_amd.ops import gate_combine
