@@ -11,11 +11,12 @@
 //
 // Forward and dQ are query-stationary: a work-group of 4 waves owns 128 rows (128/G consecutive
 // queries x the G heads of one kv group, so the group shares every K/V tile), each wave 32 rows.
-// 64-key K/V tiles are gathered with coalesced 16-byte loads into registers one tile ahead,
-// committed to row-major LDS tiles and read back as MFMA operands: row operands with 16-byte LDS
-// reads, transposed operands (V^T, K^T) with the gfx950 LDS transpose load.  dK/dV is
-// key-stationary: two waves own a 64-key tile (32 keys each) and stream the query rows that can
-// see it, like the dK/dV walk of the block-selection kernels.
+// 64-key K/V tiles are copied straight from global memory into swizzled LDS tiles one tile ahead
+// (global_load_lds_dwordx4: no staging registers, two buffers, one barrier per tile) and read
+// back as MFMA operands: row operands with 16-byte LDS reads, transposed operands (V^T, K^T)
+// with the gfx950 LDS transpose load.  dK/dV is key-stationary: two waves own a 64-key tile
+// (32 keys each) and stream the query rows that can see it through registers and padded LDS
+// tiles, like the dK/dV walk of the block-selection kernels.
 #include <type_traits>
 #include "nsa_common.hpp"
 #include "nsa_dense_plan.hpp"
@@ -48,25 +49,6 @@ __device__ __forceinline__ int xcd_contiguous(int x, int count) {
   return (x & 7) * per + (x >> 3);
 }
 static inline unsigned xcd_grid_for(int count) { return 8u * (unsigned)((count + 7) >> 3); }
-
-// One thread's share of a cooperative, coalesced load of `nrows` rows of D bf16 (row index ->
-// memory row through `first_row`, rows >= limit read as zero) by a work-group of NT threads.
-template <int D, int NT>
-struct TileRegs {
-  static constexpr int CPR = D / 8, RPI = NT / CPR, N = kBK / RPI;
-  bf16x8 r[N];
-  __device__ __forceinline__ void load(const __bf16* __restrict__ base, long s_row, long first_row, long limit, int tid) {
-#pragma unroll
-    for (int t = 0; t < N; ++t) {
-      const long row = first_row + t * RPI + tid / CPR;
-      r[t] = (row < limit) ? load8(base + row * s_row + 8 * (tid % CPR)) : zero_frag();
-    }
-  }
-  __device__ __forceinline__ void commit(__bf16* tile_s, int RS, int tid) const {
-#pragma unroll
-    for (int t = 0; t < N; ++t) *reinterpret_cast<bf16x8*>(tile_s + (t * RPI + tid / CPR) * RS + 8 * (tid % CPR)) = r[t];
-  }
-};
 
 // Key tiles walked by a query tile: t = -1 is the memory tile (stride mode), then 64-key tiles
 // t_lo .. t_hi of the interval union.
