@@ -371,34 +371,13 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
 }
 
 // ------------------------------------------------------------------------------ backward
-// delta[b,hq,i] = sum_d out * d_out
-template <int D>
-__global__ __launch_bounds__(256) void dense_delta_kernel(const DensePlan P, const __bf16* __restrict__ out, const __bf16* __restrict__ dout, float* __restrict__ delta) {
-  constexpr int LPR = D / 8, RPB = 256 / LPR;
-  const int tid = threadIdx.x;
-  const long row = (long)blockIdx.x * RPB + tid / LPR;
-  const long rows = (long)P.bh * P.g * P.n;
-  const int dd = (tid % LPR) * 8;
-  float s = 0.f;
-  if (row < rows) {
-    const long i = row % P.n, bhq = row / P.n;
-    const long b = bhq / (P.hkv * P.g), hq = bhq % (P.hkv * P.g);
-    const bf16x8 o = load8(out + b * P.so[0] + hq * P.so[1] + i * P.so[2] + dd);
-    const bf16x8 d = load8(dout + b * P.sdo[0] + hq * P.sdo[1] + i * P.sdo[2] + dd);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s += (float)o[e] * (float)d[e];
-  }
-#pragma unroll
-  for (int mk = LPR / 2; mk >= 1; mk >>= 1) s += __shfl_xor(s, mk, 64);
-  if (row < rows && (tid % LPR) == 0) delta[row] = s;
-}
-
 // dQ, query-stationary (same tile walk as the forward): dS^T = P^T o (V dO^T - delta),
 // dQ^T += K^T dS^T with K^T read through the LDS transpose load.
 template <int D>
 __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
-                                                           const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
-                                                           const float* __restrict__ lse, const float* __restrict__ delta, __bf16* __restrict__ dq) {
+                                                           const __bf16* __restrict__ v, const __bf16* __restrict__ out,
+                                                           const __bf16* __restrict__ dout, const float* __restrict__ lse,
+                                                           float* __restrict__ delta, __bf16* __restrict__ dq) {
   constexpr int KS = D / 16, DT = D / 32, TILE = kBK * D;
   // as in the forward kernel: two swizzled tiles each for K and V, filled by asynchronous copies, one barrier per tile
   __shared__ __align__(1024) __bf16 k_s[2 * TILE];
@@ -424,7 +403,21 @@ __global__ __launch_bounds__(256, 2) void dense_bwd_dq_kernel(const DensePlan P,
     for (int ks = 0; ks < KS; ++ks) { Qf[ks] = load8(qp + 16 * ks); Gf[ks] = load8(gp + 16 * ks); }
   }
   const long srow = ((long)b * P.hkv * P.g + hq) * P.n + i;
-  const float lse_r = lse[srow] * kLog2e, del_r = delta[srow];
+  const float lse_r = lse[srow] * kLog2e;
+  // delta = sum_d out * d_out of this lane's row: this kernel holds the row's d_out anyway, reads the row of out beside it
+  // and leaves the sums for the dK/dV kernel that follows on the stream (a pass of its own over out and d_out before)
+  float del_r = 0.f;
+  {
+    const __bf16* op = out + b * P.so[0] + (long)hq * P.so[1] + (long)i * P.so[2] + 8 * h;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8 o8 = load8(op + 16 * ks);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) del_r = __builtin_fmaf((float)o8[e], (float)Gf[ks][e], del_r);
+    }
+    del_r = halves_sum(del_r);
+    if (valid && h == 0) delta[srow] = del_r;
+  }
   const Interval me = visible_range(P, i);
   const TileWalk walk = make_walk(P, q0, min(P.n - 1, q0 + 4 * ppt - 1));
   const int my_hi = visible_range(P, min(P.n - 1, i0 + ppt - 1)).hi, my_lo = visible_range(P, min(i0, P.n - 1)).lo;
@@ -832,13 +825,9 @@ static int dense_bwd_launch(const DensePlan& P, const void* q, const void* k, co
                             void* ws, void* dq, void* dk, void* dv, hipStream_t st) {
   float* delta = reinterpret_cast<float*>((char*)ws + P.off_delta);
   float* part = reinterpret_cast<float*>((char*)ws + P.off_part);
-  const long rows = (long)P.bh * P.g * P.n;
-  constexpr int RPB = 256 / (D / 8);
-  hipLaunchKernelGGL((dense_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, delta);
-  NSA_LAUNCH_CHECK();
   const int qpw = 4 * (32 >> P.lg);
   hipLaunchKernelGGL((dense_bwd_dq_kernel<D>), dim3(P.mode == 0 ? xcd_grid_for((P.n + qpw - 1) / qpw) : (unsigned)((P.n + qpw - 1) / qpw), P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
-                     (const __bf16*)v, (const __bf16*)dout, lse, delta, (__bf16*)dq);
+                     (const __bf16*)v, (const __bf16*)out, (const __bf16*)dout, lse, delta, (__bf16*)dq);      // also writes delta
   NSA_LAUNCH_CHECK();
   hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
