@@ -110,6 +110,9 @@ int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const
  *                     the query's own block when stride != sel_block) make the softmax term zero.
  *                     sel_block / stride must be a power of two <= 32 (with sel_block == stride the
  *                     output holds one logit per compressed key, which serves every other ratio).
+ *                     pool = 2 (causal only, otherwise as 1): row i of `pooled` is defined only below
+ *                     column floor(i / sel_block), the part a causal query can select from; the rest of
+ *                     the row (all -inf with pool = 1) is left unwritten - for nsa_topk_prefix.
  * out/lse as for nsa_select_fwd; dq contiguous [batch, heads, seq, d]; dk, dv contiguous
  * [batch, kv_heads, num_mem + num_keys, d] (bf16, or fp32 with dkv_fp32: the compressed keys are few and their
  * gradient feeds sums over every window, where a bf16 rounding per key is the largest error left).
@@ -140,6 +143,12 @@ int nsa_dense_bwd(const nsa_dense_desc* d, const void* q, const void* k, const v
  * comes out as value NaN with fmask 0.  Limits: nb <= 2048, k <= min(nb, 64) (NSA_E_UNSUPPORTED otherwise). */
 int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k, int32_t apply_softmax,
              int32_t* idx, float* vals, uint8_t* fmask, void* stream);
+/* The same for the logits of a causal compressed forward (nsa_dense_fwd with pool = 2): row r belongs to query
+ * r % seq, and only its columns below floor(query / block) - the selection blocks that lie completely before the
+ * query, NSA.py:676-689 - are defined; the rest counts as -inf and is never read (about half the matrix).  Same
+ * results as nsa_topk on a matrix whose undefined part holds -inf.  rows must be a multiple of seq. */
+int nsa_topk_prefix(const float* scores, int64_t rows, int32_t nb, int32_t k, int32_t apply_softmax,
+                    int32_t seq, int32_t block, int32_t* idx, float* vals, uint8_t* fmask, void* stream);
 
 /* Fused strategy-gate combine.  Replaces Sigmoid + Rearrange('b n (h s) -> b h n s') + the
  * stack/einsum + merge_heads of NSA.py:323-327, 854-860.  logits: bf16 contiguous [batch, seq,

@@ -89,6 +89,7 @@ def lib():
         L.nsa_dense_fwd.argtypes = [C.POINTER(DenseDesc)] + [vp] * 7
         L.nsa_dense_bwd.argtypes = [C.POINTER(DenseDesc)] + [vp] * 7 + [sz] + [vp] * 4
         L.nsa_topk.argtypes = [vp, C.c_int64, C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp]
+        L.nsa_topk_prefix.argtypes = [vp, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp]
         i3 = C.POINTER(C.c_int64)
         L.nsa_gate_fwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp]
         L.nsa_gate_bwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp, vp, vp, vp, vp]
@@ -121,7 +122,7 @@ def lib():
         L.nsa_dense_fwd_f32.argtypes = [C.POINTER(DenseDesc)] + [vp] * 5 + [C.c_int32, vp]
         L.nsa_select_fwd_f32.argtypes = [C.POINTER(SelectDesc)] + [vp] * 7 + [C.c_int32, C.c_int32, vp]
         L.nsa_dense_fwd_f32.restype = L.nsa_select_fwd_f32.restype = C.c_int
-        for name in ("nsa_dense_workspace_bytes", "nsa_dense_fwd", "nsa_dense_bwd", "nsa_topk", "nsa_gate_fwd", "nsa_gate_bwd"):
+        for name in ("nsa_dense_workspace_bytes", "nsa_dense_fwd", "nsa_dense_bwd", "nsa_topk", "nsa_topk_prefix", "nsa_gate_fwd", "nsa_gate_bwd"):
             getattr(L, name).restype = C.c_int
         for name in ("nsa_select_workspace_bytes", "nsa_select_build_index", "nsa_select_fwd", "nsa_select_bwd"):
             getattr(L, name).restype = C.c_int

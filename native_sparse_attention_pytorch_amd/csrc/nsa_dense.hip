@@ -336,7 +336,7 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
     }
   }
 
-  if (POOL) {
+  if (POOL && !P.nofill) {
     // fine blocks whose compressed keys no query of this wave's tile can see were never visited
     const int last_visited = my_hi >= 0 ? min(walk.t_hi, my_hi / kBK) : -1;
     const int jstart = min(P.nb, (kBK * (last_visited + 1)) / (POOL ? NPF : 1));

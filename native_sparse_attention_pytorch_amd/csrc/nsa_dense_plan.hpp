@@ -10,7 +10,7 @@ struct DensePlan {
   int b, hkv, g, lg, n, nkeys, mem, krows, D, bh;
   int mode, causal, wb, wf, st;
   int st_sh;                 // log2(st) when the stride is a power of two (the division becomes a shift), else -1
-  int pool, npf, nb, B, share, mask_own;
+  int pool, npf, nb, B, share, mask_own, nofill;
   int dkv_fp32;              // dk / dv leave the reduce kernel as fp32 instead of bf16
   float scale;
   int key_tiles, chunks, chunk_q;
@@ -34,7 +34,7 @@ static inline int make_dense_plan(const nsa_dense_desc* d, DensePlan& P) {
   const long bh = (long)P.b * P.hkv;
   if (bh > 65535) return NSA_E_UNSUPPORTED;
   P.bh = (int)bh;
-  P.wb = P.wf = 0; P.st = 1; P.pool = 0; P.npf = 1; P.nb = 0; P.B = 1; P.share = 1; P.mask_own = 0;
+  P.wb = P.wf = 0; P.st = 1; P.pool = 0; P.npf = 1; P.nb = 0; P.B = 1; P.share = 1; P.mask_own = 0; P.nofill = 0;
   if (P.mode == 0) {
     if (d->window < 0 || P.mem != 0 || P.nkeys != P.n) return NSA_E_ARG;
     P.wb = d->window; P.wf = P.causal ? 0 : d->window;
@@ -47,6 +47,7 @@ static inline int make_dense_plan(const nsa_dense_desc* d, DensePlan& P) {
       P.npf = d->sel_block / d->stride;
       if (P.npf > 32 || (P.npf & (P.npf - 1))) return NSA_E_UNSUPPORTED;
       P.pool = 1; P.B = d->sel_block; P.share = d->share ? 1 : 0;
+      P.nofill = (d->pool == 2 && d->causal) ? 1 : 0;      // the caller reads row i only below column floor(i / B)
       P.mask_own = d->stride != d->sel_block;
       P.nb = P.nkeys / P.npf;
       if (P.nb == 0) P.pool = 0;

@@ -40,10 +40,14 @@ struct TopkDyn { const int* state; int per_block; };
 
 template <int VPL, bool POOL>
 __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in, long rows, int nb, int k, int softmax, int vec4, PoolArgs pool,
-                                                   int* __restrict__ idx, float* __restrict__ vals, uint8_t* __restrict__ fmask, int kstride, TopkDyn dyn) {
+                                                   int* __restrict__ idx, float* __restrict__ vals, uint8_t* __restrict__ fmask, int kstride, TopkDyn dyn,
+                                                   int pseq, int pblk) {
   const int lane = threadIdx.x & 63;
   const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
+  // pseq > 0: row r belongs to query r % pseq, and only its columns below floor(query / pblk) are defined (the blocks that
+  // lie completely before the query); the rest counts as -inf and is not read
+  const int lim = pseq > 0 ? min(nb, (int)(row % pseq) / pblk) : nb;
   if (dyn.state != nullptr) {
     nb = min(nb, dyn.state[1] / dyn.per_block);
     k = min(k, nb);
@@ -100,9 +104,9 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in,
       for (int r4 = 0; r4 < VPL / 4; ++r4) {
         const int j = lane * VPL + 4 * r4;
         floatx4 t = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-        if (j < nb) t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(src + j));      // read once
+        if (j < lim) t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(src + j));      // read once
 #pragma unroll
-        for (int e = 0; e < 4; ++e) x[4 * r4 + e] = t[e];
+        for (int e = 0; e < 4; ++e) x[4 * r4 + e] = (j + e < lim) ? t[e] : -INFINITY;
       }
       loaded = true;
     }
@@ -111,7 +115,7 @@ __global__ __launch_bounds__(256) void topk_kernel(const float* __restrict__ in,
 #pragma unroll
     for (int r = 0; r < VPL; ++r) {
       const int j = lane * VPL + r;
-      x[r] = j < nb ? src[j] : -INFINITY;
+      x[r] = j < lim ? src[j] : -INFINITY;
     }
   }
   if (softmax) {
@@ -200,7 +204,8 @@ __device__ __forceinline__ float row16_sum(float v) {
 
 template <int VPL>
 __global__ __launch_bounds__(256) void topk_rows4_kernel(const float* __restrict__ in, long rows, int nb, int k, int softmax, int vec4,
-                                                         int* __restrict__ idx, float* __restrict__ vals, uint8_t* __restrict__ fmask) {
+                                                         int* __restrict__ idx, float* __restrict__ vals, uint8_t* __restrict__ fmask,
+                                                         int pseq, int pblk) {
   constexpr int GS = VPL < 8 ? VPL : 8, NG = VPL / GS;
   constexpr int SEG = VPL + 4;                            // a lane's segment, padded: 16-byte reads of 16 lanes hit 64 distinct banks
   __shared__ __align__(16) float xs[16][16 * SEG];        // [row of the work-group][lane `sub`][entries sub*VPL ..]
@@ -208,6 +213,7 @@ __global__ __launch_bounds__(256) void topk_rows4_kernel(const float* __restrict
   const long row = (long)blockIdx.x * 16 + wave * 4 + rs;
   const bool live = row < rows;                             // a dead row group works on the last row and stores nothing
   const float* src = in + (live ? row : rows - 1) * nb;
+  const int lim = pseq > 0 ? min(nb, (int)((live ? row : rows - 1) % pseq) / pblk) : nb;      // see topk_kernel
   float* row_s = xs[wave * 4 + rs];
   float* mine_s = row_s + sub * SEG;
   float x[VPL];
@@ -219,15 +225,15 @@ __global__ __launch_bounds__(256) void topk_rows4_kernel(const float* __restrict
     for (int r4 = 0; r4 < VPL / 4; ++r4) {
       const int j = 4 * (sub + 16 * r4);
       floatx4 t = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-      if (j < nb) t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(src + j));      // read once
+      if (j < lim) t = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(src + j));      // read once
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[4 * r4 + e] = t[e];
+      for (int e = 0; e < 4; ++e) x[4 * r4 + e] = (j + e < lim) ? t[e] : -INFINITY;
     }
   } else {
 #pragma unroll
     for (int r = 0; r < VPL; ++r) {
       const int j = sub * VPL + r;
-      x[r] = j < nb ? src[j] : -INFINITY;
+      x[r] = j < lim ? src[j] : -INFINITY;
     }
   }
   if (softmax) {
@@ -320,8 +326,8 @@ __global__ __launch_bounds__(256) void topk_rows4_kernel(const float* __restrict
 }  // namespace nsa
 
 #define NSA_TOPK_POOL false
-extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k, int32_t apply_softmax,
-                        int32_t* idx, float* vals, uint8_t* fmask, void* stream) {
+static int topk_launch(const float* scores, int64_t rows, int32_t nb, int32_t k, int32_t apply_softmax, int32_t pseq, int32_t pblk,
+                       int32_t* idx, float* vals, uint8_t* fmask, void* stream) {
   using namespace nsa;
   if (!scores || !idx || !vals || !fmask || rows <= 0 || nb <= 0 || k <= 0 || k > nb) return NSA_E_ARG;
   if (nb > 64 * 32 || k > 64) return NSA_E_UNSUPPORTED;
@@ -331,7 +337,7 @@ extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k
   const int vec4 = (nb % 4 == 0) && ((reinterpret_cast<uintptr_t>(scores) & 15) == 0);
   if (k <= 16 && nb <= 512) {          // four rows per wave
     const dim3 grid4((unsigned)((rows + 15) / 16));
-#define NSA_TOPK4(V) hipLaunchKernelGGL((topk_rows4_kernel<V>), grid4, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, idx, vals, fmask)
+#define NSA_TOPK4(V) hipLaunchKernelGGL((topk_rows4_kernel<V>), grid4, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, idx, vals, fmask, pseq, pblk)
     if (nb <= 64) NSA_TOPK4(4);
     else if (nb <= 128) NSA_TOPK4(8);
     else if (nb <= 256) NSA_TOPK4(16);
@@ -342,7 +348,7 @@ extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k
   }
   const PoolArgs pool{0, 1, 0, 1};
   const TopkDyn dyn{nullptr, 1};
-#define NSA_TOPK(V) hipLaunchKernelGGL((topk_kernel<V, NSA_TOPK_POOL>), grid, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, pool, idx, vals, fmask, k, dyn)
+#define NSA_TOPK(V) hipLaunchKernelGGL((topk_kernel<V, NSA_TOPK_POOL>), grid, block, 0, st, scores, (long)rows, nb, k, apply_softmax, vec4, pool, idx, vals, fmask, k, dyn, pseq, pblk)
 #define NSA_TOPK_DISPATCH()            \
   if (vpl <= 1) NSA_TOPK(1);           \
   else if (vpl <= 2) NSA_TOPK(2);      \
@@ -353,6 +359,17 @@ extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k
   NSA_TOPK_DISPATCH();
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : (int)e;
+}
+
+extern "C" int nsa_topk(const float* scores, int64_t rows, int32_t nb, int32_t k, int32_t apply_softmax,
+                        int32_t* idx, float* vals, uint8_t* fmask, void* stream) {
+  return topk_launch(scores, rows, nb, k, apply_softmax, 0, 1, idx, vals, fmask, stream);
+}
+
+extern "C" int nsa_topk_prefix(const float* scores, int64_t rows, int32_t nb, int32_t k, int32_t apply_softmax, int32_t seq, int32_t block,
+                               int32_t* idx, float* vals, uint8_t* fmask, void* stream) {
+  if (seq <= 0 || block <= 0 || rows % seq != 0) return NSA_E_ARG;
+  return topk_launch(scores, rows, nb, k, apply_softmax, seq, block, idx, vals, fmask, stream);
 }
 
 #undef NSA_TOPK_POOL
@@ -376,6 +393,7 @@ int decode_topk_launch(const float* logits, int32_t batch, int32_t kv_heads, int
   const float* scores = logits;
   const PoolArgs pool{share ? group : 1, per_block, num_compressed, units};
   const TopkDyn dyn{state, per_block};
+  const int pseq = 0, pblk = 1;
   NSA_TOPK_DISPATCH();
 #undef NSA_TOPK_DISPATCH
 #undef NSA_TOPK

@@ -249,7 +249,7 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
         # the reference's second output (TRI.py:195-277 with SLIDING): causal attention over the last block_size + 1 keys,
         # 0 <= i - j <= block_size (test_triton_nsa.py:45-51); here it is the sliding-window kernel with that window
         qp, g0, gp0 = _pad_groups(fq.to(_BF16), kv_heads)
-        sliding_out, sliding_lse, _ = dense_fwd(qp, fk, fv, 0, True, int(block_size), 1, 0, False, 1, True, float(scale))
+        sliding_out, sliding_lse, _ = dense_fwd(qp, fk, fv, 0, True, int(block_size), 1, 0, 0, 1, True, float(scale))
         sliding_out = _unpad_groups(sliding_out, kv_heads, g0, gp0)[..., :d_head].to(dtype)
         sliding_lse = _unpad_groups(sliding_lse, kv_heads, g0, gp0)
     if kv_heads != sel_heads:                         # per-query-head selection: TRI.py:1961-1962
@@ -295,7 +295,9 @@ def _dense_desc(q, k, v, o, do, mode, causal, window, stride, num_mem, pool, sel
 
 @torch.library.custom_op("nsa_amd::dense_fwd", mutates_args=())
 def dense_fwd(q: Tensor, k: Tensor, v: Tensor, mode: int, causal: bool, window: int, stride: int, num_mem: int,
-              pool: bool, sel_block: int, share: bool, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+              pool: int, sel_block: int, share: bool, scale: float) -> tuple[Tensor, Tensor, Tensor]:
+    """pool: 0 no importance logits, 1 logits with -inf wherever a block cannot be selected, 2 (causal) logits defined only
+    below column i // sel_block of row i, the rest unwritten (for `importance_topk(..., prefix=...)`)."""
     q, k, v = _prep(q), _prep(k), _prep(v)
     b, hq, n, d = q.shape
     hk = k.shape[1]
@@ -307,7 +309,7 @@ def dense_fwd(q: Tensor, k: Tensor, v: Tensor, mode: int, causal: bool, window: 
     if pool:
         npf = sel_block // stride
         nb = (k.shape[2] - num_mem) // npf
-    pool = bool(pool and nb > 0)
+    pool = int(pool) if nb > 0 else 0
     pooled = torch.empty((b, hk if share else hq, n, nb), dtype=torch.float32, device=q.device)
     dsc = _dense_desc(q, k, v, out, out, mode, causal, window, stride, num_mem, pool, sel_block, share, scale)
     _lib.check(_lib.lib().nsa_dense_fwd(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(pooled) if pool else 0, _stream()),
@@ -413,16 +415,20 @@ def sliding_attend(q: Tensor, k: Tensor, v: Tensor, window_size: int, causal: bo
     d = q.shape[-1]
     D = _kernel_dim(d)
     qp, g, gp = _pad_groups(_pad_dim(q, D), k.shape[1])
-    out, _, _ = dense_fwd(qp, _pad_dim(k, D), _pad_dim(v, D), 0, bool(causal), int(window_size), 1, 0, False, 1, True, float(d ** -0.5))
+    out, _, _ = dense_fwd(qp, _pad_dim(k, D), _pad_dim(v, D), 0, bool(causal), int(window_size), 1, 0, 0, 1, True, float(d ** -0.5))
     return _unpad_groups(out, k.shape[1], g, gp)[..., :d]
 
 
 def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int, causal: bool,
-                    sel_block: int | None = None, share: bool = True):
+                    sel_block: int | None = None, share: bool = True, prefix_only: bool = False):
     """Compressed branch: attend(q, [mem; ck], [mem; cv], cmask, return_sim=True) of NSA.py:621-639.
     Returns (out, importance_logits) where importance_logits [b, Hkv|Hq, n, nb] are the block
     importance logits of NSA.py:652-691 before the softmax (None if sel_block is None or no full
-    fine block exists): the logits matrix itself is never written to memory."""
+    fine block exists): the logits matrix itself is never written to memory.
+    With `prefix_only` the result is (out, importance_logits, prefix): if `prefix` is not None it is (n, sel_block) and row i
+    of the logits is defined only below column i // sel_block - what a causal query can select from; the rest (all -inf
+    otherwise) was not written and must not be read: pass `prefix` on to `importance_topk`.  Only for logits nothing else
+    reads (no gradient through them)."""
     pool = sel_block is not None
     d = q.shape[-1]
     scale = float(d ** -0.5)
@@ -443,21 +449,28 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
         # the reference's own inference test) take the per-key logits from the kernel (a "block" of one key: head mean and
         # visibility as usual) and finish NSA.py:676-689 with three elementwise ops: mean over the block's keys (-inf as
         # soon as one key is invisible), own block masked.
-        out, _, per_key = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), True, int(stride), bool(share), scale)
+        out, _, per_key = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), 1, int(stride), bool(share), scale)
         out = _unpad_groups(out, hk, g, gp)[..., :d]
         n, nb = q.shape[2], per_key.shape[-1] // npf
         if nb == 0:
-            return out, None
+            return (out, None, None) if prefix_only else (out, None)
         imp = logits_of(per_key)[..., :nb * npf].unflatten(-1, (nb, npf)).mean(dim=-1)
         own = (torch.arange(n, device=q.device) // int(sel_block))[:, None] == torch.arange(nb, device=q.device)[None, :]
-        return out, imp.masked_fill(own, float("-inf"))
-    out, _, pooled = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), pool, int(sel_block or stride), bool(share), scale)
-    return _unpad_groups(out, hk, g, gp)[..., :d], (logits_of(pooled) if pool and pooled.shape[-1] > 0 else None)
+        imp = imp.masked_fill(own, float("-inf"))
+        return (out, imp, None) if prefix_only else (out, imp)
+    use_prefix = bool(prefix_only and pool and causal and g == gp)
+    out, _, pooled = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), (2 if use_prefix else 1) if pool else 0,
+                               int(sel_block or stride), bool(share), scale)
+    out = _unpad_groups(out, hk, g, gp)[..., :d]
+    imp = logits_of(pooled) if pool and pooled.shape[-1] > 0 else None
+    if not prefix_only:
+        return out, imp
+    return out, imp, ((q.shape[2], int(sel_block)) if use_prefix and imp is not None else None)
 
 
 # ------------------------------------------------------------------------------------ top-k
 
-def _topk_impl(scores: Tensor, k: int, apply_softmax: bool):
+def _topk_impl(scores: Tensor, k: int, apply_softmax: bool, prefix=None):
     if scores.dtype != torch.float32 or not scores.is_cuda:
         raise RuntimeError("importance scores must be fp32 device tensors")
     scores = scores.contiguous()
@@ -467,7 +480,14 @@ def _topk_impl(scores: Tensor, k: int, apply_softmax: bool):
     idx = torch.empty(shp, dtype=torch.int32, device=scores.device)
     vals = torch.empty(shp, dtype=torch.float32, device=scores.device)
     fm = torch.empty(shp, dtype=torch.uint8, device=scores.device)
-    _lib.check(_lib.lib().nsa_topk(_ptr(scores), rows, nb, k, int(apply_softmax), _ptr(idx), _ptr(vals), _ptr(fm), _stream()), "nsa_topk")
+    if prefix is not None:
+        seq, block = prefix
+        if scores.shape[-2] != seq:
+            raise RuntimeError(f"prefix {prefix}: the logits have {scores.shape[-2]} rows per sequence")
+        _lib.check(_lib.lib().nsa_topk_prefix(_ptr(scores), rows, nb, k, int(apply_softmax), int(seq), int(block), _ptr(idx), _ptr(vals), _ptr(fm),
+                                              _stream()), "nsa_topk_prefix")
+    else:
+        _lib.check(_lib.lib().nsa_topk(_ptr(scores), rows, nb, k, int(apply_softmax), _ptr(idx), _ptr(vals), _ptr(fm), _stream()), "nsa_topk")
     return idx, vals, fm
 
 
@@ -503,10 +523,14 @@ class _ImportanceTopk(torch.autograd.Function):
         return dl, None
 
 
-def importance_topk(importance_logits: Tensor, num_selected: int):
+def importance_topk(importance_logits: Tensor, num_selected: int, prefix=None):
     """softmax with the -1e3 pad column (NSA.py:693-695) + topk (NSA.py:713) + `> 1e-10` mask
     (NSA.py:721).  Returns (values fp32, indices int32, fmask bool), each [..., num_selected];
-    `values` is differentiable with respect to the logits."""
+    `values` is differentiable with respect to the logits.  `prefix` = (n, sel_block) as returned by
+    `compress_attend(..., prefix_only=True)`: row i is read only below column i // sel_block (no gradient)."""
+    if prefix is not None:
+        idx, vals, fm = _topk_impl(importance_logits.detach(), int(num_selected), True, prefix)
+        return vals, idx, fm.view(torch.bool)
     if importance_logits.requires_grad and torch.is_grad_enabled():
         vals, idx, fm = _ImportanceTopk.apply(importance_logits, int(num_selected))
     elif torch.compiler.is_compiling():

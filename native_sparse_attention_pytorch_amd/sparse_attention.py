@@ -384,8 +384,15 @@ class SparseAttention(nn.Module):
 
         want_sel = self.num_selected_blocks > 0 and nc > 0
         share = self.query_heads_share_selected_kv
-        c_out, imp = ops.compress_attend(q16 if fused else q.to(bf16), ck.to(bf16), cv.to(bf16), M, st, self.causal,
-                                         sel_block=B if want_sel else None, share=share)
+        # without differentiable top-k nothing but the top-k reads the importance logits: under a causal mask the kernel then
+        # writes, and the top-k reads, only the part of every row a query can select from (`prefix`)
+        prefix = None
+        if self.use_diff_topk:
+            c_out, imp = ops.compress_attend(q16 if fused else q.to(bf16), ck.to(bf16), cv.to(bf16), M, st, self.causal,
+                                             sel_block=B if want_sel else None, share=share)
+        else:
+            c_out, imp, prefix = ops.compress_attend(q16 if fused else q.to(bf16), ck.to(bf16), cv.to(bf16), M, st, self.causal,
+                                                     sel_block=B if want_sel else None, share=share, prefix_only=True)
 
         if not fused:
             # rotary positions for the selection and sliding branches (NSA.py:643), one HIP kernel each
@@ -394,7 +401,7 @@ class SparseAttention(nn.Module):
 
         num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
         if num_sel > 0:
-            vals, idx, fmask = ops.importance_topk(imp, num_sel)
+            vals, idx, fmask = ops.importance_topk(imp, num_sel, prefix=prefix)
             # straight-through gates (NSA.py:715): value 1, gradient flows into the importance scores
             gates = (vals + (1. - vals).detach()) if self.use_diff_topk else None
             f_out = ops.native_sparse_attend(rq16, rk16, v16, B, idx, fmask, sel_scale=gates, include_block_causal=self.causal)

@@ -144,6 +144,43 @@ def test_topk_bit_exact_on_given_scores():
         assert torch.equal(fm.cpu().bool(), wv > 1e-10)
 
 
+def test_topk_prefix_equals_topk_on_filled_logits():
+    """nsa_topk_prefix on logits whose undefined part holds garbage (NaN) = nsa_topk on the same logits with -inf there,
+    bit for bit (indices, values, mask): both kernel families (<= 512 blocks with k <= 16, and the general one), rows that
+    see nothing, rows whose limit is not a multiple of 4, limits beyond the number of blocks."""
+    from native_sparse_attention_pytorch_amd.ops import importance_topk
+    g = torch.Generator().manual_seed(2)
+    for b, h, n, nb, k, B in [(2, 2, 600, 37, 8, 16), (1, 3, 1000, 512, 16, 2), (1, 2, 700, 600, 16, 1), (2, 1, 300, 64, 20, 4), (1, 1, 130, 8, 8, 16)]:
+        logits = torch.randn(b, h, n, nb, generator=g) * 2
+        lim = (torch.arange(n) // B)[:, None]
+        dead = torch.arange(nb)[None, :] >= lim
+        full = logits.masked_fill(dead, float('-inf')).to(DEV)
+        junk = logits.masked_fill(dead, float('nan')).to(DEV)
+        v1, i1, f1 = importance_topk(full, k)
+        v2, i2, f2 = importance_topk(junk, k, prefix=(n, B))
+        assert torch.equal(i1, i2) and torch.equal(f1, f2), f"nb={nb} k={k} B={B}"
+        assert torch.equal(v1, v2)
+
+
+@pytest.mark.parametrize("hq,hk,n,d,st,B,mem,share", [(8, 2, 515, 128, 16, 64, 1, True), (4, 2, 700, 64, 4, 16, 2, True), (4, 2, 300, 64, 8, 8, 1, False)])
+def test_compress_prefix_logits_select_the_same_blocks(hq, hk, n, d, st, B, mem, share):
+    """The module's path without differentiable top-k (logits written and read below each row's causal limit only) against
+    the full logits: same output, same selected blocks and mask."""
+    from native_sparse_attention_pytorch_amd.ops import compress_attend, importance_topk
+    g = torch.Generator().manual_seed(n + st)
+    nc = n // st
+    q = _rand((1, hq, n, d), g, d ** -0.25).to(DEV)
+    ck, cv = _rand((1, hk, nc + mem, d), g, d ** -0.25).to(DEV), _rand((1, hk, nc + mem, d), g).to(DEV)
+    o1, imp1 = compress_attend(q, ck, cv, mem, st, True, sel_block=B, share=share)
+    o2, imp2, prefix = compress_attend(q, ck, cv, mem, st, True, sel_block=B, share=share, prefix_only=True)
+    assert prefix == (n, B)
+    assert torch.equal(o1, o2)
+    k = min(6, imp1.shape[-1])
+    v1, i1, f1 = importance_topk(imp1, k)
+    v2, i2, f2 = importance_topk(imp2, k, prefix=prefix)
+    assert torch.equal(i1, i2) and torch.equal(f1, f2) and torch.equal(v1, v2)
+
+
 def test_importance_softmax_topk_matches_oracle():
     from native_sparse_attention_pytorch_amd.ops import importance_topk
     g = torch.Generator().manual_seed(1)

@@ -87,8 +87,8 @@ def test_config3_full_module_forward_backward():
 
     captured = {}
     orig = ops.importance_topk
-    def spy(imp, k_):
-        r = orig(imp, k_)
+    def spy(imp, k_, **kw_):
+        r = orig(imp, k_, **kw_)
         captured["sel"] = (r[1].cpu().long(), r[2].cpu())
         return r
 

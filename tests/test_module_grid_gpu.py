@@ -47,8 +47,8 @@ def _case(diff, causal, n, kvh, B, cbs, st, S, share, seed):
     captured = {}
     orig = ops.importance_topk
 
-    def spy(imp, k):
-        r = orig(imp, k)
+    def spy(imp, k, **kw_):
+        r = orig(imp, k, **kw_)
         captured["sel"] = (r[1].cpu().long(), r[2].cpu())
         return r
     ops.importance_topk = spy
