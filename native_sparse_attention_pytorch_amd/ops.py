@@ -502,6 +502,17 @@ def _(scores, k, apply_softmax):
     return (scores.new_empty(shp, dtype=torch.int32), scores.new_empty(shp), scores.new_empty(shp, dtype=torch.uint8))
 
 
+@torch.library.custom_op("nsa_amd::topk_prefix", mutates_args=())
+def topk_prefix_op(scores: Tensor, k: int, apply_softmax: bool, seq: int, block: int) -> tuple[Tensor, Tensor, Tensor]:
+    return _topk_impl(scores, k, apply_softmax, (seq, block))
+
+
+@topk_prefix_op.register_fake
+def _(scores, k, apply_softmax, seq, block):
+    shp = (*scores.shape[:-1], k)
+    return (scores.new_empty(shp, dtype=torch.int32), scores.new_empty(shp), scores.new_empty(shp, dtype=torch.uint8))
+
+
 class _ImportanceTopk(torch.autograd.Function):
     """HIP top-k in the forward; the backward of `values` through the padded softmax (plain
     elementwise torch, O(rows * nb)) - only used for the differentiable top-k gates."""
@@ -529,7 +540,10 @@ def importance_topk(importance_logits: Tensor, num_selected: int, prefix=None):
     `values` is differentiable with respect to the logits.  `prefix` = (n, sel_block) as returned by
     `compress_attend(..., prefix_only=True)`: row i is read only below column i // sel_block (no gradient)."""
     if prefix is not None:
-        idx, vals, fm = _topk_impl(importance_logits.detach(), int(num_selected), True, prefix)
+        if torch.compiler.is_compiling():
+            idx, vals, fm = topk_prefix_op(importance_logits.detach(), int(num_selected), True, int(prefix[0]), int(prefix[1]))
+        else:
+            idx, vals, fm = _topk_impl(importance_logits.detach(), int(num_selected), True, prefix)
         return vals, idx, fm.view(torch.bool)
     if importance_logits.requires_grad and torch.is_grad_enabled():
         vals, idx, fm = _ImportanceTopk.apply(importance_logits, int(num_selected))
