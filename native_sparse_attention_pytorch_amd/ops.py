@@ -1151,6 +1151,58 @@ def qkv_prep(qkv: Tensor, freqs: Tensor, k_positions: Tensor, v_positions: Tenso
                           int(compress_stride), int(offset))
 
 
+# ------------------------------------------------------------------ projections
+
+def _wgrad_splits(rows: int, n_in: int, n_out: int) -> int:
+    """How many slices of the token axis the weight gradient 'o i' = dy^T x is cut into.  The library's GEMM gives one work-group
+    per output tile the whole token axis: with a few dozen tiles of a small weight and tens of thousands of tokens most of the
+    256 CUs idle (measured on 16384 tokens: 1024 x 1024 weight 109 us whole, 52 us in 8 slices + the sum; 48 x 1024 99 -> 31 us;
+    a 2048 x 2048 weight over 4080 tokens has its 256 tiles already and is left whole)."""
+    tiles = -(-n_in // 128) * -(-n_out // 128)
+    s = 8
+    while s > 1 and (s * tiles > 768 or rows % s or rows // s < 1024):
+        s //= 2
+    return s if s >= 4 else 1
+
+
+class _Linear(torch.autograd.Function):
+    """F.linear whose weight gradient is a batched GEMM over slices of the token axis, summed in fp32 (see _wgrad_splits):
+    the same products as the one GEMM autograd would launch (NSA.py:583 to_qkv, 853 to_strategy_combine, 858 combine_heads)."""
+
+    @staticmethod
+    def forward(ctx, x, w, b):
+        ctx.save_for_backward(x, w)
+        ctx.has_bias = b is not None
+        return torch.nn.functional.linear(x, w, b)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        n_out, n_in = w.shape
+        dy2, x2 = dy.reshape(-1, n_out), x.reshape(-1, n_in)
+        rows = x2.shape[0]
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = (dy2 @ w).view(x.shape)
+        if ctx.needs_input_grad[1]:
+            s = _wgrad_splits(rows, n_in, n_out) if x2.is_cuda and x2.dtype in (_BF16, torch.float16) and dy2.dtype == x2.dtype else 1
+            if s > 1:
+                part = torch.bmm(dy2.view(s, rows // s, n_out).transpose(1, 2), x2.view(s, rows // s, n_in), out_dtype=torch.float32)
+                dw = part.sum(0).to(w.dtype)
+            else:
+                dw = (dy2.t() @ x2).to(w.dtype)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            db = dy2.sum(0)
+        return dx, dw, db
+
+
+def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
+    """torch.nn.functional.linear with the split weight-gradient GEMM (see _Linear)."""
+    if not (torch.is_grad_enabled() and weight.requires_grad) or torch.compiler.is_compiling() or x.dtype != weight.dtype:
+        return torch.nn.functional.linear(x, weight, bias)
+    return _Linear.apply(x, weight, bias)
+
+
 # ------------------------------------------------------------------ fp32 forward (inference)
 
 def _f32(t: Tensor) -> Tensor:

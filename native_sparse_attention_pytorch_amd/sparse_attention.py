@@ -160,6 +160,13 @@ class SparseAttention(nn.Module):
 
     # ------------------------------------------------------------------------------ pieces
 
+    @staticmethod
+    def _linear(layer, x):
+        # a plain nn.Linear without hooks goes through ops.linear (its weight gradient fills the chip); anything else is called
+        if type(layer) is nn.Linear and not (layer._forward_hooks or layer._forward_pre_hooks or layer._backward_hooks):
+            return ops.linear(x, layer.weight, layer.bias)
+        return layer(x)
+
     def _split_heads(self, t):
         b, n, hd = t.shape
         return t.view(b, n, hd // self.dim_head, self.dim_head).permute(0, 2, 1, 3)
@@ -357,7 +364,7 @@ class SparseAttention(nn.Module):
         bf16 = torch.bfloat16
 
         x = self.norm(inp)
-        qkv = self.to_qkv(x)
+        qkv = self._linear(self.to_qkv, x)
         if (self.fp32_inference_kernels and qkv.dtype == torch.float32 and not (torch.is_grad_enabled() and qkv.requires_grad)
                 and self.dim_head <= 128 and self.dim_head % 4 == 0 and not torch.compiler.is_compiling()):
             return self._forward_fp32(x, qkv, return_cache)
@@ -417,9 +424,9 @@ class SparseAttention(nn.Module):
 
         s_out = ops.sliding_attend(rq16, rk16, v16, self.sliding_window_size, causal=self.causal)
 
-        logits = self.to_strategy_combine[0](x)
+        logits = self._linear(self.to_strategy_combine[0], x)
         merged = ops.gate_combine(logits, c_out, f_out, s_out)
-        out = self.combine_heads(merged.to(x.dtype))
+        out = self._linear(self.combine_heads, merged.to(x.dtype))
 
         if not return_cache:
             return out

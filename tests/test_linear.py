@@ -1,0 +1,63 @@
+"""ops.linear: the projections' weight gradient as a GEMM over slices of the token axis.  It computes what autograd's own
+F.linear backward computes (NSA.py:583, 853, 858 are plain nn.Linear calls), so the checks are against torch itself."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from native_sparse_attention_pytorch_amd import ops
+
+
+def test_slices_by_shape():
+    assert ops._wgrad_splits(16384, 1024, 1024) == 8
+    assert ops._wgrad_splits(16384, 1024, 1536) == 8
+    assert ops._wgrad_splits(16384, 1024, 48) == 8
+    assert ops._wgrad_splits(4080, 2048, 2048) == 1        # 256 tiles already
+    assert ops._wgrad_splits(4080, 2048, 64) == 1          # too few tokens a slice
+    assert ops._wgrad_splits(4096, 1024, 1024) == 4
+    assert ops._wgrad_splits(16383, 1024, 1024) == 1       # no even cut
+    assert ops._wgrad_splits(2048, 64, 64) == 1
+
+
+def test_whole_gemm_path_equals_autograd_cpu():
+    torch.manual_seed(0)
+    x = torch.randn(3, 37, 24, requires_grad=True)
+    w = torch.randn(40, 24, requires_grad=True)
+    b = torch.randn(40, requires_grad=True)
+    dy = torch.randn(3, 37, 40)
+    ref = torch.autograd.grad(F.linear(x, w, b), (x, w, b), dy)
+    got = torch.autograd.grad(ops.linear(x, w, b), (x, w, b), dy)
+    for r, g in zip(ref, got):
+        torch.testing.assert_close(g, r, rtol=1e-5, atol=1e-5)
+    assert torch.equal(ops.linear(x, w, b), F.linear(x, w, b))
+    with torch.no_grad():
+        assert torch.equal(ops.linear(x, w), F.linear(x, w))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,n_in,n_out,bias", [(16384, 1024, 1536, False), (8192, 512, 48, True), (4096, 256, 1024, False),
+                                                  ((4, 2048), 128, 320, True)])
+def test_sliced_weight_gradient_equals_autograd(rows, n_in, n_out, bias):
+    torch.manual_seed(1)
+    dev, dt = "cuda", torch.bfloat16
+    lead = rows if isinstance(rows, tuple) else (rows,)
+    tokens = 1
+    for r in lead:
+        tokens *= r
+    assert ops._wgrad_splits(tokens, n_in, n_out) > 1
+    x = torch.randn(*lead, n_in, device=dev, dtype=dt, requires_grad=True)
+    w = (torch.randn(n_out, n_in, device=dev, dtype=dt) * n_in ** -0.5).requires_grad_()
+    b = torch.randn(n_out, device=dev, dtype=dt, requires_grad=True) if bias else None
+    dy = torch.randn(*lead, n_out, device=dev, dtype=dt)
+    ins = (x, w, b) if bias else (x, w)
+    y = ops.linear(x, w, b)
+    assert torch.equal(y, F.linear(x, w, b))
+    got = torch.autograd.grad(y, ins, dy)
+    ref = torch.autograd.grad(F.linear(x, w, b), ins, dy)
+    assert torch.equal(got[0], ref[0])                                   # the same GEMM
+    # fp32 truth of the weight gradient; both bf16 results round it once (fp32 accumulation, in a different order)
+    truth = dy.reshape(-1, n_out).float().t() @ x.detach().reshape(-1, n_in).float()
+    tol = 2 ** -8 * truth.abs().max().item()
+    assert (got[1].float() - truth).abs().max().item() <= tol
+    assert (got[1].float() - truth).abs().max().item() <= 1.05 * (ref[1].float() - truth).abs().max().item() + 1e-6
+    if bias:
+        torch.testing.assert_close(got[2], ref[2], rtol=2e-2, atol=2e-2 * tokens ** 0.5)
