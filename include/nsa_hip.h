@@ -216,6 +216,30 @@ int nsa_qkv_prep_fwd(const nsa_qkv_desc* d, const void* qkv, const float* freqs,
 int nsa_qkv_prep_bwd(const nsa_qkv_desc* d, const void* d_q16, const void* d_rq, const void* d_rk, const void* d_v16,
                      const void* d_k_windows, const void* d_v_windows, const float* freqs, void* d_qkv, void* stream);
 
+/* RMS norm over the model dimension in front of the projections.  Replaces self.norm = nn.RMSNorm(dim)
+ * (NSA.py:230, applied at NSA.py:369 and 579) and its backward.  x: bf16 [rows, dim], row stride x_row_stride
+ * elements; weight: bf16 [dim]; y, dy, dx: bf16 [rows, dim] contiguous; rstd: fp32 [rows], written by the
+ * forward and read by the backward.  y = x * rsqrt(mean(x^2) + eps) * weight in fp32, rounded once.
+ * nsa_rmsnorm_bwd: dweight (or NULL) is [dim], fp32 if dweight_fp32 else bf16, and then needs partials:
+ * fp32 [nsa_rmsnorm_partials(rows) * dim] of scratch.  dim a multiple of 8, at most 4096 (NSA_E_UNSUPPORTED
+ * otherwise). */
+int nsa_rmsnorm_partials(int64_t rows);
+int nsa_rmsnorm_fwd(int64_t rows, int32_t dim, const void* x, int64_t x_row_stride, const void* weight, float eps,
+                    void* y, float* rstd, void* stream);
+int nsa_rmsnorm_bwd(int64_t rows, int32_t dim, const void* x, int64_t x_row_stride, const void* weight, const float* rstd,
+                    const void* dy, void* dx, void* dweight, int32_t dweight_fp32, float* partials, void* stream);
+
+/* Column sums of a bf16 matrix in fp32: the bias gradient of a projection (the sum of d_out over tokens that
+ * autograd takes for the nn.Linear layers of NSA.py:244-262, 853) and the gradient of the intra-window positions
+ * (the sum of the window gradients over batch and windows, NSA.py:599-600).  Row (o, i) of group g starts at
+ * x + g * group_stride + o * outer_stride + i * inner_stride (elements) and has `cols` contiguous entries;
+ * out: [groups, cols], fp32 if out_fp32 else bf16, out[g] = sum over o < outer, i < inner.  workspace: fp32,
+ * nsa_colsum_workspace(outer * inner, cols, groups) bytes.  cols and the strides multiples of 8
+ * (NSA_E_UNSUPPORTED otherwise).  The order of the additions depends on the shape only. */
+int64_t nsa_colsum_workspace(int64_t rows, int32_t cols, int32_t groups);
+int nsa_colsum(const void* x, int32_t groups, int64_t group_stride, int64_t outer, int64_t outer_stride, int64_t inner,
+               int64_t inner_stride, int32_t cols, void* out, int32_t out_fp32, float* workspace, void* stream);
+
 /* fp32 forward of the attention branches, for fp32 modules run for inference: products, softmax and
  * accumulation in fp32 on the vector ALUs, so that the result agrees with the reference's fp32 torch path
  * to its own test tolerance (1e-5, tests/test_sparse_attn.py:86), which the bf16 MFMA kernels cannot.

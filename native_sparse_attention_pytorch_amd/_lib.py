@@ -90,6 +90,14 @@ def lib():
         L.nsa_dense_bwd.argtypes = [C.POINTER(DenseDesc)] + [vp] * 7 + [sz] + [vp] * 4
         L.nsa_topk.argtypes = [vp, C.c_int64, C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp]
         L.nsa_topk_prefix.argtypes = [vp, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp]
+        fp = C.POINTER(C.c_float)
+        L.nsa_rmsnorm_partials.argtypes = [C.c_int64]
+        L.nsa_rmsnorm_fwd.argtypes = [C.c_int64, C.c_int32, vp, C.c_int64, vp, C.c_float, vp, vp, vp]
+        L.nsa_rmsnorm_bwd.argtypes = [C.c_int64, C.c_int32, vp, C.c_int64, vp, vp, vp, vp, vp, C.c_int32, vp, vp]
+        L.nsa_colsum_workspace.argtypes = [C.c_int64, C.c_int32, C.c_int32]
+        L.nsa_colsum_workspace.restype = C.c_int64
+        L.nsa_colsum.argtypes = [vp, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int32, vp, C.c_int32, vp, vp]
+        L.nsa_rmsnorm_partials.restype = L.nsa_rmsnorm_fwd.restype = L.nsa_rmsnorm_bwd.restype = L.nsa_colsum.restype = C.c_int
         i3 = C.POINTER(C.c_int64)
         L.nsa_gate_fwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp]
         L.nsa_gate_bwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp, vp, vp, vp, vp]

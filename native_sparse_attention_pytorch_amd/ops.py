@@ -1135,8 +1135,9 @@ class _QkvPrep(torch.autograd.Function):
         dsc = _qkv_desc(dqkv, heads, kv_heads, d, block, stride, offset)
         _lib.check(_lib.lib().nsa_qkv_prep_bwd(C.byref(dsc), _ptr(dq16), _ptr(drq), _ptr(drk), _ptr(dv16), _ptr(dkw), _ptr(dvw),
                                                _ptr(freqs32), _ptr(dqkv), _stream()), "nsa_qkv_prep_bwd")
-        dkp = dkw.sum(dim=(0, 2), dtype=torch.float32).to(kp_dtype) if kp_grad and dkw is not None else None
-        dvp = dvw.sum(dim=(0, 2), dtype=torch.float32).to(vp_dtype) if vp_grad and dvw is not None else None
+        pos_grad = lambda t, dt: window_position_grad(t, dt) if colsum_supported(t) else t.sum(dim=(0, 2), dtype=torch.float32).to(dt)
+        dkp = pos_grad(dkw, kp_dtype) if kp_grad and dkw is not None else None
+        dvp = pos_grad(dvw, vp_dtype) if vp_grad and dvw is not None else None
         return dqkv, None, dkp, dvp, None, None, None, None, None, None
 
 
@@ -1149,6 +1150,100 @@ def qkv_prep(qkv: Tensor, freqs: Tensor, k_positions: Tensor, v_positions: Tenso
         raise RuntimeError("qkv_prep: needs a bf16 / fp32 device projection 'b n (h d)' with dim_head 64 or 128")
     return _QkvPrep.apply(qkv, freqs, k_positions, v_positions, int(heads), int(kv_heads), int(dim_head), int(compress_block_size),
                           int(compress_stride), int(offset))
+
+
+# ------------------------------------------------------------------ norm and column sums
+
+def colsum_supported(x: Tensor) -> bool:
+    return bool(x.is_cuda and x.dtype == _BF16 and x.shape[-1] % 8 == 0 and x.numel() > 0)
+
+
+def colsum(x: Tensor, out_dtype=None) -> Tensor:
+    """Sum of a bf16 matrix '... c' over all leading axes in fp32, one pass over the matrix (the bias gradient of a projection)."""
+    c = x.shape[-1]
+    x2 = x.reshape(-1, c)
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    out = torch.empty((c,), dtype=out_dtype or x.dtype, device=x.device)
+    L = _lib.lib()
+    ws = torch.empty((max(L.nsa_colsum_workspace(x2.shape[0], c, 1), 4) // 4,), dtype=torch.float32, device=x.device)
+    _lib.check(L.nsa_colsum(_ptr(x2), 1, 0, 1, 0, x2.shape[0], x2.stride(0), c, _ptr(out), int(out.dtype == torch.float32), _ptr(ws),
+                            _stream()), "nsa_colsum")
+    return out
+
+
+def window_position_grad(dwin: Tensor, out_dtype) -> Tensor:
+    """Gradient of the intra-window positions 'h j d' from the gradient of the windows 'b h w j d' (contiguous bf16): its sum
+    over batch and windows (NSA.py:599-600 add the positions to every window)."""
+    b, h, w, j, d = dwin.shape
+    out = torch.empty((h, j, d), dtype=torch.float32, device=dwin.device)
+    L = _lib.lib()
+    ws = torch.empty((max(L.nsa_colsum_workspace(b * w, j * d, h), 4) // 4,), dtype=torch.float32, device=dwin.device)
+    _lib.check(L.nsa_colsum(_ptr(dwin), h, dwin.stride(1), b, dwin.stride(0), w, dwin.stride(2), j * d, _ptr(out), 1, _ptr(ws), _stream()),
+               "nsa_colsum")
+    return out.to(out_dtype)
+
+
+def rms_norm_supported(x: Tensor, weight: Tensor | None) -> bool:
+    return bool(weight is not None and x.is_cuda and x.dtype == _BF16 and weight.dtype == _BF16 and x.shape[-1] % 8 == 0
+                and x.shape[-1] <= 4096 and x.numel() > 0 and weight.shape == x.shape[-1:])
+
+
+def _rms_rows(x: Tensor) -> Tensor:
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    return x2
+
+
+def _rms_fwd(x2: Tensor, weight: Tensor, eps: float):
+    rows, dim = x2.shape
+    y = torch.empty((rows, dim), dtype=_BF16, device=x2.device)
+    rstd = torch.empty((rows,), dtype=torch.float32, device=x2.device)
+    _lib.check(_lib.lib().nsa_rmsnorm_fwd(rows, dim, _ptr(x2), x2.stride(0), _ptr(weight), eps, _ptr(y), _ptr(rstd), _stream()),
+               "nsa_rmsnorm_fwd")
+    return y, rstd
+
+
+def _rms_bwd(x2: Tensor, weight: Tensor, rstd: Tensor, dy2: Tensor, want_dw: bool):
+    rows, dim = x2.shape
+    if not dy2.is_contiguous() or dy2.data_ptr() % 16:
+        dy2 = dy2.clone(memory_format=torch.contiguous_format)
+    dx = torch.empty((rows, dim), dtype=_BF16, device=x2.device)
+    dw = part = None
+    L = _lib.lib()
+    if want_dw:
+        dw = torch.empty((dim,), dtype=weight.dtype, device=x2.device)
+        part = torch.empty((L.nsa_rmsnorm_partials(rows) * dim,), dtype=torch.float32, device=x2.device)
+    _lib.check(L.nsa_rmsnorm_bwd(rows, dim, _ptr(x2), x2.stride(0), _ptr(weight), _ptr(rstd), _ptr(dy2), _ptr(dx), _ptr(dw), 0, _ptr(part),
+                                 _stream()), "nsa_rmsnorm_bwd")
+    return dx, dw
+
+
+class _RmsNorm(torch.autograd.Function):
+    """nn.RMSNorm over the last axis (NSA.py:230, 579) as one HBM-bound kernel in each direction (see nsa_rmsnorm_fwd)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        x2 = _rms_rows(x)
+        w = weight.detach().contiguous()
+        y, rstd = _rms_fwd(x2, w, eps)
+        ctx.save_for_backward(x2, w, rstd)
+        return y.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, w, rstd = ctx.saved_tensors
+        dx, dw = _rms_bwd(x2, w, rstd, dy.reshape(x2.shape), ctx.needs_input_grad[1])
+        return dx.view(dy.shape), dw, None
+
+
+def rms_norm(x: Tensor, weight: Tensor, eps: float | None = None) -> Tensor:
+    """torch.nn.functional.rms_norm(x, (dim,), weight, eps) for a bf16 device tensor.  eps None, as nn.RMSNorm(dim) has it, is
+    the machine epsilon of the type the norm is computed in - fp32 for a bf16 input, in the library's kernel as here."""
+    if not rms_norm_supported(x, weight) or torch.compiler.is_compiling():
+        return torch.nn.functional.rms_norm(x, x.shape[-1:], weight, eps)
+    return _RmsNorm.apply(x, weight, float(torch.finfo(torch.float32).eps if eps is None else eps))
 
 
 # ------------------------------------------------------------------ projections
@@ -1180,19 +1275,13 @@ class _Linear(torch.autograd.Function):
         x, w = ctx.saved_tensors
         n_out, n_in = w.shape
         dy2, x2 = dy.reshape(-1, n_out), x.reshape(-1, n_in)
-        rows = x2.shape[0]
         dx = dw = db = None
         if ctx.needs_input_grad[0]:
             dx = (dy2 @ w).view(x.shape)
         if ctx.needs_input_grad[1]:
-            s = _wgrad_splits(rows, n_in, n_out) if x2.is_cuda and x2.dtype in (_BF16, torch.float16) and dy2.dtype == x2.dtype else 1
-            if s > 1:
-                part = torch.bmm(dy2.view(s, rows // s, n_out).transpose(1, 2), x2.view(s, rows // s, n_in), out_dtype=torch.float32)
-                dw = part.sum(0).to(w.dtype)
-            else:
-                dw = (dy2.t() @ x2).to(w.dtype)
+            dw = _wgrad(dy2, x2, w.dtype)
         if ctx.has_bias and ctx.needs_input_grad[2]:
-            db = dy2.sum(0)
+            db = colsum(dy2) if colsum_supported(dy2) else dy2.sum(0)
         return dx, dw, db
 
 
@@ -1201,6 +1290,59 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
     if not (torch.is_grad_enabled() and weight.requires_grad) or torch.compiler.is_compiling() or x.dtype != weight.dtype:
         return torch.nn.functional.linear(x, weight, bias)
     return _Linear.apply(x, weight, bias)
+
+
+def _wgrad(dy2: Tensor, x2: Tensor, dtype) -> Tensor:
+    """Weight gradient 'o i' = dy2^T x2 of a projection, over slices of the token axis where that fills the chip."""
+    rows, n_in, n_out = x2.shape[0], x2.shape[1], dy2.shape[1]
+    s = _wgrad_splits(rows, n_in, n_out) if x2.is_cuda and x2.dtype in (_BF16, torch.float16) and dy2.dtype == x2.dtype else 1
+    if s > 1 and dy2.is_contiguous() and x2.is_contiguous():
+        part = torch.bmm(dy2.view(s, rows // s, n_out).transpose(1, 2), x2.view(s, rows // s, n_in), out_dtype=torch.float32)
+        return part.sum(0).to(dtype)
+    return (dy2.t() @ x2).to(dtype)
+
+
+class _NormedProjections(torch.autograd.Function):
+    """The module's front end as one node: RMS norm of the input (NSA.py:579), the fused q / k / v projection (NSA.py:583) and the
+    gate logits (NSA.py:853) of the normed input.  One node so that the two gradients of the normed input are accumulated by the
+    second GEMM (beta = 1) instead of an extra pass over them, and the norm's backward is one kernel."""
+
+    @staticmethod
+    def forward(ctx, inp, norm_w, eps, w_qkv, w_gate, b_gate):
+        x2 = _rms_rows(inp)
+        nw = norm_w.detach().contiguous()
+        xn, rstd = _rms_fwd(x2, nw, eps)
+        qkv = xn @ w_qkv.t()
+        logits = torch.addmm(b_gate, xn, w_gate.t()) if b_gate is not None else xn @ w_gate.t()
+        ctx.save_for_backward(x2, nw, rstd, xn, w_qkv, w_gate)
+        ctx.has_bias = b_gate is not None
+        lead = inp.shape[:-1]
+        return qkv.view(*lead, -1), logits.view(*lead, -1)
+
+    @staticmethod
+    def backward(ctx, dqkv, dlogits):
+        x2, nw, rstd, xn, w_qkv, w_gate = ctx.saved_tensors
+        dq2 = dqkv.reshape(-1, w_qkv.shape[0])
+        dl2 = dlogits.reshape(-1, w_gate.shape[0])
+        need = ctx.needs_input_grad
+        dinp = dnw = dwq = dwg = dbg = None
+        if need[0] or need[1]:
+            dxn = dq2 @ w_qkv
+            dxn.addmm_(dl2, w_gate)
+            dinp, dnw = _rms_bwd(x2, nw, rstd, dxn, need[1])
+            dinp = dinp.view(*dqkv.shape[:-1], -1) if need[0] else None
+        if need[3]:
+            dwq = _wgrad(dq2 if dq2.is_contiguous() else dq2.contiguous(), xn, w_qkv.dtype)
+        if need[4]:
+            dwg = _wgrad(dl2 if dl2.is_contiguous() else dl2.contiguous(), xn, w_gate.dtype)
+        if ctx.has_bias and need[5]:
+            dbg = colsum(dl2) if colsum_supported(dl2) else dl2.sum(0)
+        return dinp, dnw, None, dwq, dwg, dbg
+
+
+def normed_projections(inp: Tensor, norm_weight: Tensor, eps: float | None, w_qkv: Tensor, w_gate: Tensor, b_gate: Tensor | None):
+    """(to_qkv(norm(inp)), gate_logits(norm(inp))) for a bf16 module with gradients (see _NormedProjections)."""
+    return _NormedProjections.apply(inp, norm_weight, float(torch.finfo(torch.float32).eps if eps is None else eps), w_qkv, w_gate, b_gate)
 
 
 # ------------------------------------------------------------------ fp32 forward (inference)

@@ -160,12 +160,42 @@ class SparseAttention(nn.Module):
 
     # ------------------------------------------------------------------------------ pieces
 
-    @staticmethod
-    def _linear(layer, x):
+    @classmethod
+    def _linear(cls, layer, x):
         # a plain nn.Linear without hooks goes through ops.linear (its weight gradient fills the chip); anything else is called
-        if type(layer) is nn.Linear and not (layer._forward_hooks or layer._forward_pre_hooks or layer._backward_hooks):
-            return ops.linear(x, layer.weight, layer.bias)
-        return layer(x)
+        return ops.linear(x, layer.weight, layer.bias) if cls._plain(layer, nn.Linear) else layer(x)
+
+    @staticmethod
+    def _plain(layer, kind):
+        return type(layer) is kind and not (layer._forward_hooks or layer._forward_pre_hooks or layer._backward_hooks)
+
+    def _front_is_one_node(self, inp):
+        """Norm, qkv projection and gate logits as ops.normed_projections: a bf16 module with its default layers, under autograd."""
+        norm, qkv, gate = self.norm, self.to_qkv, self.to_strategy_combine[0]
+        if not (torch.is_grad_enabled() and inp.is_cuda and inp.dtype == torch.bfloat16 and not torch.compiler.is_compiling()):
+            return False
+        if not (self._plain(norm, nn.RMSNorm) and self._plain(qkv, nn.Linear) and self._plain(gate, nn.Linear)):
+            return False
+        if qkv.bias is not None or any(t is not None and t.dtype != torch.bfloat16 for t in (norm.weight, qkv.weight, gate.weight, gate.bias)):
+            return False
+        if tuple(norm.normalized_shape) != tuple(inp.shape[-1:]) or torch.is_autocast_enabled():
+            return False
+        return ops.rms_norm_supported(inp, norm.weight) and (inp.requires_grad or any(p.requires_grad for p in self.parameters()))
+
+    def _normed(self, x):
+        norm = self.norm
+        if self._plain(norm, nn.RMSNorm) and tuple(norm.normalized_shape) == tuple(x.shape[-1:]) and ops.rms_norm_supported(x, norm.weight):
+            return ops.rms_norm(x, norm.weight, norm.eps)
+        return norm(x)
+
+    @classmethod
+    def _compress(cls, mlp, windows):
+        # the default network (flatten, linear, relu, linear) layer by layer, so that its projections go through ops.linear
+        if not cls._plain(mlp, nn.Sequential):
+            return mlp(windows)
+        for layer in mlp:
+            windows = cls._linear(layer, windows)
+        return windows
 
     def _split_heads(self, t):
         b, n, hd = t.shape
@@ -363,9 +393,15 @@ class SparseAttention(nn.Module):
         M, G = self.num_mem_compress_kv, self.num_grouped_queries
         bf16 = torch.bfloat16
 
-        x = self.norm(inp)
-        qkv = self._linear(self.to_qkv, x)
-        if (self.fp32_inference_kernels and qkv.dtype == torch.float32 and not (torch.is_grad_enabled() and qkv.requires_grad)
+        logits = None
+        if self._front_is_one_node(inp):
+            x = None
+            qkv, logits = ops.normed_projections(inp, self.norm.weight, self.norm.eps, self.to_qkv.weight,
+                                                 self.to_strategy_combine[0].weight, self.to_strategy_combine[0].bias)
+        else:
+            x = self._normed(inp)
+            qkv = self._linear(self.to_qkv, x)
+        if (x is not None and self.fp32_inference_kernels and qkv.dtype == torch.float32 and not (torch.is_grad_enabled() and qkv.requires_grad)
                 and self.dim_head <= 128 and self.dim_head % 4 == 0 and not torch.compiler.is_compiling()):
             return self._forward_fp32(x, qkv, return_cache)
         q, k, v = qkv.split(self.qkv_split, dim=-1)
@@ -383,7 +419,7 @@ class SparseAttention(nn.Module):
             # window gather + intra-window positions in one HIP kernel per tensor (NSA.py:589-603)
             kw, vw = ops.compress_windows_pair(k.to(bf16), v.to(bf16), self.k_intrablock_positions, self.v_intrablock_positions, cbs, st)
             kw, vw = kw.to(k.dtype), vw.to(v.dtype)
-        ck0, cv0 = self.k_compress(kw), self.v_compress(vw)
+        ck0, cv0 = self._compress(self.k_compress, kw), self._compress(self.v_compress, vw)
         mem_k, mem_v = self.compress_mem_kv[0].to(ck0.dtype), self.compress_mem_kv[1].to(cv0.dtype)
         ck = torch.cat((mem_k[None].expand(b, -1, -1, -1), ck0), dim=-2)
         cv = torch.cat((mem_v[None].expand(b, -1, -1, -1), cv0), dim=-2)
@@ -424,9 +460,10 @@ class SparseAttention(nn.Module):
 
         s_out = ops.sliding_attend(rq16, rk16, v16, self.sliding_window_size, causal=self.causal)
 
-        logits = self._linear(self.to_strategy_combine[0], x)
+        if logits is None:
+            logits = self._linear(self.to_strategy_combine[0], x)
         merged = ops.gate_combine(logits, c_out, f_out, s_out)
-        out = self._linear(self.combine_heads, merged.to(x.dtype))
+        out = self._linear(self.combine_heads, merged.to(qkv.dtype))
 
         if not return_cache:
             return out

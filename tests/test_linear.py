@@ -61,3 +61,36 @@ def test_sliced_weight_gradient_equals_autograd(rows, n_in, n_out, bias):
     assert (got[1].float() - truth).abs().max().item() <= 1.05 * (ref[1].float() - truth).abs().max().item() + 1e-6
     if bias:
         torch.testing.assert_close(got[2], ref[2], rtol=2e-2, atol=2e-2 * tokens ** 0.5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("b,n,dim,n_qkv,n_gate,bias", [(2, 4096, 256, 384, 24, True), (1, 333, 128, 192, 12, False)])
+def test_front_end_as_one_node_equals_its_pieces(b, n, dim, n_qkv, n_gate, bias):
+    """norm -> (qkv projection, gate logits) as one autograd node (NSA.py:579, 583, 853) against the same three layers run one
+    by one in fp32 (the truth) and in bf16 by the library (the yardstick for the rounding)."""
+    torch.manual_seed(2)
+    dev, dt = "cuda", torch.bfloat16
+    inp = torch.randn(b, n, dim, device=dev).to(dt)
+    nw = (1 + 0.1 * torch.randn(dim, device=dev)).to(dt)
+    wq = (torch.randn(n_qkv, dim, device=dev) * dim ** -0.5).to(dt)
+    wg = (torch.randn(n_gate, dim, device=dev) * dim ** -0.5).to(dt)
+    bg = torch.randn(n_gate, device=dev).to(dt) if bias else None
+    dq = torch.randn(b, n, n_qkv, device=dev).to(dt)
+    dl = torch.randn(b, n, n_gate, device=dev).to(dt)
+
+    def pieces(cast):
+        ts = [t if t is None else cast(t).detach().requires_grad_() for t in (inp, nw, wq, wg, bg)]
+        i_, nw_, wq_, wg_, bg_ = ts
+        xn = F.rms_norm(i_, (dim,), nw_, None if cast(inp).dtype == dt else torch.finfo(torch.float32).eps)
+        qkv, lg = F.linear(xn, wq_), F.linear(xn, wg_, bg_)
+        grads = torch.autograd.grad((qkv, lg), [t for t in ts if t is not None], (cast(dq), cast(dl)))
+        return (qkv, lg), grads
+
+    ts = [t if t is None else t.clone().requires_grad_() for t in (inp, nw, wq, wg, bg)]
+    outs = ops.normed_projections(ts[0], ts[1], None, ts[2], ts[3], ts[4])
+    grads = torch.autograd.grad(outs, [t for t in ts if t is not None], (dq, dl))
+    (o32, g32), (o16, g16) = pieces(lambda t: t.float()), pieces(lambda t: t)
+    rel = lambda a, r: ((a.float() - r).norm() / r.norm().clamp_min(1e-9)).item()
+    for got, want32, want16 in zip(list(outs) + list(grads), list(o32) + list(g32), list(o16) + list(g16)):
+        assert got.shape == want32.shape and got.dtype == dt
+        assert rel(got, want32) <= max(1.2 * rel(want16, want32), 2e-3), (rel(got, want32), rel(want16, want32))
