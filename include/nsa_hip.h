@@ -237,6 +237,10 @@ int nsa_rmsnorm_bwd(int64_t rows, int32_t dim, const void* x, int64_t x_row_stri
  * nsa_colsum_workspace(outer * inner, cols, groups) bytes.  cols and the strides multiples of 8
  * (NSA_E_UNSUPPORTED otherwise).  The order of the additions depends on the shape only. */
 int64_t nsa_colsum_workspace(int64_t rows, int32_t cols, int32_t groups);
+/* out[i] = sum over p < parts of slices[p * n + i] (fp32 in; out fp32 if out_fp32 else bf16): the sum of the partial
+ * products of a weight gradient computed as a batched GEMM over slices of the token axis (the gradient autograd takes
+ * for the projections of NSA.py:583, 853, 858 in one GEMM).  n a multiple of 4 (NSA_E_UNSUPPORTED otherwise). */
+int nsa_sum_slices(const float* slices, int32_t parts, int64_t n, void* out, int32_t out_fp32, void* stream);
 int nsa_colsum(const void* x, int32_t groups, int64_t group_stride, int64_t outer, int64_t outer_stride, int64_t inner,
                int64_t inner_stride, int32_t cols, void* out, int32_t out_fp32, float* workspace, void* stream);
 

@@ -97,6 +97,8 @@ def lib():
         L.nsa_colsum_workspace.argtypes = [C.c_int64, C.c_int32, C.c_int32]
         L.nsa_colsum_workspace.restype = C.c_int64
         L.nsa_colsum.argtypes = [vp, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int32, vp, C.c_int32, vp, vp]
+        L.nsa_sum_slices.argtypes = [vp, C.c_int32, C.c_int64, vp, C.c_int32, vp]
+        L.nsa_sum_slices.restype = C.c_int
         L.nsa_rmsnorm_partials.restype = L.nsa_rmsnorm_fwd.restype = L.nsa_rmsnorm_bwd.restype = L.nsa_colsum.restype = C.c_int
         i3 = C.POINTER(C.c_int64)
         L.nsa_gate_fwd.argtypes = [C.c_int32] * 4 + [vp, vp, i3, vp, i3, vp, i3, vp, vp]

@@ -123,33 +123,68 @@ struct ColsumArgs {
 
 // partial[g][blockIdx.x][cols] = sum of this work-group's rows of group g
 __global__ __launch_bounds__(256) void colsum_kernel(const ColsumArgs A, const __bf16* __restrict__ x, float* __restrict__ partial) {
-  __shared__ float red[256][9];
+  __shared__ float red[8][256];
   const int cl = threadIdx.x % A.lpr, rl = threadIdx.x / A.lpr, rpi = 256 / A.lpr;
   const int col = (blockIdx.y * A.lpr + cl) * 8;
   const bool in = col < A.cols;
-  const long first = (long)blockIdx.x * A.chunk, last = min(first + A.chunk, A.rows);
+  const long first = (long)blockIdx.x * A.chunk + rl, last = min((long)blockIdx.x * A.chunk + A.chunk, A.rows);
   const __bf16* base = x + blockIdx.z * A.sg + col;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  if (in) {
-#pragma unroll 8
-    for (long r = first + rl; r < last; r += rpi) {
-      const bf16x8 t = load8(base + (r / A.r1) * A.s0 + (r % A.r1) * A.s1);
+  if (in && first < last) {
+    // rows are walked as (outer, inner) pairs: one division up front, none in the loop
+    long o = first / A.r1, i = first - o * A.r1;
+    const int count = (int)((last - first + rpi - 1) / rpi);
+#pragma unroll 4
+    for (int it = 0; it < count; ++it) {
+      const bf16x8 t = load8(base + o * A.s0 + i * A.s1);
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] += (float)t[e];
+      i += rpi;
+      while (i >= A.r1) { i -= A.r1; ++o; }
     }
   }
+  float* out = partial + ((long)blockIdx.z * gridDim.x + blockIdx.x) * A.cols + col;
+  if (rpi == 1) {
+    if (in) {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) red[threadIdx.x][e] = acc[e];
-  __syncthreads();
+      for (int e = 0; e < 8; ++e) out[e] = acc[e];
+    }
+    return;
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) red[e][threadIdx.x] = acc[e];
+  for (int half = rpi / 2; half >= 1; half /= 2) {               // rows rl and rl + half of the same columns
+    __syncthreads();
+    if (rl < half) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) red[e][threadIdx.x] += red[e][threadIdx.x + half * A.lpr];
+    }
+  }
   if (rl == 0 && in) {
-    float* out = partial + ((long)blockIdx.z * gridDim.x + blockIdx.x) * A.cols + col;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float s = 0.f;
-      for (int j = 0; j < rpi; ++j) s += red[j * A.lpr + cl][e];
-      out[e] = s;
-    }
+    for (int e = 0; e < 8; ++e) out[e] = red[e][threadIdx.x];
   }
+}
+
+// out[i] = sum over p < parts of slices[p][i], four entries a thread (the split weight-gradient GEMM's partial products)
+template <class OT>
+__global__ __launch_bounds__(256) void sum_slices_kernel(const float* __restrict__ slices, int parts, long n, OT* __restrict__ out) {
+  const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= n) return;
+  float4 a = *reinterpret_cast<const float4*>(slices + i);
+  int p = 1;
+  for (; p + 3 < parts; p += 4) {
+    float4 t[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = *reinterpret_cast<const float4*>(slices + (long)(p + j) * n + i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { a.x += t[j].x; a.y += t[j].y; a.z += t[j].z; a.w += t[j].w; }
+  }
+  for (; p < parts; ++p) {
+    const float4 t = *reinterpret_cast<const float4*>(slices + (long)p * n + i);
+    a.x += t.x; a.y += t.y; a.z += t.z; a.w += t.w;
+  }
+  out[i] = (OT)a.x; out[i + 1] = (OT)a.y; out[i + 2] = (OT)a.z; out[i + 3] = (OT)a.w;
 }
 
 // out[g][col] = sum over p of partial[g][p][col]; 32 columns x 32 slices of p a work-group, 8 loads in flight a thread
@@ -210,7 +245,7 @@ extern "C" int nsa_rmsnorm_fwd(int64_t rows, int32_t dim, const void* x, int64_t
   if (!nv || dim % 8 || x_row_stride % 8 || x_row_stride < dim || ((uintptr_t)x | (uintptr_t)weight | (uintptr_t)y) % 16)
     return NSA_E_UNSUPPORTED;
   hipStream_t st = (hipStream_t)stream;
-  const int grid = norm_groups(rows);
+  const int grid = (int)std::min<long>((rows + 3) / 4, 2048);
 #define NSA_FWD(NV) rmsnorm_fwd_kernel<NV><<<grid, 256, 0, st>>>(rows, dim, x_row_stride, (const __bf16*)x, (const __bf16*)weight, eps, (__bf16*)y, rstd)
   switch (nv) { case 1: NSA_FWD(1); break; case 2: NSA_FWD(2); break; case 4: NSA_FWD(4); break; default: NSA_FWD(8); }
 #undef NSA_FWD
@@ -278,4 +313,16 @@ extern "C" int nsa_colsum(const void* x, int32_t groups, int64_t group_stride, i
   colsum_kernel<<<dim3(s.parts, s.colblocks, groups), 256, 0, st>>>(A, (const __bf16*)x, workspace);
   if (hipError_t e = hipGetLastError()) return (int)e;
   return reduce_launch(workspace, groups, s.parts, cols, out, out_fp32, st);
+}
+
+extern "C" int nsa_sum_slices(const float* slices, int32_t parts, int64_t n, void* out, int32_t out_fp32, void* stream) {
+  if (parts <= 0 || n < 0) return NSA_E_ARG;
+  if (n == 0) return 0;
+  if (!slices || !out) return NSA_E_ARG;
+  if (n % 4 || (uintptr_t)slices % 16 || (uintptr_t)out % 8 || n > ((int64_t)1 << 40)) return NSA_E_UNSUPPORTED;
+  hipStream_t st = (hipStream_t)stream;
+  const unsigned grid = (unsigned)((n / 4 + 255) / 256);
+  if (out_fp32) sum_slices_kernel<float><<<grid, 256, 0, st>>>(slices, parts, n, (float*)out);
+  else sum_slices_kernel<__bf16><<<grid, 256, 0, st>>>(slices, parts, n, (__bf16*)out);
+  return (int)hipGetLastError();
 }

@@ -169,11 +169,14 @@ def _select_setup(ctx, inputs, output):
     out, lse, index_ws = output
     ctx.save_for_backward(q, k, v, out, lse, idx, fmask, index_ws)
     ctx.args = (block, causal, scale, sel_scale is not None and sel_scale.requires_grad, None if sel_scale is None else sel_scale.dtype)
+    ctx.set_materialize_grads(False)          # no zero tensors for the unused gradients of lse and the index workspace
 
 
 def _select_backward(ctx, dout, dlse, dws):
     q, k, v, out, lse, idx, fmask, index_ws = ctx.saved_tensors
     block, causal, scale, want, sdtype = ctx.args
+    if dout is None:
+        return (None,) * 9
     dq, dk, dv, dsel = select_bwd(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale, want)
     return dq, dk, dv, None, None, (dsel.to(sdtype) if want else None), None, None, None
 
@@ -395,7 +398,8 @@ def _dense_backward(ctx, dout, dlse, dpooled):
         # the compressed keys are few and every one of their gradients is summed over all windows into the compression
         # network's parameters: they leave the kernel as fp32 and are rounded to the keys' dtype once, after the
         # importance term has been added
-        dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale, mode == 1)
+        dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale,
+                               mode == 1 and dpooled is not None and dpooled.numel() > 0)
     if dpooled is not None and dpooled.numel() > 0:
         dq2, dk2 = _importance_backward(q, k, dpooled, num_mem, stride, sel_block, share, scale)
         dq = dq2.to(q.dtype) if dq is None else (dq.float() + dq2).to(q.dtype)
@@ -1241,7 +1245,7 @@ class _RmsNorm(torch.autograd.Function):
 def rms_norm(x: Tensor, weight: Tensor, eps: float | None = None) -> Tensor:
     """torch.nn.functional.rms_norm(x, (dim,), weight, eps) for a bf16 device tensor.  eps None, as nn.RMSNorm(dim) has it, is
     the machine epsilon of the type the norm is computed in - fp32 for a bf16 input, in the library's kernel as here."""
-    if not rms_norm_supported(x, weight) or torch.compiler.is_compiling():
+    if not rms_norm_supported(x, weight) or torch.compiler.is_compiling() or torch.is_autocast_enabled():
         return torch.nn.functional.rms_norm(x, x.shape[-1:], weight, eps)
     return _RmsNorm.apply(x, weight, float(torch.finfo(torch.float32).eps if eps is None else eps))
 
@@ -1287,7 +1291,8 @@ class _Linear(torch.autograd.Function):
 
 def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
     """torch.nn.functional.linear with the split weight-gradient GEMM (see _Linear)."""
-    if not (torch.is_grad_enabled() and weight.requires_grad) or torch.compiler.is_compiling() or x.dtype != weight.dtype:
+    if (not (torch.is_grad_enabled() and weight.requires_grad) or torch.compiler.is_compiling() or x.dtype != weight.dtype
+            or torch.is_autocast_enabled()):               # under autocast the library casts the operands itself
         return torch.nn.functional.linear(x, weight, bias)
     return _Linear.apply(x, weight, bias)
 
@@ -1298,7 +1303,11 @@ def _wgrad(dy2: Tensor, x2: Tensor, dtype) -> Tensor:
     s = _wgrad_splits(rows, n_in, n_out) if x2.is_cuda and x2.dtype in (_BF16, torch.float16) and dy2.dtype == x2.dtype else 1
     if s > 1 and dy2.is_contiguous() and x2.is_contiguous():
         part = torch.bmm(dy2.view(s, rows // s, n_out).transpose(1, 2), x2.view(s, rows // s, n_in), out_dtype=torch.float32)
-        return part.sum(0).to(dtype)
+        if dtype not in (_BF16, torch.float32) or (n_out * n_in) % 4:
+            return part.sum(0).to(dtype)
+        dw = torch.empty((n_out, n_in), dtype=dtype, device=x2.device)
+        _lib.check(_lib.lib().nsa_sum_slices(_ptr(part), s, n_out * n_in, _ptr(dw), int(dtype == torch.float32), _stream()), "nsa_sum_slices")
+        return dw
     return (dy2.t() @ x2).to(dtype)
 
 

@@ -420,7 +420,7 @@ class SparseAttention(nn.Module):
             kw, vw = ops.compress_windows_pair(k.to(bf16), v.to(bf16), self.k_intrablock_positions, self.v_intrablock_positions, cbs, st)
             kw, vw = kw.to(k.dtype), vw.to(v.dtype)
         ck0, cv0 = self._compress(self.k_compress, kw), self._compress(self.v_compress, vw)
-        mem_k, mem_v = self.compress_mem_kv[0].to(ck0.dtype), self.compress_mem_kv[1].to(cv0.dtype)
+        mem_k, mem_v = self.compress_mem_kv.to(ck0.dtype).unbind(0)       # unbind: its backward is one stack, not two zero-filled slices
         ck = torch.cat((mem_k[None].expand(b, -1, -1, -1), ck0), dim=-2)
         cv = torch.cat((mem_v[None].expand(b, -1, -1, -1), cv0), dim=-2)
         nc = ck0.shape[-2]

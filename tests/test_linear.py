@@ -94,3 +94,16 @@ def test_front_end_as_one_node_equals_its_pieces(b, n, dim, n_qkv, n_gate, bias)
     for got, want32, want16 in zip(list(outs) + list(grads), list(o32) + list(g32), list(o16) + list(g16)):
         assert got.shape == want32.shape and got.dtype == dt
         assert rel(got, want32) <= max(1.2 * rel(want16, want32), 2e-3), (rel(got, want32), rel(want16, want32))
+
+
+@pytest.mark.gpu
+def test_under_autocast_the_library_layer_runs():
+    torch.manual_seed(3)
+    x = torch.randn(4096, 64, device="cuda", requires_grad=True)
+    w = torch.randn(32, 64, device="cuda", requires_grad=True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = ops.linear(x, w)
+        ref = F.linear(x, w)
+    assert y.dtype == torch.bfloat16 and torch.equal(y, ref)
+    gx, gw = torch.autograd.grad(y.float().sum(), (x, w))
+    assert gx.dtype == torch.float32 and gw.dtype == torch.float32

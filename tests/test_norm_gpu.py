@@ -123,3 +123,20 @@ def test_colsum_limits_through_the_abi():
     torch.cuda.synchronize()
     assert torch.equal(out, torch.full_like(out, 4.0))
     assert L.nsa_colsum_workspace(4, 16, 1) >= 4 * 16
+
+
+@pytest.mark.parametrize("parts,shape,out_dtype", [(8, (1024, 1024), BF), (8, (48, 1024), BF), (4, (64, 2048), torch.float32), (1, (4, 4), BF),
+                                                   (7, (33, 12), BF)])
+def test_sum_slices(parts, shape, out_dtype):
+    torch.manual_seed(parts)
+    L = _lib.lib()
+    sl = torch.randn(parts, *shape, device="cuda")
+    out = torch.empty(shape, device="cuda", dtype=out_dtype)
+    n = shape[0] * shape[1]
+    assert L.nsa_sum_slices(C.c_void_p(sl.data_ptr()), parts, n, C.c_void_p(out.data_ptr()), int(out_dtype == torch.float32), None) == 0
+    torch.cuda.synchronize()
+    truth = sl.double().sum(0)
+    tol = (1e-6 if out_dtype == torch.float32 else 2 ** -8) * truth.abs() + 1e-6 * sl.double().abs().sum(0)
+    assert ((out.double() - truth).abs() <= tol).all()
+    assert L.nsa_sum_slices(C.c_void_p(sl.data_ptr()), parts, 6, C.c_void_p(out.data_ptr()), 0, None) == -2      # n not a multiple of 4
+    assert L.nsa_sum_slices(C.c_void_p(sl.data_ptr()), 0, n, C.c_void_p(out.data_ptr()), 0, None) == -1
