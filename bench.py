@@ -252,7 +252,7 @@ def main():
                                         # (delta + dQ + dK/dV + reduce kernels together) over the HIP-event time of each call
                                         roofline=dict(bound="mfma", peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
                                                       fwd=dict(kernel="dense_fwd_kernel<128,4>", achieved=round(cf, 2), frac=round(cf / MFMA_PEAK_TFLOPS, 4)),
-                                                      bwd=dict(kernel="dense_bwd_dq_kernel<128> + dense_bwd_dkv_kernel<128>", achieved=round(cb, 2),
+                                                      bwd=dict(kernel="dense_bwd_dq_kernel<128> + dense_bwd_dkv_pipe_kernel<128>", achieved=round(cb, 2),
                                                                frac=round(cb / MFMA_PEAK_TFLOPS, 4)),
                                                       # bytes: the visible prefix of every row (row i: i // B logits) + the outputs
                                                       topk=dict(bound="hbm", bytes=int(topk_bytes),

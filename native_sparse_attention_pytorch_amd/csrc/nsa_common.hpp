@@ -12,6 +12,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 typedef __attribute__((__vector_size__(8 * sizeof(float)))) float floatx8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t uintx4;
+typedef __attribute__((__vector_size__(4 * sizeof(int)))) int intx4;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t uintx2;
 
 constexpr float kLog2e = 1.4426950408889634f;

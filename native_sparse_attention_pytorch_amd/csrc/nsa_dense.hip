@@ -566,6 +566,9 @@ static inline unsigned dkv_grid(const DensePlan& P) {
 #ifndef NSA_DKV_AHEAD
 #define NSA_DKV_AHEAD 3
 #endif
+#ifndef NSA_DKV_PIPE_MIN_D
+#define NSA_DKV_PIPE_MIN_D 128    // head dimensions from here on take dense_bwd_dkv_pipe_kernel (one wave per SIMD)
+#endif
 #ifndef NSA_DKV_STAGES
 #define NSA_DKV_STAGES 1      // measured on MI355X (compressed branch, seq 32k, d 128): 1, 2 or 3 tiles ahead all 4.7 ms
 #endif
@@ -742,6 +745,267 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_kernel(const DensePlan P, c
     }
 }
 
+// The same walk for head dimensions whose accumulators leave room for one wave per SIMD only (d = 128: 128 registers of dK / dV
+// accumulators, 64 of K / V operands).  With one wave per SIMD nothing overlaps a wave's MFMAs but its own instruction order,
+// so the step is laid out by hand and fenced (cycle stamps of the kernel above at d = 128: 23 % of a step in the tile's LDS
+// write, 11 % in two barriers, 6 % issuing loads, and the softmax entirely outside the MFMA runs):
+//   * the tile's arithmetic is six runs of MFMAs in dependency order - S = Q K^T, dP = dO V^T, dV from rows 0-15, dV from rows
+//     16-31, dK from rows 0-15, dK from rows 16-31 - and the softmax is dealt out in slices beside the MFMAs of the run
+//     before the one that needs the slice's result (p of rows 0-15 beside dP, p of rows 16-31 beside the first dV run, ...);
+//   * the Q / dO tile is double-buffered in LDS: the next tile goes from its staging registers to the other buffer beside the
+//     S MFMAs, each row's staging register is reloaded with the tile after that right behind its store, and one barrier per
+//     step is left, which stands before the last run (see the loop).
+template <int D>
+__global__ __launch_bounds__(128) void dense_bwd_dkv_pipe_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+                                                                 const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
+                                                                 const float* __restrict__ lse, const float* __restrict__ delta,
+                                                                 float* __restrict__ part) {
+  constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
+  __shared__ __align__(16) float lse_s[2][32];
+  __shared__ __align__(16) float del_s[2][32];
+  __shared__ __align__(16) int lo_s[2][32];
+  __shared__ __align__(16) int hi_s[2][32];
+  __shared__ __align__(16) __bf16 tile_s[2][2][32 * RS];        // [buffer][Q rows | dO rows]: one array, so that a read's address
+                                                                 // is one lane-dependent base per buffer + an immediate
+  const int kt = threadIdx.x >> 6, lane = threadIdx.x & 63, n_ = lane & 31, h = lane >> 5;
+  const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
+  int T, c, qlo, qhi, c0, c1;
+  if (!chunk_of(P, blockIdx.x, T, c, qlo, qhi, c0, c1)) return;
+  if (c0 >= c1) return;
+
+  const int kr_ = kBK * T + 32 * kt + n_;                // this lane's row of k/v
+  const bool kok = kr_ < P.krows;
+  bf16x8 Kf[KS], Vf[KS];
+  {
+    const long krow = kok ? kr_ : 0;
+    const __bf16* kp = k + b * P.sk[0] + hk * P.sk[1] + krow * P.sk[2] + 8 * h;
+    const __bf16* vp = v + b * P.sv[0] + hk * P.sv[1] + krow * P.sv[2] + 8 * h;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      Kf[ks] = kok ? load8(kp + 16 * ks) : zero_frag();
+      Vf[ks] = kok ? load8(vp + 16 * ks) : zero_frag();
+    }
+  }
+  floatx16 dKa[DT], dVa[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) { dKa[dt] = zero_acc(); dVa[dt] = zero_acc(); }
+  const float sc = P.scale * kLog2e;
+  const int ppt = 32 >> P.lg;
+  const int pq = n_ >> P.lg, g = n_ & (P.g - 1);
+  const int hq = hk * P.g + g;
+  constexpr int CPR = D / 8, RPI = 64 / CPR, NT = 32 / RPI;
+  static_assert(NT == KS, "one staged row group beside every S MFMA");
+
+  // wave 0 stages the tile's Q rows, wave 1 its dO rows, through buffer loads: the descriptor starts at the tile's first
+  // query of this kv head's query heads and ends with the last row of the last of them, so a lane's offset is the same in
+  // every step (no address arithmetic in the loop) and rows past the end of the sequence read as zeros instead of needing
+  // a clamp (the launcher checks that the heads of a group span less than 2^31 elements).
+  const int ktu = __builtin_amdgcn_readfirstlane(kt);
+  const __bf16* slab = ktu == 0 ? q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1] : dout + b * P.sdo[0] + (long)(hk * P.g) * P.sdo[1];
+  const long sh = ktu == 0 ? P.sq[1] : P.sdo[1], sn = ktu == 0 ? P.sq[2] : P.sdo[2];
+  const long extent = (long)(P.g - 1) * sh + (long)(P.n - 1) * sn + D;            // elements from slab to the end of its last row
+  const long srow0 = ((long)b * P.hkv * P.g + hq) * P.n;
+  unsigned voff[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int rr = t * RPI + lane / CPR;
+    voff[t] = 2u * (unsigned)((long)(rr & (P.g - 1)) * sh + (long)(rr >> P.lg) * sn + 8 * (lane % CPR));
+  }
+  bf16x8 raw[NT];
+  float lse_r, del_r;
+  __amdgpu_buffer_rsrc_t rows_of_tile;
+  auto aim_rows = [&](int i0) {
+    const long first = min((long)i0 * sn, extent);
+    rows_of_tile = __builtin_amdgcn_make_buffer_rsrc((void*)(slab + first), 0, (int)(2 * (extent - first)), 0x00020000);
+  };
+  auto load_rows = [&](int t) {
+    raw[t] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(rows_of_tile, (int)voff[t], 0, 0));
+  };
+  // Per-row scalars of a tile: wave 0 stages log-sum-exp and delta (buffer loads again: one descriptor per array, moved along
+  // with the tile), wave 1 the bounds of the rows' visible ranges - and those only for tiles that are not visible as a whole
+  // to all 64 key rows, the others never read them.  Split like this the two waves carry about the same number of
+  // instructions per step, which at one wave per SIMD is what a step costs.
+  const float* lse_slab = lse + ((long)b * P.hkv + hk) * P.g * (long)P.n;
+  const float* del_slab = delta + ((long)b * P.hkv + hk) * P.g * (long)P.n;
+  const long rows_slab = (long)P.g * P.n;
+  const int soff = 4 * (g * P.n + pq);
+  __amdgpu_buffer_rsrc_t lse_of_tile, del_of_tile;
+  auto load_smalls = [&](int i0) {
+    if (ktu == 0) {
+      const long first = min((long)i0, rows_slab);
+      lse_of_tile = __builtin_amdgcn_make_buffer_rsrc((void*)(lse_slab + first), 0, (int)(4 * (rows_slab - first)), 0x00020000);
+      del_of_tile = __builtin_amdgcn_make_buffer_rsrc((void*)(del_slab + first), 0, (int)(4 * (rows_slab - first)), 0x00020000);
+      lse_r = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(lse_of_tile, soff, 0, 0));
+      del_r = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(del_of_tile, soff, 0, 0));
+    }
+  };
+  const int t0 = kBK * T;
+  auto whole_tile_visible = [&](int i0) {
+    const Interval vf = visible_range(P, min(i0, P.n - 1)), vl = visible_range(P, min(i0 + ppt - 1, P.n - 1));
+    const int all_lo = P.mode == 0 ? vl.lo : 0, all_hi = P.mode == 0 ? vf.hi : vf.hi + P.mem;
+    return t0 >= all_lo && t0 + kBK - 1 <= all_hi;
+  };
+  auto store_rows = [&](int t, int buf) {
+    __bf16* dst = tile_s[buf][kt];
+    *reinterpret_cast<bf16x8*>(dst + (t * RPI + lane / CPR) * RS + 8 * (lane % CPR)) = raw[t];
+  };
+  auto store_smalls = [&](int i0, int buf) {
+    if (ktu == 0) {
+      if (h == 0) {
+        lse_s[buf][n_] = i0 + pq < c1 ? lse_r * kLog2e : INFINITY;   // +inf: a padding row gets p = 0
+        del_s[buf][n_] = del_r;
+      }
+    } else if (!whole_tile_visible(i0)) {
+      if (h == 0) {
+        const Interval me = visible_range(P, min(i0 + pq, P.n - 1));
+        lo_s[buf][n_] = P.mode == 0 ? me.lo : 0;
+        hi_s[buf][n_] = P.mode == 0 ? me.hi : me.hi + P.mem;
+      }
+    }
+  };
+  // tile c0 into buffer 0, tile c0 + ppt into the staging registers
+  aim_rows(c0);
+#pragma unroll
+  for (int t = 0; t < NT; ++t) load_rows(t);
+  load_smalls(c0);
+#pragma unroll
+  for (int t = 0; t < NT; ++t) store_rows(t, 0);
+  store_smalls(c0, 0);
+  aim_rows(c0 + ppt);
+#pragma unroll
+  for (int t = 0; t < NT; ++t) load_rows(t);
+  load_smalls(c0 + ppt);
+  __syncthreads();
+
+  // The step's barrier stands before the tile's last run of MFMAs (dK from rows 16-31), not behind it: that run's operands
+  // are read from LDS before the barrier and the run itself is carried into the next step, where its MFMAs cover the round
+  // trips of the next tile's first LDS reads (cycle stamps: 490 of 2650 ticks of a step passed between the barrier and the
+  // first MFMA).  Carried across: the run's B operand Sf1c, its A operands opc[], and whether the next tile needs the mask.
+  bf16x8 Sf1c = zero_frag(), opc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) opc[dt] = zero_frag();
+  const int r0 = kBK * T + 32 * __builtin_amdgcn_readfirstlane(kt);
+  auto unmasked_at = [&](int i0) {
+    // rows of this wave are visible to every query of the tile iff they lie between the largest lower
+    // and the smallest upper bound, which consecutive queries take at the tile's ends (wave-uniform)
+    const Interval vf = visible_range(P, min(i0, P.n - 1)), vl = visible_range(P, min(i0 + ppt - 1, P.n - 1));
+    const int all_lo = P.mode == 0 ? vl.lo : 0, all_hi = P.mode == 0 ? vf.hi : vf.hi + P.mem;
+    return r0 >= all_lo && r0 + 31 <= all_hi;
+  };
+  bool unmasked = unmasked_at(c0);
+  int buf = 0;
+  for (int i0 = c0; i0 < c1; i0 += ppt, buf ^= 1) {
+    const __bf16* xq = tile_s[buf][0];
+    const __bf16* xg = tile_s[buf][1];
+    aim_rows(i0 + 2 * ppt);
+    {
+      constexpr int N = 2 * KS + 3 * DT, AH = NSA_DKV_AHEAD;
+      auto rd = [&](int i) {
+        if (i < KS) return lds_row_operand(xq, RS, i, lane);
+        if (i < 2 * KS) return lds_row_operand(xg, RS, i - KS, lane);
+        const int j = i - 2 * KS, run = j / DT, dt = j % DT;
+        return lds_transposed_operand(run < 2 ? xg : xq, RS, 16 * (run & 1), 32 * dt, lane);
+      };
+      // this tile's first reads, then the carried run
+      bf16x8 ring[AH + 1];
+#pragma unroll
+      for (int i = 0; i < AH; ++i) ring[i] = rd(i);
+      floatx4 l4[4], d4[4];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) l4[a] = *reinterpret_cast<const floatx4*>(&lse_s[buf][8 * a + 4 * h]);
+      // One copy of the step for all tiles (two copies, with and without the mask, cost the register allocator 150 registers).
+      // The mask costs the arithmetic nothing: a row that must not see this lane's key gets +inf for its log-sum-exp, so its
+      // exponent is -inf and p = 0; only tiles at an edge of the visible range read the bounds and patch l4.
+      if (!unmasked) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const intx4 lo = *reinterpret_cast<const intx4*>(&lo_s[buf][8 * a + 4 * h]);
+          const intx4 hi = *reinterpret_cast<const intx4*>(&hi_s[buf][8 * a + 4 * h]);
+#pragma unroll
+          for (int bb = 0; bb < 4; ++bb) l4[a][bb] = ((kr_ >= lo[bb]) & (kr_ <= hi[bb])) ? l4[a][bb] : INFINITY;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        dKa[dt] = mfma32(opc[dt], Sf1c, dKa[dt]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      floatx16 Sa = zero_acc(), Pa = zero_acc();
+      bf16x8 Pf0, Pf1, Sf0, Sf1;
+      // softmax slices: p (from S) for this lane's rows first .. first + count - 1, then dS (from p and dP, in dP's place)
+      auto soft1 = [&](int first, int count) {
+#pragma unroll
+        for (int e = 0; e < count; ++e) {
+          const int i2 = first + e, a = i2 >> 2, bb = i2 & 3;
+          Sa[i2] = fast_exp2(__builtin_fmaf(Sa[i2], sc, -l4[a][bb]));
+        }
+        if (first + count == 8) Pf0 = pack8(Sa, 0);
+        if (first + count == 16) Pf1 = pack8(Sa, 8);
+      };
+      auto soft2 = [&](int first, int count) {
+#pragma unroll
+        for (int e = 0; e < count; ++e) {
+          const int i2 = first + e, a = i2 >> 2, bb = i2 & 3;
+          Pa[i2] = Sa[i2] * (Pa[i2] - d4[a][bb]);
+        }
+        if (first + count == 8) Sf0 = pack8(Pa, 0);
+        if (first + count == 16) Sf1 = pack8(Pa, 8);
+      };
+      constexpr int EA = 8 / KS, EB = 8 / DT;
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        if (i + AH < N) ring[(i + AH) % (AH + 1)] = rd(i + AH);
+        const bf16x8 a = ring[i % (AH + 1)];
+        if (i < KS) {
+          Sa = mfma32(a, Kf[i], Sa);                                  // [row][key]: lane <-> key, registers <-> rows
+          store_rows(i, buf ^ 1);                                     // next tile: registers -> the other buffer,
+          load_rows(i);                                               // the tile after it -> the freed registers
+        } else if (i < 2 * KS) {
+          Pa = mfma32(a, Vf[i - KS], Pa);
+          soft1(EA * (i - KS), EA);
+        } else {
+          const int j = i - 2 * KS, run = j / DT, dt = j % DT;
+          if (run == 0) {
+            dVa[dt] = mfma32(a, Pf0, dVa[dt]);
+            soft1(8 + EB * dt, EB);
+            if (dt == 0) {
+#pragma unroll
+              for (int a2 = 0; a2 < 4; ++a2) d4[a2] = *reinterpret_cast<const floatx4*>(&del_s[buf][8 * a2 + 4 * h]);
+            }
+          }
+          else if (run == 1) { dVa[dt] = mfma32(a, Pf1, dVa[dt]); soft2(EB * dt, EB); }
+          else {
+            dKa[dt] = mfma32(a, Sf0, dKa[dt]);
+            soft2(8 + EB * dt, EB);
+            opc[dt] = lds_transposed_operand(xq, RS, 16, 32 * dt, lane);       // the carried run's operands
+            if (dt == 0) { store_smalls(i0 + ppt, buf ^ 1); load_smalls(i0 + 2 * ppt); }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      Sf1c = Sf1;
+    }
+    unmasked = unmasked_at(i0 + ppt);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) dKa[dt] = mfma32(opc[dt], Sf1c, dKa[dt]);
+  // partial [bh][tile][chunk][2][64][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][row 32kt + n_]
+  float* pk = part + (((size_t)bh * P.key_tiles + T) * P.chunks + c) * (2 * kBK * D) + (size_t)(32 * kt + n_) * D + 4 * h;
+  float* pv = pk + kBK * D;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      floatx4 x, y;
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) { x[bb] = dKa[dt][4 * a + bb]; y[bb] = dVa[dt][4 * a + bb]; }
+      *reinterpret_cast<floatx4*>(pk + 32 * dt + 8 * a) = x;
+      *reinterpret_cast<floatx4*>(pv + 32 * dt + 8 * a) = y;
+    }
+}
+
 template <int D>
 __global__ __launch_bounds__(256) void dense_bwd_dkv_reduce_kernel(const DensePlan P, const float* __restrict__ part, void* __restrict__ dk, void* __restrict__ dv) {
   const int T = blockIdx.x, bh = blockIdx.y;
@@ -829,8 +1093,13 @@ static int dense_bwd_launch(const DensePlan& P, const void* q, const void* k, co
   hipLaunchKernelGGL((dense_bwd_dq_kernel<D>), dim3(P.mode == 0 ? xcd_grid_for((P.n + qpw - 1) / qpw) : (unsigned)((P.n + qpw - 1) / qpw), P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, (const __bf16*)out, (const __bf16*)dout, lse, delta, (__bf16*)dq);      // also writes delta
   NSA_LAUNCH_CHECK();
-  hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
-                     (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
+  const auto group_span = [&](const long* st) { return (long)(P.g - 1) * st[1] + (long)(P.n - 1) * st[2] + D; };
+  if (D >= NSA_DKV_PIPE_MIN_D && group_span(P.sq) < (1l << 30) && group_span(P.sdo) < (1l << 30))
+    hipLaunchKernelGGL((dense_bwd_dkv_pipe_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+                       (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
+  else
+    hipLaunchKernelGGL((dense_bwd_dkv_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+                       (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
   NSA_LAUNCH_CHECK();
   hipLaunchKernelGGL((dense_bwd_dkv_reduce_kernel<D>), dim3(P.key_tiles, P.bh), dim3(256), 0, st, P, part, dk, dv);
   NSA_LAUNCH_CHECK();

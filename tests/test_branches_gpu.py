@@ -228,6 +228,28 @@ def test_dense_strided_views_equal_contiguous(d):
             assert torch.equal(a, b_)
 
 
+def test_dense_backward_with_query_heads_2gb_apart():
+    """The d = 128 dK / dV kernel stages its Q / dO rows through buffer loads whose 32-bit offsets span the query heads of one
+    kv head; heads further apart than that take the kernel with 64-bit addresses.  Same gradients either way."""
+    from native_sparse_attention_pytorch_amd import ops
+    hq, hk, n, d = 2, 1, 200, 128
+    g = torch.Generator().manual_seed(9)
+    far = (1 << 30) + 64
+    big = torch.empty(far + n * d, dtype=torch.bfloat16, device=DEV)
+    q = big.as_strided((1, hq, n, d), (0, far, d, 1))
+    qc = _rand((1, hq, n, d), g, d ** -0.5).cuda()
+    q.copy_(qc)
+    k, v = _rand((1, hk, n, d), g, d ** -0.5).cuda(), _rand((1, hk, n, d), g).cuda()
+    do = _rand((1, hq, n, d), g).cuda()
+    o1, l1, _ = ops.dense_fwd(q, k, v, 0, True, 64, 1, 0, False, 1, True, d ** -0.5)
+    o2, l2, _ = ops.dense_fwd(qc, k, v, 0, True, 64, 1, 0, False, 1, True, d ** -0.5)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+    g1 = ops.dense_bwd(q, k, v, o1, do, l1, 0, True, 64, 1, 0, d ** -0.5)
+    g2 = ops.dense_bwd(qc, k, v, o2, do, l2, 0, True, 64, 1, 0, d ** -0.5)
+    for name, a, b_ in zip(("dq", "dk", "dv"), g1, g2):
+        assert_close(a, b_, 1e-2, 1e-2, name)
+
+
 @pytest.mark.parametrize("b,h,n,d", [(2, 4, 100, 64), (1, 8, 333, 128)])
 def test_gate_combine_matches_oracle(b, h, n, d):
     from native_sparse_attention_pytorch_amd.ops import gate_combine
