@@ -1094,7 +1094,8 @@ static int dense_bwd_launch(const DensePlan& P, const void* q, const void* k, co
                      (const __bf16*)v, (const __bf16*)out, (const __bf16*)dout, lse, delta, (__bf16*)dq);      // also writes delta
   NSA_LAUNCH_CHECK();
   const auto group_span = [&](const long* st) { return (long)(P.g - 1) * st[1] + (long)(P.n - 1) * st[2] + D; };
-  if (D >= NSA_DKV_PIPE_MIN_D && group_span(P.sq) < (1l << 30) && group_span(P.sdo) < (1l << 30))
+  // the pipelined kernel's buffer loads take 32-bit byte offsets within one kv head's query heads (rows) and their lse / delta
+  if (D >= NSA_DKV_PIPE_MIN_D && group_span(P.sq) < (1l << 30) && group_span(P.sdo) < (1l << 30) && (long)P.g * P.n < (1l << 29))
     hipLaunchKernelGGL((dense_bwd_dkv_pipe_kernel<D>), dim3(dkv_grid(P), P.bh), dim3(128), 0, st, P, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (const __bf16*)dout, lse, delta, part);
   else
