@@ -225,3 +225,48 @@ def test_fp32_module_runs_and_matches_oracle():
     seq = torch.cat(outs, dim=1)
     bad = ((seq.float().cpu() - want).abs() > 4e-2 * want.abs().max()).any(dim=-1).float().mean().item()
     assert bad < 0.05, f"{bad:.3f} of the tokens differ between prefill+decode and the oracle's parallel forward"
+
+
+def test_module_front_end_paths_agree():
+    """The default bf16 module runs norm, qkv projection and gate logits as one autograd node, its weight gradients as
+    sliced GEMMs and its bias / position gradients as column sums; a module whose layers carry hooks (or a custom gate
+    network, or no norm) calls the layers one by one.  Same function either way: outputs and every gradient agree to
+    bf16 rounding, and the fused path is really the one taken by default."""
+    from native_sparse_attention_pytorch_amd import ops
+    kw = CONFIGS[1]
+    _, mod = _pair(3, **kw)
+    torch.manual_seed(5)
+    x = torch.randn(2, 4096, kw["dim"], device=DEV).to(torch.bfloat16)
+    do = torch.randn_like(x)
+
+    def run(m):
+        for p in m.parameters():
+            p.grad = None
+        xg = x.clone().requires_grad_()
+        out = m(xg)
+        out.backward(do)
+        return out, xg.grad, {n: p.grad for n, p in m.named_parameters() if p.grad is not None}
+
+    calls = {"front": 0}
+    orig = ops.normed_projections
+    def spy(*a, **k):
+        calls["front"] += 1
+        return orig(*a, **k)
+    ops.normed_projections = spy
+    try:
+        out1, dx1, g1 = run(mod)
+        assert calls["front"] == 1
+        hooks = [m.register_forward_hook(lambda *_: None) for m in (mod.norm, mod.to_qkv, mod.to_strategy_combine[0], mod.combine_heads,
+                                                                  mod.k_compress, mod.v_compress)]
+        out2, dx2, g2 = run(mod)
+        assert calls["front"] == 1                      # hooks: layer by layer
+        for h_ in hooks:
+            h_.remove()
+    finally:
+        ops.normed_projections = orig
+    rel = lambda a, b_: ((a.float() - b_.float()).norm() / b_.float().norm().clamp_min(1e-9)).item()
+    assert rel(out1, out2) < 1e-2
+    assert rel(dx1, dx2) < 2e-2
+    assert g1.keys() == g2.keys()
+    for n in g1:
+        assert rel(g1[n], g2[n]) < 3e-2, (n, rel(g1[n], g2[n]))
