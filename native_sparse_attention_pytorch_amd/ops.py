@@ -1180,12 +1180,13 @@ def window_position_grad(dwin: Tensor, out_dtype) -> Tensor:
     """Gradient of the intra-window positions 'h j d' from the gradient of the windows 'b h w j d' (contiguous bf16): its sum
     over batch and windows (NSA.py:599-600 add the positions to every window)."""
     b, h, w, j, d = dwin.shape
-    out = torch.empty((h, j, d), dtype=torch.float32, device=dwin.device)
+    direct = out_dtype in (_BF16, torch.float32)            # the kernel rounds the fp32 sums to bf16 itself
+    out = torch.empty((h, j, d), dtype=out_dtype if direct else torch.float32, device=dwin.device)
     L = _lib.lib()
     ws = torch.empty((max(L.nsa_colsum_workspace(b * w, j * d, h), 4) // 4,), dtype=torch.float32, device=dwin.device)
-    _lib.check(L.nsa_colsum(_ptr(dwin), h, dwin.stride(1), b, dwin.stride(0), w, dwin.stride(2), j * d, _ptr(out), 1, _ptr(ws), _stream()),
-               "nsa_colsum")
-    return out.to(out_dtype)
+    _lib.check(L.nsa_colsum(_ptr(dwin), h, dwin.stride(1), b, dwin.stride(0), w, dwin.stride(2), j * d, _ptr(out),
+                            int(out.dtype == torch.float32), _ptr(ws), _stream()), "nsa_colsum")
+    return out if direct else out.to(out_dtype)
 
 
 def rms_norm_supported(x: Tensor, weight: Tensor | None) -> bool:
