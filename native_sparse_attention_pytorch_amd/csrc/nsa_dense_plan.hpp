@@ -2,6 +2,7 @@
 #pragma once
 #include <stddef.h>
 #include <stdint.h>
+#include <algorithm>
 #include "../../include/nsa_hip.h"
 
 namespace nsa {
@@ -66,8 +67,19 @@ static inline int make_dense_plan(const nsa_dense_desc* d, DensePlan& P) {
   // are cut into chunks of chunk_q; smaller chunks when there would be too few work-groups
   P.key_tiles = (P.krows + 63) / 64;
   const long span = P.mode == 0 ? ((long)64 + P.wb + P.wf < P.n ? (long)64 + P.wb + P.wf : P.n) : P.n;
-  P.chunk_q = 1024;
-  while (P.chunk_q > 128 && bh * P.key_tiles * ((span + P.chunk_q - 1) / P.chunk_q) < 2048) P.chunk_q /= 2;
+#ifndef NSA_DKV_MIN_WGS
+#define NSA_DKV_MIN_WGS 2048
+#endif
+  if (P.mode == 0) {
+    // band: a tile's visible queries (64 + window of them) in equal chunks, as few as give the chip NSA_DKV_MIN_WGS work-groups
+    // (a chunk of 512 beside one of 64 is a work-group that runs eight times longer than its neighbour)
+    long want = (NSA_DKV_MIN_WGS + bh * P.key_tiles - 1) / (bh * P.key_tiles);
+    want = std::max<long>(1, std::min<long>(want, (span + 127) / 128));
+    P.chunk_q = (int)(((span + want - 1) / want + 31) / 32 * 32);
+  } else {
+    P.chunk_q = 1024;
+    while (P.chunk_q > 128 && bh * P.key_tiles * ((span + P.chunk_q - 1) / P.chunk_q) < 2048) P.chunk_q /= 2;
+  }
   P.chunks = (int)((span + P.chunk_q - 1) / P.chunk_q);
   size_t o = 0;
   P.off_delta = o; o = dense_align_up(o + (size_t)bh * P.g * P.n * 4);

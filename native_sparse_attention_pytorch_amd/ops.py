@@ -1303,7 +1303,10 @@ def _wgrad(dy2: Tensor, x2: Tensor, dtype) -> Tensor:
     rows, n_in, n_out = x2.shape[0], x2.shape[1], dy2.shape[1]
     s = _wgrad_splits(rows, n_in, n_out) if x2.is_cuda and x2.dtype in (_BF16, torch.float16) and dy2.dtype == x2.dtype else 1
     if s > 1 and dy2.is_contiguous() and x2.is_contiguous():
-        part = torch.bmm(dy2.view(s, rows // s, n_out).transpose(1, 2), x2.view(s, rows // s, n_in), out_dtype=torch.float32)
+        try:
+            part = torch.bmm(dy2.view(s, rows // s, n_out).transpose(1, 2), x2.view(s, rows // s, n_in), out_dtype=torch.float32)
+        except TypeError:                     # a torch without fp32 output from a bf16 batched GEMM: partial products in bf16
+            part = torch.bmm(dy2.view(s, rows // s, n_out).transpose(1, 2), x2.view(s, rows // s, n_in)).float()
         if dtype not in (_BF16, torch.float32) or (n_out * n_in) % 4:
             return part.sum(0).to(dtype)
         dw = torch.empty((n_out, n_in), dtype=dtype, device=x2.device)
