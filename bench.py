@@ -123,9 +123,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="only the headline workload (for profiler runs): no compressed-branch, module or decode legs")
-    ap.add_argument("--skip", default="", help="comma-separated legs to leave out: rowtraffic, compressed, module, decode, train, generate")
+    ap.add_argument("--skip", default="", help="comma-separated legs to leave out: select_config2, rowtraffic, compressed, module, decode, train, generate")
     args = ap.parse_args()
-    skip = set(filter(None, args.skip.split(","))) | ({"rowtraffic", "compressed", "module", "decode", "train", "generate"} if args.headline_only else set())
+    skip = set(filter(None, args.skip.split(","))) | ({"select_config2", "rowtraffic", "compressed", "module", "decode", "train", "generate"} if args.headline_only else set())
 
     def leg(name):
         """Announce a leg on stderr (a long profiler run must not look hung) or skip it."""
@@ -143,48 +143,53 @@ def main():
     from native_sparse_attention_pytorch_amd import _lib, ops
     L = _lib.lib()
     dev = "cuda"
-    cfg = CFG
-    b, n, hq, hk, d, B, S = cfg["batch"], cfg["seq"], cfg["heads"], cfg["kv_heads"], cfg["dim_head"], cfg["block"], cfg["num_sel"]
-    g = torch.Generator(device=dev).manual_seed(0)
-    mk = lambda h: (torch.randn(b, h, n, d, generator=g, device=dev) * d ** -0.5).to(torch.bfloat16)
-    q, k, v, do = mk(hq), mk(hk), mk(hk), mk(hq)
-    idx, msk = selection(b, hk, n, B, S, 0, dev)
-    fm = msk.view(torch.uint8)
-
-    out = torch.empty_like(q)
-    lse = torch.empty(b, hq, n, dtype=torch.float32, device=dev)
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    dsc = ops._select_desc(q, k, v, out, S, B, True, d ** -0.5, True)
-    ib, fb, wb = ops._ws_sizes(dsc)
-    iws = torch.empty(ib, dtype=torch.uint8, device=dev)
-    # forward and backward workspaces are never live together: share one allocation
-    ws = torch.empty(max(fb, wb), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     hev = HipEvents()
     P = lambda t: t.data_ptr()
 
-    def step(ev):
-        if ev is not None:
-            hev.record(ev[0], stream)
-        _lib.check(L.nsa_select_build_index(C.byref(dsc), P(idx), P(fm), P(iws), ib, stream), "build_index")
-        fe = C.cast(C.byref(ev, 1 * C.sizeof(C.c_void_p)), C.c_void_p) if ev is not None else None
-        be = C.cast(C.byref(ev, 4 * C.sizeof(C.c_void_p)), C.c_void_p) if ev is not None else None
-        _lib.check(L.nsa_select_fwd_timed(C.byref(dsc), P(q), P(k), P(v), P(idx), P(fm), P(iws), P(ws), fb, P(out), P(lse), stream,
-                                          fe, 3 if ev is not None else 0), "fwd")
-        _lib.check(L.nsa_select_bwd_timed(C.byref(dsc), P(q), P(k), P(v), P(out), P(do), P(lse), P(idx), P(fm), P(iws), P(ws), wb,
-                                          P(dq), P(dk), P(dv), None, stream, be, 6 if ev is not None else 0), "bwd")
+    def run_select(cfg, steps, warmup, seed=0):
+        """`steps` timed steps (index build + forward + backward of block-selection attention through the C ABI) on the workload
+        `cfg`; returns (ms per step, per-step event arrays, tensors)."""
+        b, n, hq, hk, d, B, S = cfg["batch"], cfg["seq"], cfg["heads"], cfg["kv_heads"], cfg["dim_head"], cfg["block"], cfg["num_sel"]
+        g = torch.Generator(device=dev).manual_seed(seed)
+        mk = lambda h: (torch.randn(b, h, n, d, generator=g, device=dev) * d ** -0.5).to(torch.bfloat16)
+        q, k, v, do = mk(hq), mk(hk), mk(hk), mk(hq)
+        idx, msk = selection(b, hk, n, B, S, seed, dev)
+        fm = msk.view(torch.uint8)
+        out = torch.empty_like(q)
+        lse = torch.empty(b, hq, n, dtype=torch.float32, device=dev)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dsc = ops._select_desc(q, k, v, out, S, B, True, d ** -0.5, True)
+        ib, fb, wb = ops._ws_sizes(dsc)
+        iws = torch.empty(ib, dtype=torch.uint8, device=dev)
+        # forward and backward workspaces are never live together: share one allocation
+        ws = torch.empty(max(fb, wb), dtype=torch.uint8, device=dev)
 
-    for _ in range(args.warmup):
-        step(None)
-    torch.cuda.synchronize()
-    evs = [hev.make(10) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for e in evs:
-        step(e)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_step = dt / args.steps * 1e3
+        def step(ev):
+            if ev is not None:
+                hev.record(ev[0], stream)
+            _lib.check(L.nsa_select_build_index(C.byref(dsc), P(idx), P(fm), P(iws), ib, stream), "build_index")
+            fe = C.cast(C.byref(ev, 1 * C.sizeof(C.c_void_p)), C.c_void_p) if ev is not None else None
+            be = C.cast(C.byref(ev, 4 * C.sizeof(C.c_void_p)), C.c_void_p) if ev is not None else None
+            _lib.check(L.nsa_select_fwd_timed(C.byref(dsc), P(q), P(k), P(v), P(idx), P(fm), P(iws), P(ws), fb, P(out), P(lse), stream,
+                                              fe, 3 if ev is not None else 0), "fwd")
+            _lib.check(L.nsa_select_bwd_timed(C.byref(dsc), P(q), P(k), P(v), P(out), P(do), P(lse), P(idx), P(fm), P(iws), P(ws), wb,
+                                              P(dq), P(dk), P(dv), None, stream, be, 6 if ev is not None else 0), "bwd")
+
+        for _ in range(warmup):
+            step(None)
+        torch.cuda.synchronize()
+        evs = [hev.make(10) for _ in range(steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for e in evs:
+            step(e)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3, evs, (q, k, v, do, idx, msk, out)
+
+    cfg = CFG
+    b, n, hq, hk, d, B, S = cfg["batch"], cfg["seq"], cfg["heads"], cfg["kv_heads"], cfg["dim_head"], cfg["block"], cfg["num_sel"]
+    ms_step, evs, (q, k, v, do, idx, msk, out) = run_select(cfg, args.steps, args.warmup)
 
     names = ["index_build", "fwd_block_walk", "fwd_merge", None, "bwd_delta", "bwd_dq_walk", "bwd_dkv_walk", "bwd_dq_merge", "bwd_dkv_reduce"]
     kern = {}
@@ -218,6 +223,30 @@ def main():
                            tokens_per_s=round(b * n / (ms_step * 1e-3), 1), attended_pairs=int(pairs), flop_per_step=total_flop),
                kernels_ms={k_: round(v_, 4) for k_, v_ in kern.items()},
                roofline=roofline)
+
+    # BASELINE configs[1]: the isolated selection kernels at b1 n8192 Hq16 Hkv4 d64 B64, 15 selected + own block (the d = 64
+    # family of the same kernels), timed the same way with its own roofline block
+    try:
+        leg("select_config2")
+        cfg2 = dict(batch=1, seq=8192, heads=16, kv_heads=4, dim_head=64, block=64, num_sel=15)
+        ms2, evs2, _t2 = run_select(cfg2, max(args.steps, 20), max(args.warmup, 3), seed=2)
+        kern2 = {nm: sum(hev.ms(e[i], e[i + 1]) for e in evs2) / len(evs2) for i, nm in enumerate(names) if nm is not None}
+        pairs2 = attended_pairs(1, 16, 8192, 64, 16)
+        unit2 = 2.0 * 64 * pairs2
+        dom2 = max(("fwd_block_walk", "bwd_dkv_walk"), key=lambda nm: kern2[nm])
+        ach2 = (2 if dom2 == "fwd_block_walk" else 5) * unit2 / (kern2[dom2] * 1e-3) / 1e12
+        res["select_config2"] = dict(workload="BASELINE configs[1]: selection attention fwd+bwd, b1 n8192 Hq16 Hkv4 d64 B64, 15 selected + own block",
+                                     ms_per_step=round(ms2, 4), tflops=round(7 * unit2 / (ms2 * 1e-3) / 1e12, 2),
+                                     tokens_per_s=round(8192 / (ms2 * 1e-3), 1), attended_pairs=int(pairs2), flop_per_step=7 * unit2,
+                                     kernels_ms={k_: round(v_, 4) for k_, v_ in kern2.items()},
+                                     roofline=dict(bound="mfma", kernel=dom2, achieved=round(ach2, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                                                   frac=round(ach2 / MFMA_PEAK_TFLOPS, 4),
+                                                   step_frac=round(7 * unit2 / (ms2 * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4)))
+        del _t2
+    except _Skip:
+        pass
+    except Exception as ex:
+        res["select_config2"] = dict(error=repr(ex))
 
     # the other half of BASELINE configs[3]: compressed attention with fused importance logits +
     # top-k over 2048 compressed keys (+1 memory slot), forward and backward, reported beside the headline

@@ -296,7 +296,8 @@ int nsa_decode_attend(const nsa_decode_desc* desc, const void* q, const void* k,
  * nsa_decode_workspace_bytes(desc) exceeds NSA_DECODE_NOALLOC_SCRATCH_BYTES.  All calls on one GPU share the
  * array: calls that overlap on one GPU (different streams or threads) race; calls ordered on one stream do not.
  * The first call on a device looks the array's address up (hipGetSymbolAddress) and should be made outside a
- * stream capture. */
+ * stream capture.  The array used is the current device's (hipGetDevice at the time of the call): `stream` must
+ * belong to the current device, as every pointer argument does. */
 #define NSA_DECODE_NOALLOC_SCRATCH_BYTES ((size_t)16 << 20)
 int nsa_decode_attend_noalloc(const nsa_decode_desc* desc, const void* q, const void* k, const void* v, const void* mem_k,
                               const void* mem_v, const void* idx, const uint8_t* fmask, void* out, float* logits, void* stream);

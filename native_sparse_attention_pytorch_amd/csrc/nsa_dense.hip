@@ -798,8 +798,12 @@ __global__ __launch_bounds__(128) void dense_bwd_dkv_pipe_kernel(const DensePlan
 
   // wave 0 stages the tile's Q rows, wave 1 its dO rows, through buffer loads: the descriptor starts at the tile's first
   // query of this kv head's query heads and ends with the last row of the last of them, so a lane's offset is the same in
-  // every step (no address arithmetic in the loop) and rows past the end of the sequence read as zeros instead of needing
-  // a clamp (the launcher checks that the heads of a group span less than 2^31 elements).
+  // every step (no address arithmetic in the loop) and no row index needs a clamp (the launcher checks that the heads of a
+  // group span less than 2^31 elements).  What a row past the end of the sequence reads depends on the head: in the group's
+  // last head it lies beyond the descriptor and reads as zeros; in an earlier head of a contiguous 'h n d' array it lands on
+  // the leading rows of the next head (and its lse / delta likewise).  Either way such a row is neutralised by its
+  // log-sum-exp, which store_smalls replaces by +inf for every row at or beyond c1: p = exp2(finite - inf) = 0 and
+  // dS = 0 * (finite) = 0, so finite values of any size in the aliased rows add nothing to dK / dV.
   const int ktu = __builtin_amdgcn_readfirstlane(kt);
   const __bf16* slab = ktu == 0 ? q + b * P.sq[0] + (long)(hk * P.g) * P.sq[1] : dout + b * P.sdo[0] + (long)(hk * P.g) * P.sdo[1];
   const long sh = ktu == 0 ? P.sq[1] : P.sdo[1], sn = ktu == 0 ? P.sq[2] : P.sdo[2];

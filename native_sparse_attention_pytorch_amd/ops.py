@@ -1358,7 +1358,45 @@ def normed_projections(inp: Tensor, norm_weight: Tensor, eps: float | None, w_qk
     return _NormedProjections.apply(inp, norm_weight, float(torch.finfo(torch.float32).eps if eps is None else eps), w_qkv, w_gate, b_gate)
 
 
-# ------------------------------------------------------------------ fp32 forward (inference)
+# ------------------------------------------------------------------ fp32 forward
+
+class _Fp32ValueBf16Grad(torch.autograd.Function):
+    """An attention branch of an fp32 module under autograd.  The fp32 kernels are forward kernels; there is no fp32 backward.
+    The forward value is theirs (the reference's fp32 bound, 1e-5, holds with gradients enabled too, so the parallel forward
+    and the decode steps of tests/test_sparse_attn.py:50-91 agree whatever the grad mode); the gradient is the gradient of
+    the same branch evaluated by the bf16 kernels on the bf16-rounded inputs (forward + backward, run in `backward`), which
+    meets the gradient bound of a bf16 run (5e-2).  `fwd32(*tensors)` and `fwd16(*tensors)` evaluate the branch; every tensor
+    argument is a candidate for a gradient."""
+
+    @staticmethod
+    def forward(ctx, fwd32, fwd16, *tensors):
+        ctx.fwd16 = fwd16
+        ctx.save_for_backward(*tensors)
+        return fwd32(*tensors)
+
+    @staticmethod
+    def backward(ctx, dout):
+        tensors = ctx.saved_tensors
+        need = ctx.needs_input_grad[2:]
+        with torch.enable_grad():
+            ins = [t.detach().to(_BF16).requires_grad_(bool(nd)) for t, nd in zip(tensors, need)]
+            out = ctx.fwd16(*ins)
+            wanted = [t for t in ins if t.requires_grad]
+            grads = iter(torch.autograd.grad(out, wanted, dout.to(out.dtype), allow_unused=True)) if wanted else iter(())
+        res = []
+        for t, nd in zip(tensors, need):
+            g = next(grads) if nd else None
+            res.append(None if g is None else g.to(t.dtype))
+        return (None, None, *res)
+
+
+def fp32_value_bf16_grad(fwd32, fwd16, *tensors: Tensor) -> Tensor:
+    """`fwd32(*tensors)` (fp32 kernels), differentiable through `fwd16` (bf16 kernels) when gradients are being recorded."""
+    if torch.is_grad_enabled() and any(t.requires_grad for t in tensors):
+        return _Fp32ValueBf16Grad.apply(fwd32, fwd16, *tensors)
+    with torch.no_grad():
+        return fwd32(*tensors)
+
 
 def _f32(t: Tensor) -> Tensor:
     if t.dtype != torch.float32 or not t.is_cuda:
@@ -1417,13 +1455,12 @@ def native_sparse_attend_f32(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int
     return (out, lse) if return_lse else out
 
 
-@torch.no_grad()
 def importance_logits_f32(q: Tensor, ck: Tensor, stride: int, sel_block: int, share: bool, causal: bool, mask_own: bool = True):
     """Block-importance logits of NSA.py:652-691 in fp32.  They are the mean, over a fine block's compressed keys and (if
     shared) the group's heads, of scale * q . ck - linear in both, so one fp32 GEMM against the block means of the
     compressed keys `ck` 'b hk nc d' (memory slots excluded); -inf where the reference's fill values remove the block from
     the softmax (a block not entirely before the query; the query's own block when stride != sel_block).  None when no
-    full fine block exists."""
+    full fine block exists.  Plain torch, differentiable in q and ck."""
     b, hq, n, d = q.shape
     hk = ck.shape[1]
     g = hq // hk

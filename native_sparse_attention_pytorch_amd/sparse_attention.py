@@ -147,9 +147,10 @@ class SparseAttention(nn.Module):
             print('`num_selected_blocks` should be set greater than 0, unless if you are ablating it for experimental purposes')
         self.num_selected_blocks = num_selected_blocks
         self.use_triton_kernel = use_triton_kernel      # kept for call-site compatibility; the HIP kernels always run
-        # an fp32 module that is run without gradients takes the fp32 forward kernels (agreement with the reference's fp32
-        # path to 1e-5); with gradients, or with this switched off, its attention runs in bf16 like any other module's
-        self.fp32_inference_kernels = True
+        # an fp32 module takes the fp32 forward kernels (agreement with the reference's fp32 path to 1e-5), in the parallel
+        # forward - with or without gradients, whose values then come from the bf16 kernels - and in the decode step; with
+        # this switched off its attention runs in bf16 like any other module's
+        self.fp32_kernels = True
 
         if strategy_combine_mlp is None:
             strategy_combine_mlp = nn.Linear(dim, 3 * heads)
@@ -157,6 +158,9 @@ class SparseAttention(nn.Module):
             strategy_combine_mlp.bias.data.copy_(torch.tensor([-2., -2., 2.] * heads))
         self.to_strategy_combine = nn.Sequential(strategy_combine_mlp, nn.Sigmoid(), _GateLayout(heads))
         self.combine_heads = nn.Linear(dim_inner, dim, bias=False)
+
+    # the switch's earlier name
+    fp32_inference_kernels = property(lambda self: self.fp32_kernels, lambda self, on: setattr(self, "fp32_kernels", bool(on)))
 
     # ------------------------------------------------------------------------------ pieces
 
@@ -167,7 +171,13 @@ class SparseAttention(nn.Module):
 
     @staticmethod
     def _plain(layer, kind):
-        return type(layer) is kind and not (layer._forward_hooks or layer._forward_pre_hooks or layer._backward_hooks)
+        """A library layer of exactly this kind on which nothing is hooked, neither on the instance nor globally: only then may
+        its weights be used directly (any hook is skipped when the layer's own `__call__` is)."""
+        from torch.nn.modules import module as M
+        own = (layer._forward_hooks, layer._forward_pre_hooks, layer._backward_hooks, layer._backward_pre_hooks)
+        glob = tuple(getattr(M, name, None) for name in ("_global_forward_hooks", "_global_forward_pre_hooks", "_global_backward_hooks",
+                                                         "_global_backward_pre_hooks", "_global_forward_hooks_always_called"))
+        return type(layer) is kind and not any(own) and not any(glob)
 
     def _front_is_one_node(self, inp):
         """Norm, qkv projection and gate logits as ops.normed_projections: a bf16 module with its default layers, under autograd."""
@@ -217,7 +227,7 @@ class SparseAttention(nn.Module):
         x = self.norm(inp)
         q, k, v = self.to_qkv(x).split(self.qkv_split, dim=-1)
         q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
-        if (self.fp32_inference_kernels and q.dtype == torch.float32 and self.dim_head <= 128 and self.dim_head % 4 == 0
+        if (self.fp32_kernels and q.dtype == torch.float32 and self.dim_head <= 128 and self.dim_head % 4 == 0
                 and all(t.dtype == torch.float32 for t in (cache_k, cache_v, cache_ck, cache_cv, run_k, run_v))):
             return self._forward_inference_fp32(x, q, k, v, cache, return_cache)
         # head dimensions other than the kernels' 64 / 128 run zero-padded: caches and window rows are then kept D wide
@@ -329,44 +339,61 @@ class SparseAttention(nn.Module):
             return out
         return out, ((keys, vals), ((ck, cv), (run_k, run_v)))
 
-    @torch.no_grad()
     def _forward_fp32(self, x, qkv, return_cache):
-        """The parallel forward of an fp32 module without gradients: every attention branch through the fp32 kernels
-        (ops.*_f32), the gate and the merge in fp32 torch - the same steps as `forward` (NSA.py:579-862)."""
+        """The parallel forward of an fp32 module: every attention branch through the fp32 kernels (ops.*_f32), the gate and
+        the merge in fp32 torch - the same steps as `forward` (NSA.py:579-862).  Under autograd the values are still those of
+        the fp32 kernels and each branch's gradient comes from the bf16 kernels (ops.fp32_value_bf16_grad); rotation and
+        window split are then plain differentiable torch."""
         b, n, _ = x.shape
         st, cbs, B = self.compress_block_sliding_stride, self.compress_block_size, self.selection_block_size
         M, d = self.num_mem_compress_kv, self.dim_head
+        causal, win, share = self.causal, self.sliding_window_size, self.query_heads_share_selected_kv
         q, k, v = qkv.split(self.qkv_split, dim=-1)
         q, k, v = self._split_heads(q), self._split_heads(k), self._split_heads(v)
         L = (n // st) * st
-        if d in (64, 128):
+        recording = torch.is_grad_enabled() and (qkv.requires_grad or any(p.requires_grad for p in self.parameters()))
+        if d in (64, 128) and not recording:
             _, rq, rk, _, kw, vw = ops.qkv_prep_f32(qkv, self.rotary_emb.freqs, self.k_intrablock_positions, self.v_intrablock_positions,
                                                     self.heads, self.kv_heads, d, cbs, st)
         else:
             rq, rk = self.rotary_emb.rotate(q), self.rotary_emb.rotate(k)
-            win = lambda t, pos: F.pad(t[..., :L, :], (0, 0, cbs - st, 0)).unfold(2, cbs, st).permute(0, 1, 2, 4, 3) + pos[None, :, None]
-            kw, vw = win(k, self.k_intrablock_positions), win(v, self.v_intrablock_positions)
+            def win_of(t, pos):
+                if L == 0:                                                    # fewer tokens than one stride: no window yet
+                    return t.new_zeros((b, t.shape[1], 0, cbs, d)) + pos[None, :, None]
+                return F.pad(t[..., :L, :], (0, 0, cbs - st, 0)).unfold(2, cbs, st).permute(0, 1, 2, 4, 3) + pos[None, :, None]
+            kw, vw = win_of(k, self.k_intrablock_positions), win_of(v, self.v_intrablock_positions)
         ck0, cv0 = self.k_compress(kw), self.v_compress(vw)
         ck = torch.cat((self.compress_mem_kv[0][None].expand(b, -1, -1, -1), ck0), dim=-2)
         cv = torch.cat((self.compress_mem_kv[1][None].expand(b, -1, -1, -1), cv0), dim=-2)
         nc = ck0.shape[-2]
-        c_out, _ = ops.dense_attend_f32(q, ck, cv, 1, self.causal, 0, st, M)
+        c_out = ops.fp32_value_bf16_grad(lambda q_, k_, v_: ops.dense_attend_f32(q_, k_, v_, 1, causal, 0, st, M)[0],
+                                         lambda q_, k_, v_: ops.compress_attend(q_, k_, v_, M, st, causal)[0], q, ck, cv)
         imp = None
         if self.num_selected_blocks > 0 and nc > 0:
-            imp = ops.importance_logits_f32(q, ck0, st, B, self.query_heads_share_selected_kv, self.causal)
+            imp = ops.importance_logits_f32(q, ck0, st, B, share, causal)
+            if not self.use_diff_topk:
+                imp = imp.detach()
         num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
+        gates = None
         if num_sel > 0:
-            _, idx, fmask = ops.importance_topk(imp.contiguous(), num_sel)
-            f_out = ops.native_sparse_attend_f32(rq, rk, v, B, idx, fmask, include_block_causal=self.causal)
-        elif self.causal:
+            vals, idx, fmask = ops.importance_topk(imp.contiguous(), num_sel)
+            if self.use_diff_topk:
+                gates = vals + (1. - vals).detach()                              # straight-through gates (NSA.py:715)
+            block_causal = causal
+        elif causal:
             idx = torch.zeros((b, self.kv_heads, n, 0), dtype=torch.int32, device=x.device)
-            f_out = ops.native_sparse_attend_f32(rq, rk, v, B, idx, idx.bool(), include_block_causal=True)
+            fmask, block_causal = idx.bool(), True
         else:
-            own = (torch.arange(n, device=x.device, dtype=torch.int32) // B)[None, None, :, None].expand(b, self.kv_heads, n, 1).contiguous()
-            f_out = ops.native_sparse_attend_f32(rq, rk, v, B, own, torch.ones_like(own, dtype=torch.bool), include_block_causal=False)
-        s_out, _ = ops.dense_attend_f32(rq, rk, v, 0, self.causal, self.sliding_window_size)
-        gates = self.to_strategy_combine(x)                                   # 'b h n 3' after the sigmoid
-        merged = gates[..., 0:1] * c_out + gates[..., 1:2] * f_out + gates[..., 2:3] * s_out
+            idx = (torch.arange(n, device=x.device, dtype=torch.int32) // B)[None, None, :, None].expand(b, self.kv_heads, n, 1).contiguous()
+            fmask, block_causal = torch.ones_like(idx, dtype=torch.bool), False
+        sel32 = lambda q_, k_, v_, *g_: ops.native_sparse_attend_f32(q_, k_, v_, B, idx, fmask, include_block_causal=block_causal)
+        sel16 = lambda q_, k_, v_, *g_: ops.native_sparse_attend(q_, k_, v_, B, idx, fmask, sel_scale=g_[0] if g_ else None,
+                                                                 include_block_causal=block_causal)
+        f_out = ops.fp32_value_bf16_grad(sel32, sel16, rq, rk, v, *(() if gates is None else (gates,)))
+        s_out = ops.fp32_value_bf16_grad(lambda q_, k_, v_: ops.dense_attend_f32(q_, k_, v_, 0, causal, win)[0],
+                                         lambda q_, k_, v_: ops.sliding_attend(q_, k_, v_, win, causal=causal), rq, rk, v)
+        gates3 = self.to_strategy_combine(x)                                  # 'b h n 3' after the sigmoid
+        merged = gates3[..., 0:1] * c_out + gates3[..., 1:2] * f_out + gates3[..., 2:3] * s_out
         out = self.combine_heads(merged.permute(0, 2, 1, 3).reshape(b, n, self.heads * d))
         if not return_cache:
             return out
@@ -401,7 +428,7 @@ class SparseAttention(nn.Module):
         else:
             x = self._normed(inp)
             qkv = self._linear(self.to_qkv, x)
-        if (x is not None and self.fp32_inference_kernels and qkv.dtype == torch.float32 and not (torch.is_grad_enabled() and qkv.requires_grad)
+        if (x is not None and self.fp32_kernels and qkv.dtype == torch.float32
                 and self.dim_head <= 128 and self.dim_head % 4 == 0 and not torch.compiler.is_compiling()):
             return self._forward_fp32(x, qkv, return_cache)
         q, k, v = qkv.split(self.qkv_split, dim=-1)

@@ -52,6 +52,37 @@ def test_sliding_matches_oracle(b, hq, hk, n, d, win, causal):
     _grad_close(vg.grad, vr.grad, "dv")
 
 
+@pytest.mark.parametrize("mode", ["sliding", "compressed"])
+def test_dkv_ignores_rows_past_the_sequence_end(mode):
+    """d = 128 dK/dV walk, n not a multiple of the 8-query tile of a group of 4, contiguous q / dO: the padding rows of a
+    ragged last tile of head g alias the leading rows of head g + 1.  They must add nothing to dK / dV whatever (finite)
+    values sit there: large values in the first rows of every head but the first leave the gradients at the oracle's."""
+    from native_sparse_attention_pytorch_amd.ops import sliding_attend, compress_attend
+    b, hq, hk, n, d = 1, 8, 2, 203, 128
+    g = torch.Generator().manual_seed(7)
+    q, do = _rand((b, hq, n, d), g, d ** -0.25), _rand((b, hq, n, d), g)
+    with torch.no_grad():
+        q[:, 1:, :8] *= 64.0            # (finite, far larger than anything else; scores of those rows saturate the softmax)
+        do[:, 1:, :8] *= 512.0
+    if mode == "sliding":
+        k, v = _rand((b, hk, n, d), g, d ** -0.25), _rand((b, hk, n, d), g)
+    else:
+        k, v = _rand((b, hk, 1 + n // 4, d), g, d ** -0.25), _rand((b, hk, 1 + n // 4, d), g)
+    qr, kr, vr = (t.float().requires_grad_() for t in (q, k, v))
+    if mode == "sliding":
+        ref = O.sliding_attend(qr, kr, vr, 40, causal=True)
+    else:
+        ref = O.attend(qr, kr, vr, mask=O.compress_mask(n, n // 4, 4, 1, True))
+    (ref * do.float()).sum().backward()
+    qg, kg, vg = (t.to(DEV).contiguous().requires_grad_() for t in (q, k, v))
+    out = sliding_attend(qg, kg, vg, 40, causal=True) if mode == "sliding" else compress_attend(qg, kg, vg, 1, 4, True)[0]
+    (out.float() * do.to(DEV).float()).sum().backward()
+    torch.cuda.synchronize()
+    assert torch.isfinite(kg.grad.float()).all() and torch.isfinite(vg.grad.float()).all()
+    _grad_close(kg.grad, kr.grad, "dk")
+    _grad_close(vg.grad, vr.grad, "dv")
+
+
 COMPRESS = [
     # b, hq, hk, n, d, st, B, mem, causal, share
     (2, 4, 2, 200, 64, 4, 16, 1, True, True),

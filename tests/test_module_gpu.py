@@ -184,9 +184,9 @@ def test_module_edge_shapes_run():
 
 
 def test_fp32_module_runs_and_matches_oracle():
-    """A module left in fp32 (the reference's default dtype): parameters and activations stay fp32 for the
-    projections, the kernels compute in bf16; forward, backward and cached decoding must work and agree
-    with the oracle within the bf16 tolerances."""
+    """A module left in fp32 (the reference's default dtype) under autograd: the forward values come from the fp32
+    kernels (the reference's fp32 bound), the gradients from the bf16 kernels (the bf16 gradient bound, 5e-2 norm-wise
+    against the fp32 oracle's autograd); prefill + cached decoding agrees with the parallel forward."""
     from native_sparse_attention_pytorch_amd.sparse_attention import SparseAttention
     kw = dict(dim=128, dim_head=64, heads=4, kv_heads=2, sliding_window_size=16, compress_block_size=8,
               compress_block_sliding_stride=4, selection_block_size=16, num_selected_blocks=2, causal=True)
@@ -213,8 +213,16 @@ def test_fp32_module_runs_and_matches_oracle():
     finally:
         ops.importance_topk = orig
     assert out.dtype == torch.float32 and xg.grad is not None and torch.isfinite(xg.grad).all()
-    want = ref(x, selection_override=captured["sel"])
-    assert_close(out, want, 3e-2 * want.abs().max().item(), 2e-2, "fp32 module out")
+    xr = x.clone().requires_grad_()
+    want = ref(xr, selection_override=captured["sel"])
+    assert_close(out, want, 2e-5, 1e-5, "fp32 module out")
+    want.sum().backward()
+    rel = lambda a, b_: ((a.float().cpu() - b_.float()).norm() / b_.float().norm().clamp_min(1e-6)).item()
+    assert rel(xg.grad, xr.grad) < 5e-2, f"input grad rel err {rel(xg.grad, xr.grad):.4f}"
+    for (name, p), (_, pr) in zip(mod.named_parameters(), ref.named_parameters()):
+        if pr.grad is None:
+            continue
+        assert p.grad is not None and rel(p.grad, pr.grad) < 5e-2, f"grad of {name}: rel err {rel(p.grad, pr.grad):.4f}"
     # prefill + decode with fp32 caches handed back by the parallel forward
     with torch.no_grad():
         y, cache = mod(x[:, :60].to(DEV), return_cache=True)
@@ -223,8 +231,7 @@ def test_fp32_module_runs_and_matches_oracle():
             o, cache = mod(x[:, i:i + 1].to(DEV), cache=cache, return_cache=True)
             outs.append(o)
     seq = torch.cat(outs, dim=1)
-    bad = ((seq.float().cpu() - want).abs() > 4e-2 * want.abs().max()).any(dim=-1).float().mean().item()
-    assert bad < 0.05, f"{bad:.3f} of the tokens differ between prefill+decode and the oracle's parallel forward"
+    assert_close(seq, want.detach(), 2e-5, 1e-5, "fp32 prefill + decode")
 
 
 def test_module_front_end_paths_agree():

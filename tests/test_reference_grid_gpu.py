@@ -1,7 +1,8 @@
 """The reference's own inference tests (tests/test_sparse_attn.py:46-118) run against the HIP module: token-by-token
 decoding from an empty cache equals the parallel forward, for compress block 5 and selection blocks 8 / 16 / 20, and
-greedy sampling with and without the caches gives the same tokens for selection blocks 4 and 8.  The modules are fp32 and
-run without gradients, so they take the fp32 kernels and the reference's own bound, 1e-5, applies unchanged."""
+greedy sampling with and without the caches gives the same tokens for selection blocks 4 and 8.  The modules are fp32, so
+they take the fp32 kernels - with gradient mode on, as the reference's tests leave it, as well as without - and the
+reference's own bound, 1e-5, applies unchanged."""
 import pytest
 import torch
 
@@ -20,15 +21,17 @@ def test_inference(seq_len, num_selected_blocks, compress_block_sliding_stride, 
                            selection_block_size=selection_block_size, num_selected_blocks=num_selected_blocks,
                            compress_block_sliding_stride=compress_block_sliding_stride).to(DEV)
     tokens = torch.randn(2, seq_len, 512, device=DEV)
-    with torch.no_grad():
-        parallel_out = attn(tokens)
-        cache, sequential_out = None, []
-        for i in range(seq_len):
-            one_out, cache = attn(tokens[:, i:(i + 1)], cache=cache, return_cache=True)
-            sequential_out.append(one_out)
+    # as the reference runs it: gradient mode on, parameters requiring gradients (the parallel forward then records a graph
+    # whose values still come from the fp32 kernels; the decode step never records one)
+    parallel_out = attn(tokens)
+    cache, sequential_out = None, []
+    for i in range(seq_len):
+        one_out, cache = attn(tokens[:, i:(i + 1)], cache=cache, return_cache=True)
+        sequential_out.append(one_out)
     sequential_out = torch.cat(sequential_out, dim=1)
     assert parallel_out.shape == tokens.shape
     assert parallel_out.dtype == torch.float32
+    assert parallel_out.requires_grad and not sequential_out.requires_grad
     assert torch.allclose(parallel_out, sequential_out, atol=1e-5), (parallel_out - sequential_out).abs().max().item()
 
 

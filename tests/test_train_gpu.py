@@ -51,8 +51,10 @@ def test_train_small_matches_live_oracle():
     print("oracle", want)
     print("hip   ", got)
     assert want[-1] < want[0] - 0.05, "the oracle run must actually learn, or the comparison pins nothing"
+    # measured agreement is a few 1e-5 per step (bf16 autocast against the fp32 oracle); the loss falls by ~0.07 per step, so a
+    # bound of 2e-3 tells a wrong layer from rounding
     for a, b in zip(got, want):
-        assert abs(a - b) < 3e-2, (got, want)
+        assert abs(a - b) < 2e-3, (got, want)
 
 
 def test_train_config5_matches_oracle_fixture():
@@ -63,4 +65,4 @@ def test_train_config5_matches_oracle_fixture():
     print("oracle fixture", fx["losses"])
     print("hip           ", got)
     for a, b in zip(got, fx["losses"]):
-        assert abs(a - b) < 3e-2, (got, fx["losses"])
+        assert abs(a - b) < 2e-3, (got, fx["losses"])

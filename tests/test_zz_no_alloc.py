@@ -80,6 +80,32 @@ def test_noalloc_decode_attend_matches_workspace_entry_point():
         assert torch.isfinite(o2.float()).all() and torch.equal(o1, o2), (S, kv_len)
 
 
+def test_noalloc_entry_point_leaves_device_memory_alone():
+    """After a first call (which looks the array's address up), further calls neither take nor return device memory: the
+    driver's free-memory figure and the caching allocator's counters are the same before and after."""
+    from native_sparse_attention_pytorch_amd import _lib
+    L = _lib.lib()
+    g = torch.Generator().manual_seed(1)
+    b, hq, hk, d, cap = 2, 8, 2, 128, 2100
+    k = (torch.randn(b, hk, cap, d, generator=g) * d ** -0.25).to(torch.bfloat16).to(DEV)
+    v = (torch.randn(b, hk, cap, d, generator=g) * d ** -0.25).to(torch.bfloat16).to(DEV)
+    q = (torch.randn(b, hq, d, generator=g) * d ** -0.25).to(torch.bfloat16).to(DEV)
+    out = torch.empty_like(q)
+    dsc = _desc(q, k, v, 0, start=0, count=2000, num_mem=0)
+    st = torch.cuda.current_stream().cuda_stream
+    call = lambda: L.nsa_decode_attend_noalloc(C.byref(dsc), q.data_ptr(), k.data_ptr(), v.data_ptr(), 0, 0, 0, 0, out.data_ptr(), 0, st)
+    assert call() == 0
+    torch.cuda.synchronize()
+    first = out.clone()
+    before = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    for _ in range(3):
+        assert call() == 0
+    torch.cuda.synchronize()
+    after = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    assert before == after, (before, after)
+    assert torch.equal(out, first)
+
+
 def test_noalloc_rejects_sizes_beyond_its_array():
     from native_sparse_attention_pytorch_amd import _lib
     L = _lib.lib()
