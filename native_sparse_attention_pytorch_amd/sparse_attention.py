@@ -371,7 +371,7 @@ class SparseAttention(nn.Module):
         imp = None
         if self.num_selected_blocks > 0 and nc > 0:
             imp = ops.importance_logits_f32(q, ck0, st, B, share, causal)
-            if not self.use_diff_topk:
+            if imp is not None and not self.use_diff_topk:
                 imp = imp.detach()
         num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
         gates = None
