@@ -135,6 +135,24 @@ int nsa_dense_bwd(const nsa_dense_desc* d, const void* q, const void* k, const v
                   const void* out, const void* d_out, const float* lse, void* bwd_ws, size_t bwd_bytes,
                   void* dq, void* dk, void* dv, void* stream);
 
+/* Compressed attention with the block selection made inside the forward kernel.  Replaces, in one launch,
+ * attend(q, ck, cv, cmask, return_sim=True) (NSA.py:153-184, 632-639), the importance scores (NSA.py:652-691), the
+ * padded softmax (NSA.py:693-695), topk (NSA.py:703-713) and the slot mask (NSA.py:721): the block-importance
+ * logits are never written to memory.  `d` as for nsa_dense_fwd in mode 1 with pool != 0 (sel_block, share); out /
+ * lse as there.  While the key tiles stream by, every query keeps its num_selected best blocks so far; at the end
+ * the kernel writes idx int32 and fmask uint8, both [batch, kv_heads, seq, num_selected]: block indices in
+ * descending order of their logit (equal logits: lower block first - nsa_topk orders by the softmaxed values, which
+ * agrees except where two distinct logits round to the same probability) and fmask = (probability > 1e-10), the
+ * probability taken against the selected entries and the -1e3 pad column (every logit left out is at most the
+ * smallest selected one, so this moves a probability at the threshold by less than its rounding).  Slots with
+ * fmask = 0 hold unspecified valid block indices (as torch.topk's order among the exact zeros is unspecified).
+ * Supported (nsa_compress_topk_supported != 0, else NSA_E_UNSUPPORTED): selections shared by the heads of a group
+ * (share != 0) of at least 2 heads, num_selected <= min(16, number of selection blocks); other cases go through
+ * nsa_dense_fwd + nsa_topk. */
+int nsa_compress_topk_supported(const nsa_dense_desc* d, int32_t num_selected);
+int nsa_compress_topk_fwd(const nsa_dense_desc* d, const void* q, const void* k, const void* v, void* out, float* lse,
+                          int32_t num_selected, int32_t* idx, uint8_t* fmask, void* stream);
+
 /* Block-importance softmax + per-query top-k.  Replaces NSA.py:693-695 (pad -1e3, softmax, drop
  * pad), :713 (topk) and :721 (fmask = value > 1e-10).  scores: fp32 [rows, nb]; with
  * apply_softmax != 0 they are importance logits (-inf = not selectable), otherwise ready

@@ -88,6 +88,9 @@ def lib():
         L.nsa_dense_workspace_bytes.argtypes = [C.POINTER(DenseDesc), C.POINTER(sz)]
         L.nsa_dense_fwd.argtypes = [C.POINTER(DenseDesc)] + [vp] * 7
         L.nsa_dense_bwd.argtypes = [C.POINTER(DenseDesc)] + [vp] * 7 + [sz] + [vp] * 4
+        L.nsa_compress_topk_supported.argtypes = [C.POINTER(DenseDesc), C.c_int32]
+        L.nsa_compress_topk_fwd.argtypes = [C.POINTER(DenseDesc)] + [vp] * 5 + [C.c_int32, vp, vp, vp]
+        L.nsa_compress_topk_supported.restype = L.nsa_compress_topk_fwd.restype = C.c_int
         L.nsa_topk.argtypes = [vp, C.c_int64, C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp]
         L.nsa_topk_prefix.argtypes = [vp, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, vp, vp, vp, vp]
         fp = C.POINTER(C.c_float)

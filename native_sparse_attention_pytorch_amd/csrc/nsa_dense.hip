@@ -39,6 +39,28 @@ __device__ __forceinline__ Interval visible_range(const DensePlan& P, int i) {
 
 constexpr int kBK = 64;          // keys per K/V tile
 
+// maximum / sum over the 16 lanes of a DPP row, left in every lane of the row
+__device__ __forceinline__ float row16_bcast_max(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xF, 0xF, false));
+  };
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0xB1>{}));     // quad_perm [1,0,3,2]
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x4E>{}));     // quad_perm [2,3,0,1]
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x141>{}));    // row_half_mirror
+  v = fmaxf(v, dpp(v, std::integral_constant<int, 0x140>{}));    // row_mirror
+  return v;
+}
+__device__ __forceinline__ float row16_bcast_sum(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xF, 0xF, false));
+  };
+  v += dpp(v, std::integral_constant<int, 0xB1>{});
+  v += dpp(v, std::integral_constant<int, 0x4E>{});
+  v += dpp(v, std::integral_constant<int, 0x141>{});
+  v += dpp(v, std::integral_constant<int, 0x140>{});
+  return v;
+}
+
 // Work-group ids go round-robin over the 8 XCDs, each with its own L2.  Work items that re-read each other's rows
 // (neighbouring query tiles of a sliding window, neighbouring key tiles of its backward, the key tiles of one query
 // chunk) must therefore not be neighbours in work-group id: item v = (x % 8) * ceil(count / 8) + x / 8 gives every
@@ -79,18 +101,39 @@ __device__ __forceinline__ TileWalk make_walk(const DensePlan& P, int i_first, i
 #define NSA_FWD_AHV 2
 #endif
 // ------------------------------------------------------------------------------- forward
-// NPF = selection block / compress stride when the importance logits are wanted, 0 otherwise
-template <int D, int NPF>
+// One candidate inserted into the running selections of the four queries a wave serves at a time (16 lanes per query, lane s
+// of a group holds the s-th best block so far: logit L, block I; descending, equal logits in the order they came, i.e. lower
+// block first).  c is the candidate's logit for the lane's query, ci its block.  Entries at least as large stay, the first
+// smaller one takes the candidate, the rest move one lane up (DPP row shift inside the 16 lanes); a candidate no larger
+// than the last entry changes nothing.
+__device__ __forceinline__ void topk_insert(float& L, int& I, float c, int ci) {
+  const float Lp = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0x7f800000, __builtin_bit_cast(int, L), 0x111, 0xF, 0xF, false));   // row_shr:1, lane 0: +inf
+  const int Ip = __builtin_amdgcn_update_dpp(0, I, 0x111, 0xF, 0xF, false);
+  const bool keep = L >= c, keepp = Lp >= c;
+  L = keep ? L : (keepp ? c : Lp);
+  I = keep ? I : (keepp ? ci : Ip);
+}
+
+// NPF = selection block / compress stride when the importance logits are wanted, 0 otherwise.
+// TK: the block selection itself is made here (NSA.py:693-721 on the logits of NSA.py:652-691): instead of writing the
+// logits out, every query keeps the P.topk <= 16 best blocks seen so far while the key tiles stream by, and the kernel ends
+// by writing their indices (descending logit, ties to the lower block) and the slot mask `probability > 1e-10`.
+template <int D, int NPF, bool TK = false>
 __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                         const __bf16* __restrict__ v, __bf16* __restrict__ out, float* __restrict__ lse,
-                                                        float* __restrict__ pooled) {
+                                                        float* __restrict__ pooled, int* __restrict__ tk_idx, uint8_t* __restrict__ tk_mask) {
   constexpr int KS = D / 16, DT = D / 32, TILE = kBK * D;
+  constexpr int TKP = TK ? 4 : 1;              // up to 16 queries per wave, four at a time
+  float tkL[TKP];
+  int tkI[TKP];
+#pragma unroll
+  for (int p2 = 0; p2 < TKP; ++p2) { tkL[p2] = -INFINITY; tkI[p2] = threadIdx.x & 15; }
   // two swizzled tiles each for K and V, filled by asynchronous copies: tile t+1 lands while tile t is being used
   __shared__ __align__(1024) __bf16 k_s[2 * TILE];
   __shared__ __align__(1024) __bf16 v_s[2 * TILE];
   constexpr bool POOL = NPF > 0;
   constexpr int NBT = POOL ? kBK / (POOL ? NPF : 1) : 1;        // fine blocks per key tile
-  __shared__ float pool_s[POOL ? 4 * 32 * NBT : 1];   // per wave: [rows or queries of the tile][fine blocks of the key tile]
+  __shared__ __align__(16) float pool_s[POOL ? 4 * 32 * NBT : 1];   // per wave: [rows or queries of the tile][fine blocks of the key tile]
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n_ = lane & 31, h = lane >> 5;
   const int bh = blockIdx.y, b = bh / P.hkv, hk = bh % P.hkv;
   const int ppt = 32 >> P.lg;                       // queries per wave tile
@@ -258,6 +301,25 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
                 for (int vi = 0; vi < NV; ++vi) val[vi] += __shfl_xor(val[vi], mk, 64);
               }
             }
+            if (TK) {
+              // the staged values are the final logits: scaled, -inf where the block cannot be selected, NaN ordered first
+              const float norm_t = P.scale / (float)(npf * (SH ? P.g : 1));
+              const int jbt = kb0 / npf, qi_t = i0 + prow_local;
+              const bool all_vis = P.causal && plain && i0 + ppt <= P.n && jbt + nbt <= P.nb;      // wave-uniform, as `direct` below
+#pragma unroll
+              for (int vi = 0; vi < NV; ++vi) {
+                float x = val[vi] * norm_t;
+                x = (x == x) ? x : INFINITY;
+                if (!all_vis) {
+                  const int jblk = jbt + (32 * kt + koff[vi]) / npf;
+                  const int blo = jblk * P.B, bhi = blo + P.B;
+                  const bool own = (blo <= qi_t) & (qi_t < bhi);
+                  const bool vis = (!P.causal | (bhi <= qi_t)) & !(P.mask_own & own) & (jblk < P.nb) & (qi_t < P.n);
+                  x = vis ? x : -INFINITY;
+                }
+                val[vi] = x;
+              }
+            }
             if (mine) {
 #pragma unroll
               for (int vi = 0; vi < NV; ++vi) pw[prow_local * nbt + (32 * kt + koff[vi]) / npf] = val[vi];
@@ -267,6 +329,53 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
           const int rows_here = SH ? ppt : 32;
           const float norm = P.scale / (float)(npf * (SH ? P.g : 1));
           const int jb0 = kb0 / npf;
+          if (TK) {
+            // Four queries at a time, 16 lanes each.  A lane reads all candidates of its query (broadcast reads) into
+            // registers; one of them is its own to test against the query's current last entry (read from the group's lane
+            // 15: a lower bound of the threshold once inserts have happened, which only lets a no-op insert through), the
+            // ballot says which candidate positions have a taker in any of the four queries, and only those run the insert.
+            constexpr int CAND = nbt < 16 ? nbt : 16, RDS = nbt / CAND;
+            const int sub = lane & 15, rgrp = lane >> 4;
+#pragma unroll
+            for (int p2 = 0; p2 < TKP; ++p2) {
+              if (4 * p2 < rows_here) {
+                const int rr = 4 * p2 + rgrp;
+                const bool rlive = rr < rows_here;
+                const float* prow = pw + min(rr, rows_here - 1) * nbt;
+#pragma unroll
+                for (int rd = 0; rd < RDS; ++rd) {
+                  float c[CAND];
+                  if (CAND >= 4) {
+#pragma unroll
+                    for (int j4 = 0; j4 < CAND / 4; ++j4) {
+                      const floatx4 t4 = *reinterpret_cast<const floatx4*>(prow + rd * CAND + 4 * j4);
+#pragma unroll
+                      for (int e = 0; e < 4; ++e) c[4 * j4 + e] = t4[e];
+                    }
+                  } else {
+#pragma unroll
+                    for (int j = 0; j < CAND; ++j) c[j] = prow[rd * CAND + j];
+                  }
+                  const float own_c = prow[rd * CAND + (sub < CAND ? sub : 0)];
+                  const float l15 = tkL[p2];
+                  const float t0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, l15), 15));
+                  const float t1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, l15), 31));
+                  const float t2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, l15), 47));
+                  const float t3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, l15), 63));
+                  const float thr = rgrp == 0 ? t0 : rgrp == 1 ? t1 : rgrp == 2 ? t2 : t3;
+                  const unsigned long long pend = __ballot(rlive & (sub < CAND) & (own_c > thr));
+                  const unsigned m16 = (unsigned)(pend | (pend >> 16) | (pend >> 32) | (pend >> 48)) & 0xffffu;
+                  if (m16) {
+#pragma unroll
+                    for (int j = 0; j < CAND; ++j)
+                      if (m16 & (1u << j)) topk_insert(tkL[p2], tkI[p2], c[j], jb0 + rd * CAND + j);
+                  }
+                }
+              }
+            }
+            __builtin_amdgcn_wave_barrier();
+            return;
+          }
           // The bulk of the tiles under a causal mask: every row of the wave sees every key of the tile, so every block of
           // the tile is complete, visible and not the row's own, and (checked here) rows and blocks all exist.  Then a value's
           // address is one wave-uniform base per tile plus a per-lane offset that does not depend on the tile.
@@ -336,7 +445,31 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
     }
   }
 
-  if (POOL && !P.nofill) {
+  if (TK) {
+    // A query's selections: lane s of its group holds the s-th.  Their probabilities under the padded softmax of NSA.py:693-695
+    // follow from the entries alone wherever the mask can depend on them: every logit outside the list is at most the
+    // list's smallest, so leaving them out of the normaliser moves a probability near the 1e-10 threshold by less than its
+    // fp32 rounding (nb * 1e-10 relative).
+    const int sub = lane & 15, rgrp = lane >> 4;
+    const int rows_here = max(0, min(ppt, P.n - i0));
+#pragma unroll
+    for (int p2 = 0; p2 < TKP; ++p2) {
+      if (4 * p2 < rows_here) {
+        const float L = tkL[p2];
+        const float mx = fmaxf(-1e3f, row16_bcast_max(L));
+        const float e = __expf(L - mx);
+        const float sum = row16_bcast_sum(e) + __expf(-1e3f - mx);
+        const float pr = e * (1.0f / sum);
+        const int rr = 4 * p2 + rgrp;
+        if (rr < rows_here && sub < P.topk) {
+          const long at = ((long)bh * P.n + i0 + rr) * P.topk + sub;
+          tk_idx[at] = tkI[p2];
+          tk_mask[at] = (pr < INFINITY && pr > 1e-10f) ? 1 : 0;
+        }
+      }
+    }
+  }
+  if (POOL && !TK && !P.nofill) {
     // fine blocks whose compressed keys no query of this wave's tile can see were never visited
     const int last_visited = my_hi >= 0 ? min(walk.t_hi, my_hi / kBK) : -1;
     const int jstart = min(P.nb, (kBK * (last_visited + 1)) / (POOL ? NPF : 1));
@@ -1055,25 +1188,27 @@ extern "C" int nsa_dense_workspace_bytes(const nsa_dense_desc* d, size_t* bwd_by
   return 0;
 }
 
-template <int D, int NPF>
-static int dense_fwd_launch2(const DensePlan& P, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, hipStream_t st) {
+template <int D, int NPF, bool TK>
+static int dense_fwd_launch2(const DensePlan& P, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, int* tk_idx,
+                             uint8_t* tk_mask, hipStream_t st) {
   const int qpw = 4 * (32 >> P.lg);                 // queries per work-group
-  hipLaunchKernelGGL((dense_fwd_kernel<D, NPF>), dim3(P.mode == 0 ? xcd_grid_for((P.n + qpw - 1) / qpw) : (unsigned)((P.n + qpw - 1) / qpw), P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
-                     (const __bf16*)v, (__bf16*)out, lse, pooled);
+  hipLaunchKernelGGL((dense_fwd_kernel<D, NPF, TK>), dim3(P.mode == 0 ? xcd_grid_for((P.n + qpw - 1) / qpw) : (unsigned)((P.n + qpw - 1) / qpw), P.bh), dim3(256), 0, st, P, (const __bf16*)q, (const __bf16*)k,
+                     (const __bf16*)v, (__bf16*)out, lse, pooled, tk_idx, tk_mask);
   NSA_LAUNCH_CHECK();
   return 0;
 }
 
-template <int D>
-static int dense_fwd_launch(const DensePlan& P, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, hipStream_t st) {
+template <int D, bool TK>
+static int dense_fwd_launch(const DensePlan& P, const void* q, const void* k, const void* v, void* out, float* lse, float* pooled, int* tk_idx,
+                            uint8_t* tk_mask, hipStream_t st) {
   switch (P.pool ? P.npf : 0) {
-    case 0: return dense_fwd_launch2<D, 0>(P, q, k, v, out, lse, pooled, st);
-    case 1: return dense_fwd_launch2<D, 1>(P, q, k, v, out, lse, pooled, st);
-    case 2: return dense_fwd_launch2<D, 2>(P, q, k, v, out, lse, pooled, st);
-    case 4: return dense_fwd_launch2<D, 4>(P, q, k, v, out, lse, pooled, st);
-    case 8: return dense_fwd_launch2<D, 8>(P, q, k, v, out, lse, pooled, st);
-    case 16: return dense_fwd_launch2<D, 16>(P, q, k, v, out, lse, pooled, st);
-    case 32: return dense_fwd_launch2<D, 32>(P, q, k, v, out, lse, pooled, st);
+    case 0: if (!TK) return dense_fwd_launch2<D, 0, false>(P, q, k, v, out, lse, pooled, tk_idx, tk_mask, st); break;
+    case 1: return dense_fwd_launch2<D, 1, TK>(P, q, k, v, out, lse, pooled, tk_idx, tk_mask, st);
+    case 2: return dense_fwd_launch2<D, 2, TK>(P, q, k, v, out, lse, pooled, tk_idx, tk_mask, st);
+    case 4: return dense_fwd_launch2<D, 4, TK>(P, q, k, v, out, lse, pooled, tk_idx, tk_mask, st);
+    case 8: return dense_fwd_launch2<D, 8, TK>(P, q, k, v, out, lse, pooled, tk_idx, tk_mask, st);
+    case 16: return dense_fwd_launch2<D, 16, TK>(P, q, k, v, out, lse, pooled, tk_idx, tk_mask, st);
+    case 32: return dense_fwd_launch2<D, 32, TK>(P, q, k, v, out, lse, pooled, tk_idx, tk_mask, st);
   }
   return NSA_E_UNSUPPORTED;
 }
@@ -1083,8 +1218,29 @@ extern "C" int nsa_dense_fwd(const nsa_dense_desc* d, const void* q, const void*
   const int rc = make_dense_plan(d, P);
   if (rc) return rc;
   if (!q || !k || !v || !out || !lse || (P.pool && !pooled)) return NSA_E_ARG;
-  if (P.D == 64) return dense_fwd_launch<64>(P, q, k, v, out, lse, pooled, (hipStream_t)stream);
-  if (P.D == 128) return dense_fwd_launch<128>(P, q, k, v, out, lse, pooled, (hipStream_t)stream);
+  if (P.D == 64) return dense_fwd_launch<64, false>(P, q, k, v, out, lse, pooled, nullptr, nullptr, (hipStream_t)stream);
+  if (P.D == 128) return dense_fwd_launch<128, false>(P, q, k, v, out, lse, pooled, nullptr, nullptr, (hipStream_t)stream);
+  return NSA_E_UNSUPPORTED;
+}
+
+extern "C" int nsa_compress_topk_supported(const nsa_dense_desc* d, int32_t num_selected) {
+  DensePlan P;
+  if (make_dense_plan(d, P)) return 0;
+  // a wave serves its (at most 16) queries four at a time with 16 lanes each: selections shared by a group of >= 2 heads, <= 16 of them
+  return P.mode == 1 && P.pool && P.share && P.g >= 2 && num_selected >= 1 && num_selected <= 16 && num_selected <= P.nb;
+}
+
+extern "C" int nsa_compress_topk_fwd(const nsa_dense_desc* d, const void* q, const void* k, const void* v, void* out, float* lse,
+                                     int32_t num_selected, int32_t* idx, uint8_t* fmask, void* stream) {
+  DensePlan P;
+  const int rc = make_dense_plan(d, P);
+  if (rc) return rc;
+  if (!q || !k || !v || !out || !lse || !idx || !fmask) return NSA_E_ARG;
+  if (!nsa_compress_topk_supported(d, num_selected)) return NSA_E_UNSUPPORTED;
+  P.topk = num_selected;
+  P.nofill = 1;
+  if (P.D == 64) return dense_fwd_launch<64, true>(P, q, k, v, out, lse, nullptr, idx, fmask, (hipStream_t)stream);
+  if (P.D == 128) return dense_fwd_launch<128, true>(P, q, k, v, out, lse, nullptr, idx, fmask, (hipStream_t)stream);
   return NSA_E_UNSUPPORTED;
 }
 

@@ -12,6 +12,7 @@ struct DensePlan {
   int mode, causal, wb, wf, st;
   int st_sh;                 // log2(st) when the stride is a power of two (the division becomes a shift), else -1
   int pool, npf, nb, B, share, mask_own, nofill;
+  int topk;                  // > 0: the forward selects this many blocks per query itself instead of writing the logits
   int dkv_fp32;              // dk / dv leave the reduce kernel as fp32 instead of bf16
   float scale;
   int key_tiles, chunks, chunk_q;
@@ -35,6 +36,7 @@ static inline int make_dense_plan(const nsa_dense_desc* d, DensePlan& P) {
   const long bh = (long)P.b * P.hkv;
   if (bh > 65535) return NSA_E_UNSUPPORTED;
   P.bh = (int)bh;
+  P.topk = 0;
   P.wb = P.wf = 0; P.st = 1; P.pool = 0; P.npf = 1; P.nb = 0; P.B = 1; P.share = 1; P.mask_own = 0; P.nofill = 0;
   if (P.mode == 0) {
     if (d->window < 0 || P.mem != 0 || P.nkeys != P.n) return NSA_E_ARG;

@@ -472,6 +472,81 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
     return out, imp, ((q.shape[2], int(sel_block)) if use_prefix and imp is not None else None)
 
 
+@torch.library.custom_op("nsa_amd::compress_topk_fwd", mutates_args=())
+def compress_topk_fwd(q: Tensor, k: Tensor, v: Tensor, causal: bool, stride: int, num_mem: int, sel_block: int, num_sel: int,
+                      scale: float) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    """Compressed attention whose kernel also selects the blocks (nsa_compress_topk_fwd): (out, lse, idx int32, fmask uint8)."""
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    b, hq, n, d = q.shape
+    hk = k.shape[1]
+    if k.dim() != 4 or k.shape[0] != b or k.shape[3] != d or v.shape != k.shape or hq % hk or k.shape[2] < num_mem:
+        raise RuntimeError(f"q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}: expected 'b hq n d' and 'b hk keys d' with hk dividing hq")
+    out = torch.empty((b, hq, n, d), dtype=_BF16, device=q.device)
+    lse = torch.empty((b, hq, n), dtype=torch.float32, device=q.device)
+    idx = torch.empty((b, hk, n, num_sel), dtype=torch.int32, device=q.device)
+    fm = torch.empty((b, hk, n, num_sel), dtype=torch.uint8, device=q.device)
+    dsc = _dense_desc(q, k, v, out, out, 1, causal, 0, stride, num_mem, 1, sel_block, True, scale)
+    _lib.check(_lib.lib().nsa_compress_topk_fwd(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), int(num_sel), _ptr(idx), _ptr(fm),
+                                                _stream()), "nsa_compress_topk_fwd")
+    return out, lse, idx, fm
+
+
+@compress_topk_fwd.register_fake
+def _(q, k, v, causal, stride, num_mem, sel_block, num_sel, scale):
+    b, hq, n, d = q.shape
+    hk = k.shape[1]
+    return (q.new_empty((b, hq, n, d)), q.new_empty((b, hq, n), dtype=torch.float32),
+            q.new_empty((b, hk, n, num_sel), dtype=torch.int32), q.new_empty((b, hk, n, num_sel), dtype=torch.uint8))
+
+
+def _compress_topk_setup(ctx, inputs, output):
+    q, k, v, causal, stride, num_mem, sel_block, num_sel, scale = inputs
+    out, lse, _, _ = output
+    ctx.save_for_backward(q, k, v, out, lse)
+    ctx.args = (causal, stride, num_mem, scale)
+    ctx.set_materialize_grads(False)
+
+
+def _compress_topk_backward(ctx, dout, dlse, didx, dfm):
+    q, k, v, out, lse = ctx.saved_tensors
+    causal, stride, num_mem, scale = ctx.args
+    if dout is None:
+        return (None,) * 9
+    dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, 1, causal, 0, stride, num_mem, scale, False)
+    return (dq, dk, dv) + (None,) * 6
+
+
+compress_topk_fwd.register_autograd(_compress_topk_backward, setup_context=_compress_topk_setup)
+
+
+def compress_topk_supported(q: Tensor, ck: Tensor, num_mem: int, stride: int, sel_block: int, num_selected: int, share: bool) -> bool:
+    """Whether `compress_attend_topk` serves these shapes (else: `compress_attend` + `importance_topk`)."""
+    d = q.shape[-1]
+    hk = ck.shape[1]
+    g = q.shape[1] // hk
+    npf = int(sel_block) // int(stride)
+    nb = (ck.shape[2] - num_mem) // max(npf, 1)
+    return bool(share and q.is_cuda and d <= 128 and g >= 2 and not (g & (g - 1)) and npf >= 1 and npf <= 32 and not (npf & (npf - 1))
+                and int(sel_block) % int(stride) == 0 and 1 <= num_selected <= min(16, nb))
+
+
+def compress_attend_topk(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int, causal: bool, sel_block: int, num_selected: int):
+    """Compressed branch and block selection in one kernel: attend(q, [mem; ck], [mem; cv], cmask) of NSA.py:621-639 and, from
+    its logits, the importance scores, padded softmax, top-k and slot mask of NSA.py:652-721 (selections shared by the heads of a
+    group).  The importance logits are never written to memory.  Returns (out, idx int32 'b hk n k', fmask bool); `out` is
+    differentiable, the selection carries no gradient (for the differentiable top-k use compress_attend + importance_topk).
+    Needs compress_topk_supported(...)."""
+    d = q.shape[-1]
+    D = _kernel_dim(d)
+    hk = ck.shape[1]
+    q2, g, gp = _pad_groups(_pad_dim(q, D), hk)
+    if g != gp:
+        raise RuntimeError("compress_attend_topk: the group size must be a power of two")
+    out, _, idx, fm = compress_topk_fwd(q2, _pad_dim(ck, D), _pad_dim(cv, D), bool(causal), int(stride), int(num_mem), int(sel_block),
+                                        int(num_selected), float(d ** -0.5))
+    return out[..., :d], idx, fm.view(torch.bool)
+
+
 # ------------------------------------------------------------------------------------ top-k
 
 def _topk_impl(scores: Tensor, k: int, apply_softmax: bool, prefix=None):

@@ -454,24 +454,33 @@ class SparseAttention(nn.Module):
 
         want_sel = self.num_selected_blocks > 0 and nc > 0
         share = self.query_heads_share_selected_kv
-        # without differentiable top-k nothing but the top-k reads the importance logits: under a causal mask the kernel then
-        # writes, and the top-k reads, only the part of every row a query can select from (`prefix`)
-        prefix = None
-        if self.use_diff_topk:
-            c_out, imp = ops.compress_attend(q16 if fused else q.to(bf16), ck.to(bf16), cv.to(bf16), M, st, self.causal,
-                                             sel_block=B if want_sel else None, share=share)
+        qc = q16 if fused else q.to(bf16)
+        ck16, cv16 = ck.to(bf16), cv.to(bf16)
+        npf = B // st
+        num_sel = min(self.num_selected_blocks, nc // npf) if want_sel else 0
+        vals = idx = fmask = None
+        if num_sel > 0 and not self.use_diff_topk and ops.compress_topk_supported(qc, ck16, M, st, B, num_sel, share):
+            # without differentiable top-k nothing but the selection reads the importance scores: the compressed forward makes
+            # the selection itself and the scores never reach memory
+            c_out, idx, fmask = ops.compress_attend_topk(qc, ck16, cv16, M, st, self.causal, B, num_sel)
+        elif num_sel > 0:
+            # the logits are written out (under a causal mask, without differentiable top-k, only the part of every row a
+            # query can select from: logits and `prefix` stay together between these two calls)
+            if self.use_diff_topk:
+                c_out, imp = ops.compress_attend(qc, ck16, cv16, M, st, self.causal, sel_block=B, share=share)
+                prefix = None
+            else:
+                c_out, imp, prefix = ops.compress_attend(qc, ck16, cv16, M, st, self.causal, sel_block=B, share=share, prefix_only=True)
+            vals, idx, fmask = ops.importance_topk(imp, num_sel, prefix=prefix)
         else:
-            c_out, imp, prefix = ops.compress_attend(q16 if fused else q.to(bf16), ck.to(bf16), cv.to(bf16), M, st, self.causal,
-                                                     sel_block=B if want_sel else None, share=share, prefix_only=True)
+            c_out, _ = ops.compress_attend(qc, ck16, cv16, M, st, self.causal)
 
         if not fused:
             # rotary positions for the selection and sliding branches (NSA.py:643), one HIP kernel each
             rq16, rk16 = ops.rotary_pair(q.to(bf16), k.to(bf16), self.rotary_emb.freqs)
             v16 = v.to(bf16)
 
-        num_sel = min(self.num_selected_blocks, imp.shape[-1]) if imp is not None else 0
         if num_sel > 0:
-            vals, idx, fmask = ops.importance_topk(imp, num_sel, prefix=prefix)
             # straight-through gates (NSA.py:715): value 1, gradient flows into the importance scores
             gates = (vals + (1. - vals).detach()) if self.use_diff_topk else None
             f_out = ops.native_sparse_attend(rq16, rk16, v16, B, idx, fmask, sel_scale=gates, include_block_causal=self.causal)

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import nsa_oracle as O
-from tests.util import assert_close, assert_grad_close, causal_random_selection
+from tests.util import assert_close, assert_grad_close, capture_selection, causal_random_selection
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -86,23 +86,15 @@ def test_config3_full_module_forward_backward():
     do = torch.randn(b, n, kw["dim"], generator=g).to(torch.bfloat16)
 
     captured = {}
-    orig = ops.importance_topk
-    def spy(imp, k_, **kw_):
-        r = orig(imp, k_, **kw_)
-        captured["sel"] = (r[1].cpu().long(), r[2].cpu())
-        return r
 
     def run(xs, dos):
         for p in mod.parameters():
             p.grad = None
         xg = xs.to(DEV).requires_grad_()
-        ops.importance_topk = spy
-        try:
+        with capture_selection(captured):
             out = mod(xg)
             (out.float() * dos.to(DEV).float()).sum().backward()
             torch.cuda.synchronize()
-        finally:
-            ops.importance_topk = orig
         grads = {name: p.grad.float().cpu() for name, p in mod.named_parameters() if p.grad is not None}
         return out.detach().cpu(), xg.grad.cpu(), grads, captured["sel"]
 

@@ -15,7 +15,7 @@ import torch
 from torch import nn
 
 from oracle import nsa_oracle as O
-from tests.util import assert_close
+from tests.util import assert_close, capture_selection
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -108,21 +108,12 @@ def test_module_matches_oracle(ci, n):
     do = torch.randn(b, n, kw["dim"], generator=g).to(torch.bfloat16)
 
     # --- HIP path, capturing its selection
-    from native_sparse_attention_pytorch_amd import ops
     captured = {}
-    orig = ops.importance_topk
-    def spy(imp, k, **kw_):
-        r = orig(imp, k, **kw_)
-        captured["sel"] = (r[1].cpu().long(), r[2].cpu())
-        return r
-    ops.importance_topk = spy
-    try:
+    with capture_selection(captured):
         xg = x.to(DEV).requires_grad_()
         out = mod(xg)
         (out.float() * do.to(DEV).float()).sum().backward()
         torch.cuda.synchronize()
-    finally:
-        ops.importance_topk = orig
     assert out.shape == x.shape
     idx, live = captured["sel"]
 
@@ -198,20 +189,11 @@ def test_fp32_module_runs_and_matches_oracle():
     mod.load_state_dict(ref.state_dict(), strict=True)
     mod = mod.to(DEV)                                   # fp32
     x = torch.randn(2, 90, 128, generator=torch.Generator().manual_seed(5))
-    from native_sparse_attention_pytorch_amd import ops
     captured = {}
-    orig = ops.importance_topk
-    def spy(imp, k, **kw_):
-        r = orig(imp, k, **kw_)
-        captured["sel"] = (r[1].cpu().long(), r[2].cpu())
-        return r
-    ops.importance_topk = spy
-    try:
+    with capture_selection(captured):
         xg = x.to(DEV).requires_grad_()
         out = mod(xg)
         out.sum().backward()
-    finally:
-        ops.importance_topk = orig
     assert out.dtype == torch.float32 and xg.grad is not None and torch.isfinite(xg.grad).all()
     xr = x.clone().requires_grad_()
     want = ref(xr, selection_override=captured["sel"])

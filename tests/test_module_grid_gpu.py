@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from oracle import nsa_oracle as O
-from tests.util import assert_close
+from tests.util import assert_close, capture_selection
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -45,17 +45,8 @@ def _case(diff, causal, n, kvh, B, cbs, st, S, share, seed):
     mod = mod.to(DEV).to(torch.bfloat16)
     x = torch.randn(2, n, 128, generator=torch.Generator().manual_seed(seed + 1)).to(torch.bfloat16)
     captured = {}
-    orig = ops.importance_topk
-
-    def spy(imp, k, **kw_):
-        r = orig(imp, k, **kw_)
-        captured["sel"] = (r[1].cpu().long(), r[2].cpu())
-        return r
-    ops.importance_topk = spy
-    try:
+    with capture_selection(captured):
         out = mod(x.to(DEV))
-    finally:
-        ops.importance_topk = orig
     assert out.shape == x.shape
     want = ref(x.float(), selection_override=captured.get("sel"))
     assert_close(out, want, 3e-2 * want.abs().max().item() + 1e-3, 2e-2, f"case {kw} n={n}")

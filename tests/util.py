@@ -1,4 +1,5 @@
 """Shared helpers for the parity tests."""
+import contextlib
 import math
 
 import torch
@@ -49,3 +50,27 @@ def assert_grad_close(got, want, what=""):
     e = err / max(w.norm().item(), 1e-12)
     assert e < 5e-2 or err <= floor, f"{what}: relative error {e:.4f} (norm-wise) exceeds 5e-2"
     assert_close(got, want, 2e-2 * w.abs().max().item() + 1e-6, 5e-2, what)
+
+
+@contextlib.contextmanager
+def capture_selection(captured):
+    """While active, the block selection the module makes - through `ops.importance_topk` (logits written out) or
+    `ops.compress_attend_topk` (selection inside the compressed forward) - is recorded in captured["sel"] as CPU
+    (idx int64, fmask bool), and captured["via"] names the path."""
+    from native_sparse_attention_pytorch_amd import ops
+    orig_topk, orig_fused = ops.importance_topk, ops.compress_attend_topk
+
+    def spy_topk(imp, k, **kw):
+        r = orig_topk(imp, k, **kw)
+        captured["sel"], captured["via"] = (r[1].cpu().long(), r[2].cpu()), "importance_topk"
+        return r
+
+    def spy_fused(*a, **kw):
+        r = orig_fused(*a, **kw)
+        captured["sel"], captured["via"] = (r[1].cpu().long(), r[2].cpu()), "compress_attend_topk"
+        return r
+    ops.importance_topk, ops.compress_attend_topk = spy_topk, spy_fused
+    try:
+        yield captured
+    finally:
+        ops.importance_topk, ops.compress_attend_topk = orig_topk, orig_fused
