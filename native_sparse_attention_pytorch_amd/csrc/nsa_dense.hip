@@ -302,14 +302,13 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
               }
             }
             if (TK) {
-              // the staged values are the final logits: scaled, -inf where the block cannot be selected, NaN ordered first
+              // the staged values are the final logits: scaled, -inf where the block cannot be selected
               const float norm_t = P.scale / (float)(npf * (SH ? P.g : 1));
               const int jbt = kb0 / npf, qi_t = i0 + prow_local;
               const bool all_vis = P.causal && plain && i0 + ppt <= P.n && jbt + nbt <= P.nb;      // wave-uniform, as `direct` below
 #pragma unroll
               for (int vi = 0; vi < NV; ++vi) {
-                float x = val[vi] * norm_t;
-                x = (x == x) ? x : INFINITY;
+                float x = val[vi] * norm_t;            // (a NaN logit never compares greater: it is not selected)
                 if (!all_vis) {
                   const int jblk = jbt + (32 * kt + koff[vi]) / npf;
                   const int blo = jblk * P.B, bhi = blo + P.B;
@@ -336,39 +335,52 @@ __global__ __launch_bounds__(256, 2) void dense_fwd_kernel(const DensePlan P, co
             // ballot says which candidate positions have a taker in any of the four queries, and only those run the insert.
             constexpr int CAND = nbt < 16 ? nbt : 16, RDS = nbt / CAND;
             const int sub = lane & 15, rgrp = lane >> 4;
+            // (the reads of all groups of four first, then the tests, then the inserts: one LDS round trip for the lot)
+            float own_c[TKP][RDS], thr[TKP];
+            const float* prow[TKP];
+#pragma unroll
+            for (int p2 = 0; p2 < TKP; ++p2) {
+              prow[p2] = pw + min(4 * p2 + rgrp, rows_here - 1) * nbt;
+              if (4 * p2 < rows_here) {
+#pragma unroll
+                for (int rd = 0; rd < RDS; ++rd) own_c[p2][rd] = prow[p2][rd * CAND + (sub < CAND ? sub : 0)];
+                // the group's last entry, from its lane 15 (swizzle inside 32 lanes: source lane = (lane & 16) | 15)
+                thr[p2] = __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, tkL[p2]), 0x1F0));
+              }
+            }
 #pragma unroll
             for (int p2 = 0; p2 < TKP; ++p2) {
               if (4 * p2 < rows_here) {
-                const int rr = 4 * p2 + rgrp;
-                const bool rlive = rr < rows_here;
-                const float* prow = pw + min(rr, rows_here - 1) * nbt;
+                const bool rlive = 4 * p2 + rgrp < rows_here;
 #pragma unroll
                 for (int rd = 0; rd < RDS; ++rd) {
-                  float c[CAND];
-                  if (CAND >= 4) {
-#pragma unroll
-                    for (int j4 = 0; j4 < CAND / 4; ++j4) {
-                      const floatx4 t4 = *reinterpret_cast<const floatx4*>(prow + rd * CAND + 4 * j4);
-#pragma unroll
-                      for (int e = 0; e < 4; ++e) c[4 * j4 + e] = t4[e];
-                    }
-                  } else {
-#pragma unroll
-                    for (int j = 0; j < CAND; ++j) c[j] = prow[rd * CAND + j];
-                  }
-                  const float own_c = prow[rd * CAND + (sub < CAND ? sub : 0)];
-                  const float l15 = tkL[p2];
-                  const float t0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, l15), 15));
-                  const float t1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, l15), 31));
-                  const float t2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, l15), 47));
-                  const float t3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, l15), 63));
-                  const float thr = rgrp == 0 ? t0 : rgrp == 1 ? t1 : rgrp == 2 ? t2 : t3;
-                  const unsigned long long pend = __ballot(rlive & (sub < CAND) & (own_c > thr));
+                  // (with several rounds per tile the threshold of the first serves them all: a lower bound lets no-ops through)
+                  const unsigned long long pend = __ballot(rlive & (sub < CAND) & (own_c[p2][rd] > thr[p2]));
                   const unsigned m16 = (unsigned)(pend | (pend >> 16) | (pend >> 32) | (pend >> 48)) & 0xffffu;
                   if (m16) {
+                    float c[CAND];
+                    if (CAND >= 4) {
 #pragma unroll
-                    for (int j = 0; j < CAND; ++j)
-                      if (m16 & (1u << j)) topk_insert(tkL[p2], tkI[p2], c[j], jb0 + rd * CAND + j);
+                      for (int j4 = 0; j4 < CAND / 4; ++j4) {
+                        const floatx4 t4 = *reinterpret_cast<const floatx4*>(prow[p2] + rd * CAND + 4 * j4);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) c[4 * j4 + e] = t4[e];
+                      }
+                    } else {
+#pragma unroll
+                      for (int j = 0; j < CAND; ++j) c[j] = prow[p2][rd * CAND + j];
+                    }
+                    // positions four at a time: late in a walk most groups of four have no taker
+#pragma unroll
+                    for (int j4 = 0; j4 < (CAND + 3) / 4; ++j4) {
+                      if (m16 & (0xfu << (4 * j4))) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                          const int j = 4 * j4 + e;
+                          if (j < CAND && (m16 & (1u << j))) topk_insert(tkL[p2], tkI[p2], c[j], jb0 + rd * CAND + j);
+                        }
+                      }
+                    }
                   }
                 }
               }
