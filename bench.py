@@ -173,7 +173,7 @@ def main():
             be = C.cast(C.byref(ev, 4 * C.sizeof(C.c_void_p)), C.c_void_p) if ev is not None else None
             _lib.check(L.nsa_select_fwd_timed(C.byref(dsc), P(q), P(k), P(v), P(idx), P(fm), P(iws), P(ws), fb, P(out), P(lse), stream,
                                               fe, 3 if ev is not None else 0), "fwd")
-            _lib.check(L.nsa_select_bwd_timed(C.byref(dsc), P(q), P(k), P(v), P(out), P(do), P(lse), P(idx), P(fm), P(iws), P(ws), wb,
+            _lib.check(L.nsa_select_bwd_timed(C.byref(dsc), P(q), P(k), P(v), P(out), P(do), None, P(lse), P(idx), P(fm), P(iws), P(ws), wb,
                                               P(dq), P(dk), P(dv), None, stream, be, 6 if ev is not None else 0), "bwd")
 
         for _ in range(warmup):

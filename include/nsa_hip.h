@@ -86,9 +86,12 @@ int nsa_select_fwd(const nsa_select_desc* d, const void* q, const void* k, const
  * (The reference accumulates all three through global fp32 atomics, TRI.py:758-788, 1395-1425.)
  * sel_grads: NULL, or fp32 contiguous [batch, kv_heads, seq, num_sel] receiving the gradient of a
  * multiplier of value 1 on each slot's keys (the straight-through top-k gates `sel_scale`,
- * TRI.py:1061-1080, NSA.py:793-797); dead slots get 0. */
+ * TRI.py:1061-1080, NSA.py:793-797); dead slots get 0.
+ * d_lse: NULL, or fp32 contiguous like lse: the upstream gradient of the returned log-sum-exp (the reference's lse
+ * output carries none; here it lets a caller merge the results of several calls over disjoint slot sets by their lse
+ * and still differentiate the merge). */
 int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const void* v,
-                   const void* out, const void* d_out, const float* lse,
+                   const void* out, const void* d_out, const float* d_lse, const float* lse,
                    const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
                    void* dq, void* dk, void* dv, float* sel_grads, void* stream);
 
@@ -406,7 +409,7 @@ int nsa_select_fwd_timed(const nsa_select_desc* d, const void* q, const void* k,
                          const void* idx, const uint8_t* fmask, const void* index_ws, void* fwd_ws, size_t fwd_bytes,
                          void* out, float* lse, void* stream, void* const* events, int num_events);
 int nsa_select_bwd_timed(const nsa_select_desc* d, const void* q, const void* k, const void* v,
-                         const void* out, const void* d_out, const float* lse,
+                         const void* out, const void* d_out, const float* d_lse, const float* lse,
                          const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
                          void* dq, void* dk, void* dv, float* sel_grads, void* stream, void* const* events, int num_events);
 

@@ -77,7 +77,7 @@ def lib():
         L.nsa_select_workspace_bytes.argtypes = [C.POINTER(SelectDesc), C.POINTER(sz), C.POINTER(sz), C.POINTER(sz)]
         L.nsa_select_build_index.argtypes = [C.POINTER(SelectDesc), vp, vp, vp, sz, vp]
         L.nsa_select_fwd.argtypes = [C.POINTER(SelectDesc), vp, vp, vp, vp, vp, vp, vp, sz, vp, vp, vp]
-        L.nsa_select_bwd.argtypes = [C.POINTER(SelectDesc)] + [vp] * 10 + [sz] + [vp] * 5
+        L.nsa_select_bwd.argtypes = [C.POINTER(SelectDesc)] + [vp] * 11 + [sz] + [vp] * 5
         L.nsa_selftest_mfma.argtypes = [vp] * 6
         L.nsa_selftest_mfma.restype = C.c_int
         L.nsa_probe_row_traffic.argtypes = [vp, sz, vp, sz, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_uint32, vp]

@@ -636,9 +636,11 @@ __global__ __launch_bounds__(256) void sel_fwd_combine_kernel(const SelPlan P, c
 
 // ------------------------------------------------------------------------------ backward
 
-// delta[b,hq,i] = sum_d out * d_out   (TRI.py:696-756)
+// delta[b,hq,i] = sum_d out * d_out   (TRI.py:696-756), less the gradient of the row's log-sum-exp when the caller has one:
+// d loss / d logit_j = p_j (dP_j - sum_k p_k dP_k) + d_lse p_j = p_j (dP_j - (delta - d_lse))
 template <int D>
-__global__ __launch_bounds__(256) void sel_delta_kernel(const SelPlan P, const __bf16* __restrict__ out, const __bf16* __restrict__ dout, float* __restrict__ delta) {
+__global__ __launch_bounds__(256) void sel_delta_kernel(const SelPlan P, const __bf16* __restrict__ out, const __bf16* __restrict__ dout,
+                                                        const float* __restrict__ dlse, float* __restrict__ delta) {
   constexpr int LPR = D / 8;                   // lanes per row
   constexpr int RPB = 256 / LPR;               // rows per block
   const int tid = threadIdx.x;
@@ -656,7 +658,7 @@ __global__ __launch_bounds__(256) void sel_delta_kernel(const SelPlan P, const _
   }
 #pragma unroll
   for (int m = LPR / 2; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
-  if (row < rows && (tid % LPR) == 0) delta[row] = s;
+  if (row < rows && (tid % LPR) == 0) delta[row] = dlse ? s - dlse[row] : s;
 }
 
 // dQ partial of every (query, slot) pair; same walk and register layout as the forward
@@ -1233,13 +1235,13 @@ extern "C" int nsa_select_fwd(const nsa_select_desc* d, const void* q, const voi
 }
 
 template <int D, int KT>
-static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void* v, const void* out, const void* dout, const float* lse,
+static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void* v, const void* out, const void* dout, const float* dlse, const float* lse,
                       const void* idx, const uint8_t* fmask, const void* iws, void* bws, void* dq, void* dk, void* dv, float* sel_grads, hipStream_t st, void* const* ev, int nev) {
   mark(ev, nev, 0, st);
   float* delta = reinterpret_cast<float*>((char*)bws + P.off_delta);
   const long rows = (long)P.bh * P.g * P.n;
   constexpr int RPB = 256 / (D / 8);
-  hipLaunchKernelGGL((sel_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, delta);
+  hipLaunchKernelGGL((sel_delta_kernel<D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, P, (const __bf16*)out, (const __bf16*)dout, dlse, delta);
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 1, st);
   // without gate gradients the dQ partials come out of the dK/dV walk (one gather of Q and dO
@@ -1271,7 +1273,7 @@ static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void
 }
 
 extern "C" int nsa_select_bwd_timed(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* out, const void* d_out,
-                                    const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
+                                    const float* d_lse, const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
                                     void* dq, void* dk, void* dv, float* sel_grads, void* stream, void* const* ev, int nev) {
   SelPlan P;
   const int rc = make_plan(d, P);
@@ -1280,17 +1282,17 @@ extern "C" int nsa_select_bwd_timed(const nsa_select_desc* d, const void* q, con
   if (!q || !k || !v || !out || !d_out || !lse || !index_ws || !bwd_ws || !dq || !dk || !dv) return NSA_E_ARG;
   hipStream_t st = (hipStream_t)stream;
   const int KT = (P.B + 31) / 32;
-  if (P.D == 64 && KT == 1) return launch_bwd<64, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
-  if (P.D == 64 && KT == 2) return launch_bwd<64, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
-  if (P.D == 128 && KT == 1) return launch_bwd<128, 1>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
-  if (P.D == 128 && KT == 2) return launch_bwd<128, 2>(P, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
+  if (P.D == 64 && KT == 1) return launch_bwd<64, 1>(P, q, k, v, out, d_out, d_lse, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
+  if (P.D == 64 && KT == 2) return launch_bwd<64, 2>(P, q, k, v, out, d_out, d_lse, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
+  if (P.D == 128 && KT == 1) return launch_bwd<128, 1>(P, q, k, v, out, d_out, d_lse, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
+  if (P.D == 128 && KT == 2) return launch_bwd<128, 2>(P, q, k, v, out, d_out, d_lse, lse, idx, fmask, index_ws, bwd_ws, dq, dk, dv, sel_grads, st, ev, nev);
   return NSA_E_UNSUPPORTED;
 }
 
 extern "C" int nsa_select_bwd(const nsa_select_desc* d, const void* q, const void* k, const void* v, const void* out, const void* d_out,
-                              const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
+                              const float* d_lse, const float* lse, const void* idx, const uint8_t* fmask, const void* index_ws, void* bwd_ws, size_t bwd_bytes,
                               void* dq, void* dk, void* dv, float* sel_grads, void* stream) {
-  return nsa_select_bwd_timed(d, q, k, v, out, d_out, lse, idx, fmask, index_ws, bwd_ws, bwd_bytes, dq, dk, dv, sel_grads, stream, nullptr, 0);
+  return nsa_select_bwd_timed(d, q, k, v, out, d_out, d_lse, lse, idx, fmask, index_ws, bwd_ws, bwd_bytes, dq, dk, dv, sel_grads, stream, nullptr, 0);
 }
 
-extern "C" int nsa_abi_version(void) { return 5; }
+extern "C" int nsa_abi_version(void) { return 6; }

@@ -133,8 +133,11 @@ def _(q, k, v, idx, fmask, sel_scale, block, causal, scale):
 
 @torch.library.custom_op("nsa_amd::select_bwd", mutates_args=())
 def select_bwd(q: Tensor, k: Tensor, v: Tensor, out: Tensor, dout: Tensor, lse: Tensor, idx: Tensor, fmask: Tensor,
-               index_ws: Tensor, block: int, causal: bool, scale: float, want_sel_grads: bool) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+               index_ws: Tensor, block: int, causal: bool, scale: float, want_sel_grads: bool,
+               dlse: Optional[Tensor] = None) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     q, k, v = _prep(q), _prep(k), _prep(v)
+    if dlse is not None:
+        dlse = dlse.to(torch.float32).contiguous()
     out = out.contiguous()
     dout = dout.contiguous()
     if dout.dtype != _BF16:
@@ -152,14 +155,14 @@ def select_bwd(q: Tensor, k: Tensor, v: Tensor, out: Tensor, dout: Tensor, lse: 
         raise RuntimeError("inverse index workspace does not belong to these shapes")
     bwd_ws = torch.empty(wb, dtype=torch.uint8, device=q.device)
     dsel = torch.empty(idx.shape if want_sel_grads else (0,), dtype=torch.float32, device=q.device)
-    _lib.check(_lib.lib().nsa_select_bwd(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(lse), _ptr(idx), _ptr(fm),
+    _lib.check(_lib.lib().nsa_select_bwd(C.byref(dsc), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(dout), _ptr(dlse), _ptr(lse), _ptr(idx), _ptr(fm),
                                          _ptr(index_ws), _ptr(bwd_ws), wb, _ptr(dq), _ptr(dk), _ptr(dv),
                                          _ptr(dsel) if want_sel_grads else 0, _stream()), "nsa_select_bwd")
     return dq, dk, dv, dsel
 
 
 @select_bwd.register_fake
-def _(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale, want_sel_grads):
+def _(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale, want_sel_grads, dlse=None):
     return (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
             q.new_empty(idx.shape if want_sel_grads else (0,), dtype=torch.float32))
 
@@ -175,9 +178,11 @@ def _select_setup(ctx, inputs, output):
 def _select_backward(ctx, dout, dlse, dws):
     q, k, v, out, lse, idx, fmask, index_ws = ctx.saved_tensors
     block, causal, scale, want, sdtype = ctx.args
-    if dout is None:
+    if dout is None and dlse is None:
         return (None,) * 9
-    dq, dk, dv, dsel = select_bwd(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale, want)
+    if dout is None:
+        dout = torch.zeros_like(out)
+    dq, dk, dv, dsel = select_bwd(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale, want, dlse)
     return dq, dk, dv, None, None, (dsel.to(sdtype) if want else None), None, None, None
 
 
@@ -226,6 +231,47 @@ def _dead_rows_uniform(out: Tensor, fv: Tensor, selected_block_indices: Tensor, 
     return torch.where(dead.repeat_interleave(g, dim=1)[..., None], avg.repeat_interleave(g, dim=1).to(out.dtype), out)
 
 
+_MAX_GRID_BH = 65535      # batch * kv heads of one launch (a grid dimension)
+_MAX_SLOTS = 62           # slots of one call of the selection kernels (a query's live slots are a 64-bit mask, one bit the own block)
+
+
+def _batch_pieces(b: int, hk: int):
+    """Batch ranges whose batch * kv heads fit one launch (None: the whole batch does)."""
+    if b * hk <= _MAX_GRID_BH:
+        return None
+    if hk > _MAX_GRID_BH:
+        raise RuntimeError(f"{hk} kv heads: more than one launch can address")
+    step = _MAX_GRID_BH // hk
+    return [(lo, min(b, lo + step)) for lo in range(0, b, step)]
+
+
+def _select_core(q: Tensor, k: Tensor, v: Tensor, idx: Tensor, fm: Tensor, sc: Tensor | None, block: int, causal: bool, scale: float):
+    """select_fwd on any batch size and any number of slots: (out, lse).  A batch too large for one launch is cut along the
+    batch axis; more than 62 slots are cut into groups whose results are merged by their log-sum-exp,
+    out = sum_i exp(lse_i - L) out_i with L = logsumexp_i(lse_i) - the softmax over the union of the groups' keys - with the
+    own block in the first group only (gradients flow through the merge: the selection backward takes d_lse)."""
+    pieces = _batch_pieces(q.shape[0], k.shape[1])
+    if pieces is not None:
+        outs = [_select_core(q[lo:hi], k[lo:hi], v[lo:hi], idx[lo:hi], fm[lo:hi], None if sc is None else sc[lo:hi], block, causal, scale)
+                for lo, hi in pieces]
+        return torch.cat([o for o, _ in outs], dim=0), torch.cat([l for _, l in outs], dim=0)
+    S = idx.shape[-1]
+    if S <= _MAX_SLOTS:
+        out, lse, _ = select_fwd(q, k, v, idx, fm, sc, block, causal, scale)
+        return out, lse
+    outs, lses = [], []
+    for g0 in range(0, S, _MAX_SLOTS):
+        sl = slice(g0, min(S, g0 + _MAX_SLOTS))
+        o, l, _ = select_fwd(q, k, v, idx[..., sl].contiguous(), fm[..., sl].contiguous(), None if sc is None else sc[..., sl].contiguous(),
+                             block, causal and g0 == 0, scale)
+        outs.append(o.float())
+        lses.append(l)
+    L = torch.logsumexp(torch.stack(lses), dim=0)
+    Ls = torch.where(torch.isfinite(L), L, torch.zeros_like(L))        # rows that attend nothing: every weight exp(-inf - 0) = 0
+    out = sum(torch.exp(l - Ls)[..., None] * o for o, l in zip(outs, lses))
+    return out.to(q.dtype), L
+
+
 def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, selected_block_indices: Tensor, fmask: Tensor,
                          sel_scale: Tensor | None = None, include_block_causal: bool = True, return_lse: bool = False,
                          block_dk_dv_use_dot=None, return_sliding_window_out: bool = False):
@@ -270,7 +316,7 @@ def native_sparse_attend(fq: Tensor, fk: Tensor, fv: Tensor, block_size: int, se
         sc_in = None if sc_in is None else padn(sc_in, 1.0)
     qp, g0, gp0 = _pad_groups(fq, fk.shape[1])
     idx_k, fm_k, sc_k, block_k = _split_blocks(idx_in, fm_in, sc_in, int(block_size), fq.shape[2], bool(include_block_causal))
-    out, lse, _ = select_fwd(qp, fk, fv, idx_k, fm_k, sc_k, block_k, bool(include_block_causal), float(scale))
+    out, lse = _select_core(qp, fk, fv, idx_k, fm_k, sc_k, block_k, bool(include_block_causal), float(scale))
     out, lse = _unpad_groups(out, fk.shape[1], g0, gp0)[:, :, :n, :d_head], _unpad_groups(lse, fk.shape[1], g0, gp0)[:, :, :n]
     fv = fv_given if kv_heads == sel_heads else fv_given.repeat_interleave(q_heads // kv_heads, dim=1)
     if not include_block_causal and selected_block_indices.shape[-1] > 0:
@@ -416,6 +462,9 @@ def sliding_attend(q: Tensor, k: Tensor, v: Tensor, window_size: int, causal: bo
     """Sliding-window branch: what `self.sliding_window(sq, sk, sv)` computes at NSA.py:841-850
     (LocalAttention with exact window, autopad) without materialising the repeated k/v:
     q [b,Hq,n,d], k/v [b,Hkv,n,d]; query i sees 0 <= i-j <= window_size (causal) or |i-j| <= it."""
+    pieces = _batch_pieces(q.shape[0], k.shape[1])
+    if pieces is not None:
+        return torch.cat([sliding_attend(q[lo:hi], k[lo:hi], v[lo:hi], window_size, causal) for lo, hi in pieces], dim=0)
     d = q.shape[-1]
     D = _kernel_dim(d)
     qp, g, gp = _pad_groups(_pad_dim(q, D), k.shape[1])
@@ -433,6 +482,12 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
     of the logits is defined only below column i // sel_block - what a causal query can select from; the rest (all -inf
     otherwise) was not written and must not be read: pass `prefix` on to `importance_topk`.  Only for logits nothing else
     reads (no gradient through them)."""
+    pieces = _batch_pieces(q.shape[0], ck.shape[1])
+    if pieces is not None:
+        parts = [compress_attend(q[lo:hi], ck[lo:hi], cv[lo:hi], num_mem, stride, causal, sel_block, share, prefix_only) for lo, hi in pieces]
+        cat = lambda ts: None if ts[0] is None else torch.cat(ts, dim=0)
+        res = (cat([p_[0] for p_ in parts]), cat([p_[1] for p_ in parts]))
+        return res + (parts[0][2],) if prefix_only else res
     pool = sel_block is not None
     d = q.shape[-1]
     scale = float(d ** -0.5)
@@ -536,6 +591,10 @@ def compress_attend_topk(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride
     group).  The importance logits are never written to memory.  Returns (out, idx int32 'b hk n k', fmask bool); `out` is
     differentiable, the selection carries no gradient (for the differentiable top-k use compress_attend + importance_topk).
     Needs compress_topk_supported(...)."""
+    pieces = _batch_pieces(q.shape[0], ck.shape[1])
+    if pieces is not None:
+        parts = [compress_attend_topk(q[lo:hi], ck[lo:hi], cv[lo:hi], num_mem, stride, causal, sel_block, num_selected) for lo, hi in pieces]
+        return tuple(torch.cat([p_[t] for p_ in parts], dim=0) for t in range(3))
     d = q.shape[-1]
     D = _kernel_dim(d)
     hk = ck.shape[1]
@@ -549,9 +608,61 @@ def compress_attend_topk(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride
 
 # ------------------------------------------------------------------------------------ top-k
 
+_TOPK_MAX_ROW, _TOPK_MAX_K = 2048, 64      # one call of the top-k kernel: a row in the registers of one wave, one result per lane
+
+
+def _topk_large(scores: Tensor, k: int, apply_softmax: bool, prefix=None):
+    """Rows longer than 2048 entries or more than 64 selections (the reference's topk, NSA.py:703-713, has no limit): the
+    padded softmax over the whole row is taken first (NSA.py:693-695, elementwise torch), then the kernel selects per
+    segment of 2048 columns and once more among the segments' winners, 64 at a time, taken entries struck out in between.
+    The tie rule survives both steps: a segment lists equal values lower index first, and the winners of a lower segment
+    stand before those of a higher one."""
+    nb = scores.shape[-1]
+    work = scores
+    if prefix is not None:
+        seq, block = prefix
+        lim = (torch.arange(seq, device=scores.device) // block)[:, None]
+        work = work.masked_fill(torch.arange(nb, device=scores.device)[None, :] >= lim, float("-inf"))
+    if apply_softmax:
+        work = torch.nn.functional.pad(work, (1, 0), value=-1e3).softmax(dim=-1)[..., 1:]
+    work = work.contiguous().clone()
+    segs = [(lo, min(nb, lo + _TOPK_MAX_ROW)) for lo in range(0, nb, _TOPK_MAX_ROW)]
+    idx_parts, val_parts = [], []
+    left = k
+    while left > 0:
+        kk = min(_TOPK_MAX_K, left)
+        cand_v, cand_i = [], []
+        for lo, hi in segs:
+            ks = min(kk, hi - lo)
+            i_s, v_s, _ = _topk_impl(work[..., lo:hi].contiguous(), ks, False)
+            cand_v.append(v_s)
+            cand_i.append(i_s.long() + lo)
+        cv_, ci_ = torch.cat(cand_v, dim=-1), torch.cat(cand_i, dim=-1)
+        if len(segs) > 1:
+            if cv_.shape[-1] > _TOPK_MAX_ROW:
+                raise RuntimeError(f"top-k over {nb} entries with k = {k}: more candidates than one merge step holds")
+            pos, v_m, _ = _topk_impl(torch.nan_to_num(cv_, nan=float("inf")).contiguous(), kk, False)
+            i_m = ci_.gather(-1, pos.long())
+            v_m = cv_.gather(-1, pos.long())
+        else:
+            i_m, v_m = ci_, cv_
+        idx_parts.append(i_m)
+        val_parts.append(v_m)
+        work.scatter_(-1, i_m, -3.0)                    # below every probability and the kernel's own markers
+        left -= kk
+    idx = torch.cat(idx_parts, dim=-1).to(torch.int32)
+    vals = torch.cat(val_parts, dim=-1)
+    fm = ((vals > 1e-10) & torch.isfinite(vals)).to(torch.uint8)
+    return idx, vals, fm
+
+
 def _topk_impl(scores: Tensor, k: int, apply_softmax: bool, prefix=None):
     if scores.dtype != torch.float32 or not scores.is_cuda:
         raise RuntimeError("importance scores must be fp32 device tensors")
+    if scores.shape[-1] > _TOPK_MAX_ROW or k > _TOPK_MAX_K:
+        if k > scores.shape[-1]:
+            raise RuntimeError(f"top-k of {k} among {scores.shape[-1]} entries")
+        return _topk_large(scores, int(k), bool(apply_softmax), prefix)
     scores = scores.contiguous()
     nb = scores.shape[-1]
     rows = scores.numel() // nb

@@ -353,3 +353,93 @@ def test_compress_windows_match_oracle(b, h, n, d, cbs, st):
     assert_close(got, want, 1.6e-2 * want.abs().max().item(), 1e-2, "windows")
     _grad_close(xg.grad, xr.grad, "d tokens")
     _grad_close(pg.grad, pr.grad, "d positions")
+
+
+def test_topk_long_rows_and_many_selections_bit_exact():
+    """Beyond one kernel call (rows over 2048 entries, more than 64 selections - the reference's topk has no limit): per
+    segment, then among the segments' winners, 64 at a time.  Bit-exact against the stable sort, exact ties included."""
+    from native_sparse_attention_pytorch_amd.ops import importance_topk, topk_op
+    g = torch.Generator().manual_seed(5)
+    for nb, k in [(4096, 16), (5000, 70), (2049, 3), (300, 100), (6000, 64)]:
+        s = torch.rand(2, 1, 20, nb, generator=g)
+        s = (s * 64).round() / 64                                # many exact ties
+        s[0, 0, :3] = 0.0
+        idx, vals, fm = topk_op(s.to(DEV), k, False)
+        wv, wi = O.topk_lower_index_first(s, k)
+        assert torch.equal(idx.cpu().long(), wi), f"indices differ nb={nb} k={k}"
+        assert torch.equal(vals.cpu(), wv) and torch.equal(fm.cpu().bool(), wv > 1e-10)
+    # through the padded softmax: the probabilities are torch's own (same formula as the oracle's, on the device)
+    logits = torch.randn(1, 2, 30, 4096, generator=g) * 3
+    logits[..., :10, 100:] = float("-inf")
+    vals, idx, fm = importance_topk(logits.to(DEV), 16)
+    probs = O.importance_softmax(logits.to(DEV))
+    wv, wi = O.topk_lower_index_first(probs, 16)
+    assert torch.equal(idx.long(), wi) and torch.equal(vals, wv) and torch.equal(fm, wv > 1e-10)
+
+
+def test_select_more_slots_than_one_call_holds():
+    """70 selected blocks (one call of the kernels holds 62): the slots go through in groups merged by their log-sum-exp;
+    outputs, lse and all gradients against the oracle, which has no such limit (NSA.py:741-819)."""
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    b, hq, hk, n, d, B, S = 1, 4, 2, 1400, 64, 16, 70
+    g = torch.Generator().manual_seed(9)
+    q, k, v, do = (_rand((b, h, n, d), g, d ** -0.25) for h in (hq, hk, hk, hq))
+    from tests.util import causal_random_selection
+    idx, msk = causal_random_selection(b, hk, n, B, S, seed=4)
+    qr, kr, vr = (t.float().requires_grad_() for t in (q, k, v))
+    ref, ref_lse = O.select_attend(qr, kr, vr, idx, msk, B, causal=True, return_lse=True)
+    (ref * do.float()).sum().backward()
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    out, lse = native_sparse_attend(qg, kg, vg, B, idx.to(DEV), msk.to(DEV), return_lse=True)
+    (out.float() * do.to(DEV).float()).sum().backward()
+    torch.cuda.synchronize()
+    assert_close(out, ref, 2e-2, 1e-2, "out")
+    assert_close(lse, ref_lse, 2e-2, 1e-2, "lse")
+    _grad_close(qg.grad, qr.grad, "dq")
+    _grad_close(kg.grad, kr.grad, "dk")
+    _grad_close(vg.grad, vr.grad, "dv")
+
+
+def test_select_lse_output_carries_gradient():
+    """The returned log-sum-exp is differentiable (the merge of slot groups relies on it): a loss on lse alone."""
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    from tests.util import causal_random_selection
+    b, hq, hk, n, d, B, S = 1, 4, 2, 300, 64, 16, 3
+    g = torch.Generator().manual_seed(13)
+    q, k, v = (_rand((b, h, n, d), g, d ** -0.25) for h in (hq, hk, hk))
+    w = torch.randn(b, hq, n, generator=g)
+    idx, msk = causal_random_selection(b, hk, n, B, S, seed=6)
+    qr, kr, vr = (t.float().requires_grad_() for t in (q, k, v))
+    _, ref_lse = O.select_attend(qr, kr, vr, idx, msk, B, causal=True, return_lse=True)
+    (ref_lse * w).sum().backward()
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    _, lse = native_sparse_attend(qg, kg, vg, B, idx.to(DEV), msk.to(DEV), return_lse=True)
+    (lse * w.to(DEV)).sum().backward()
+    torch.cuda.synchronize()
+    _grad_close(qg.grad, qr.grad, "dq from lse")
+    _grad_close(kg.grad, kr.grad, "dk from lse")
+    assert vg.grad is None or float(vg.grad.abs().max()) == 0.0
+
+
+def test_batch_times_heads_beyond_one_grid():
+    """batch * kv heads over 65535 (a grid dimension): the functional entry points cut the batch; every piece equals the same
+    rows computed alone."""
+    from native_sparse_attention_pytorch_amd import native_sparse_attend
+    from native_sparse_attention_pytorch_amd.ops import sliding_attend, compress_attend
+    from tests.util import causal_random_selection
+    b, hq, hk, n, d, B, S = 66000, 1, 1, 48, 64, 16, 2
+    g = torch.Generator().manual_seed(1)
+    q = (torch.randn(b, hq, n, d, generator=g) * d ** -0.25).to(torch.bfloat16).to(DEV)
+    k, v = q.roll(1, 0), q.roll(2, 0)
+    idx, msk = causal_random_selection(1, hk, n, B, S, seed=2)
+    idx, msk = idx.expand(b, -1, -1, -1).contiguous().to(DEV), msk.expand(b, -1, -1, -1).contiguous().to(DEV)
+    tail = slice(b - 300, b)
+    out = native_sparse_attend(q, k, v, B, idx, msk)
+    assert torch.equal(out[tail], native_sparse_attend(q[tail], k[tail], v[tail], B, idx[tail], msk[tail]))
+    assert torch.equal(out[:100], native_sparse_attend(q[:100], k[:100], v[:100], B, idx[:100], msk[:100]))
+    s_out = sliding_attend(q, k, v, 8, causal=True)
+    assert torch.equal(s_out[tail], sliding_attend(q[tail], k[tail], v[tail], 8, causal=True))
+    ck = k[:, :, :13].contiguous()
+    c_out, imp = compress_attend(q, ck, ck, 1, 4, True, sel_block=16, share=True)
+    c2, imp2 = compress_attend(q[tail], ck[tail], ck[tail], 1, 4, True, sel_block=16, share=True)
+    assert torch.equal(c_out[tail], c2) and torch.equal(imp[tail], imp2)
