@@ -395,6 +395,31 @@ def main():
         tt = (time.perf_counter() - t0) / 10
         res["train_config5"] = dict(ms_per_step=round(tt * 1e3, 3), tokens_per_s=round(8 * 1024 / tt, 1), loss_after=round(last.item(), 4))
         del model, opt
+        # the same step with the model in bf16 and the optimizer on fp32 master weights (no per-layer casts: the step is bound by
+        # its kernel launches)
+        from native_sparse_attention_pytorch_amd.training import Fp32Masters
+        torch.manual_seed(0)
+        model = Transformer(num_tokens=256, dim=512, depth=6, dim_head=64, heads=8, kv_heads=4,
+                            sparse_attn_kwargs=dict(sliding_window_size=64, compress_block_size=16, compress_block_sliding_stride=8,
+                                                    selection_block_size=16, num_selected_blocks=4)).to(dev)
+        mw = Fp32Masters(model)
+        opt = torch.optim.Adam(mw.masters, lr=1e-4)
+
+        def master_step():
+            loss = model(ids, return_loss=True)
+            loss.backward()
+            mw.step(opt)
+            return loss
+        for _ in range(3):
+            master_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            last = master_step()
+        torch.cuda.synchronize()
+        tt = (time.perf_counter() - t0) / 10
+        res["train_config5"]["fp32_masters"] = dict(ms_per_step=round(tt * 1e3, 3), tokens_per_s=round(8 * 1024 / tt, 1), loss_after=round(last.item(), 4))
+        del model, opt, mw
     except _Skip:
         pass
     except Exception as ex:

@@ -94,6 +94,40 @@ def _ws_sizes(dsc) -> tuple[int, int, int]:
     return a.value, f.value, w.value
 
 
+# A registered operator call costs about 70 us of host time here (dispatcher, schema checks, autograd wrapper), an
+# autograd.Function call a fraction of that; at small shapes a layer's step is bound by exactly that cost.  Outside a
+# compiler trace the attention operators therefore run as plain autograd.Functions around the same Python bodies; the
+# torch.library registrations (with their fake and autograd rules) serve traced callers.
+def _direct(op):
+    """The Python body of a registered operator, unless a compiler is tracing (then the operator itself)."""
+    return op if torch.compiler.is_compiling() else op._init_fn
+
+
+def _eager_function(op, setup, backward):
+    raw = op._init_fn
+
+    class Fn(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, *args):
+            out = raw(*args)
+            setup(ctx, args, out)
+            return out
+
+        @staticmethod
+        def backward(ctx, *grads):
+            return backward(ctx, *grads)
+
+    Fn.__name__ = Fn.__qualname__ = "Eager_" + getattr(op, "_name", "op")
+
+    def call(*args):
+        if torch.compiler.is_compiling():
+            return op(*args)
+        if not torch.is_grad_enabled() or not any(isinstance(a, Tensor) and a.requires_grad for a in args):
+            return raw(*args)
+        return Fn.apply(*args)
+    return call
+
+
 # ------------------------------------------------------------------------------- selection
 
 @torch.library.custom_op("nsa_amd::select_fwd", mutates_args=())
@@ -182,11 +216,12 @@ def _select_backward(ctx, dout, dlse, dws):
         return (None,) * 9
     if dout is None:
         dout = torch.zeros_like(out)
-    dq, dk, dv, dsel = select_bwd(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale, want, dlse)
+    dq, dk, dv, dsel = _direct(select_bwd)(q, k, v, out, dout, lse, idx, fmask, index_ws, block, causal, scale, want, dlse)
     return dq, dk, dv, None, None, (dsel.to(sdtype) if want else None), None, None, None
 
 
 select_fwd.register_autograd(_select_backward, setup_context=_select_setup)
+_select_fwd = _eager_function(select_fwd, _select_setup, _select_backward)
 
 
 def _split_blocks(idx: Tensor, fmask: Tensor, sel_scale: Tensor | None, block: int, n: int, causal: bool):
@@ -257,12 +292,12 @@ def _select_core(q: Tensor, k: Tensor, v: Tensor, idx: Tensor, fm: Tensor, sc: T
         return torch.cat([o for o, _ in outs], dim=0), torch.cat([l for _, l in outs], dim=0)
     S = idx.shape[-1]
     if S <= _MAX_SLOTS:
-        out, lse, _ = select_fwd(q, k, v, idx, fm, sc, block, causal, scale)
+        out, lse, _ = _select_fwd(q, k, v, idx, fm, sc, block, causal, scale)
         return out, lse
     outs, lses = [], []
     for g0 in range(0, S, _MAX_SLOTS):
         sl = slice(g0, min(S, g0 + _MAX_SLOTS))
-        o, l, _ = select_fwd(q, k, v, idx[..., sl].contiguous(), fm[..., sl].contiguous(), None if sc is None else sc[..., sl].contiguous(),
+        o, l, _ = _select_fwd(q, k, v, idx[..., sl].contiguous(), fm[..., sl].contiguous(), None if sc is None else sc[..., sl].contiguous(),
                              block, causal and g0 == 0, scale)
         outs.append(o.float())
         lses.append(l)
@@ -444,8 +479,8 @@ def _dense_backward(ctx, dout, dlse, dpooled):
         # the compressed keys are few and every one of their gradients is summed over all windows into the compression
         # network's parameters: they leave the kernel as fp32 and are rounded to the keys' dtype once, after the
         # importance term has been added
-        dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale,
-                               mode == 1 and dpooled is not None and dpooled.numel() > 0)
+        dq, dk, dv = _direct(dense_bwd)(q, k, v, out, dout, lse, mode, causal, window, stride, num_mem, scale,
+                                        mode == 1 and dpooled is not None and dpooled.numel() > 0)
     if dpooled is not None and dpooled.numel() > 0:
         dq2, dk2 = _importance_backward(q, k, dpooled, num_mem, stride, sel_block, share, scale)
         dq = dq2.to(q.dtype) if dq is None else (dq.float() + dq2).to(q.dtype)
@@ -456,6 +491,7 @@ def _dense_backward(ctx, dout, dlse, dpooled):
 
 
 dense_fwd.register_autograd(_dense_backward, setup_context=_dense_setup)
+_dense_fwd = _eager_function(dense_fwd, _dense_setup, _dense_backward)
 
 
 def sliding_attend(q: Tensor, k: Tensor, v: Tensor, window_size: int, causal: bool = True) -> Tensor:
@@ -468,7 +504,7 @@ def sliding_attend(q: Tensor, k: Tensor, v: Tensor, window_size: int, causal: bo
     d = q.shape[-1]
     D = _kernel_dim(d)
     qp, g, gp = _pad_groups(_pad_dim(q, D), k.shape[1])
-    out, _, _ = dense_fwd(qp, _pad_dim(k, D), _pad_dim(v, D), 0, bool(causal), int(window_size), 1, 0, 0, 1, True, float(d ** -0.5))
+    out, _, _ = _dense_fwd(qp, _pad_dim(k, D), _pad_dim(v, D), 0, bool(causal), int(window_size), 1, 0, 0, 1, True, float(d ** -0.5))
     return _unpad_groups(out, k.shape[1], g, gp)[..., :d]
 
 
@@ -508,7 +544,7 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
         # the reference's own inference test) take the per-key logits from the kernel (a "block" of one key: head mean and
         # visibility as usual) and finish NSA.py:676-689 with three elementwise ops: mean over the block's keys (-inf as
         # soon as one key is invisible), own block masked.
-        out, _, per_key = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), 1, int(stride), bool(share), scale)
+        out, _, per_key = _dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), 1, int(stride), bool(share), scale)
         out = _unpad_groups(out, hk, g, gp)[..., :d]
         n, nb = q.shape[2], per_key.shape[-1] // npf
         if nb == 0:
@@ -518,8 +554,8 @@ def compress_attend(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride: int
         imp = imp.masked_fill(own, float("-inf"))
         return (out, imp, None) if prefix_only else (out, imp)
     use_prefix = bool(prefix_only and pool and causal and g == gp)
-    out, _, pooled = dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), (2 if use_prefix else 1) if pool else 0,
-                               int(sel_block or stride), bool(share), scale)
+    out, _, pooled = _dense_fwd(q, ck, cv, 1, bool(causal), 0, int(stride), int(num_mem), (2 if use_prefix else 1) if pool else 0,
+                                int(sel_block or stride), bool(share), scale)
     out = _unpad_groups(out, hk, g, gp)[..., :d]
     imp = logits_of(pooled) if pool and pooled.shape[-1] > 0 else None
     if not prefix_only:
@@ -567,11 +603,12 @@ def _compress_topk_backward(ctx, dout, dlse, didx, dfm):
     causal, stride, num_mem, scale = ctx.args
     if dout is None:
         return (None,) * 9
-    dq, dk, dv = dense_bwd(q, k, v, out, dout, lse, 1, causal, 0, stride, num_mem, scale, False)
+    dq, dk, dv = _direct(dense_bwd)(q, k, v, out, dout, lse, 1, causal, 0, stride, num_mem, scale, False)
     return (dq, dk, dv) + (None,) * 6
 
 
 compress_topk_fwd.register_autograd(_compress_topk_backward, setup_context=_compress_topk_setup)
+_compress_topk_fwd = _eager_function(compress_topk_fwd, _compress_topk_setup, _compress_topk_backward)
 
 
 def compress_topk_supported(q: Tensor, ck: Tensor, num_mem: int, stride: int, sel_block: int, num_selected: int, share: bool) -> bool:
@@ -601,8 +638,8 @@ def compress_attend_topk(q: Tensor, ck: Tensor, cv: Tensor, num_mem: int, stride
     q2, g, gp = _pad_groups(_pad_dim(q, D), hk)
     if g != gp:
         raise RuntimeError("compress_attend_topk: the group size must be a power of two")
-    out, _, idx, fm = compress_topk_fwd(q2, _pad_dim(ck, D), _pad_dim(cv, D), bool(causal), int(stride), int(num_mem), int(sel_block),
-                                        int(num_selected), float(d ** -0.5))
+    out, _, idx, fm = _compress_topk_fwd(q2, _pad_dim(ck, D), _pad_dim(cv, D), bool(causal), int(stride), int(num_mem), int(sel_block),
+                                         int(num_selected), float(d ** -0.5))
     return out[..., :d], idx, fm.view(torch.bool)
 
 
@@ -795,10 +832,11 @@ def _gate_setup(ctx, inputs, output):
 
 def _gate_backward(ctx, dout):
     logits, c, f, s = ctx.saved_tensors
-    return gate_bwd(logits, c, f, s, dout)
+    return _direct(gate_bwd)(logits, c, f, s, dout)
 
 
 gate_fwd.register_autograd(_gate_backward, setup_context=_gate_setup)
+_gate_fwd = _eager_function(gate_fwd, _gate_setup, _gate_backward)
 
 
 def gate_combine(logits: Tensor, compressed: Tensor, selected: Tensor, sliding: Tensor) -> Tensor:
@@ -806,7 +844,7 @@ def gate_combine(logits: Tensor, compressed: Tensor, selected: Tensor, sliding: 
     'b n (h d)' (NSA.py:323-327, 854-860).  logits are the pre-sigmoid gate projection."""
     b, h, n, d = compressed.shape
     D = _kernel_dim(d)
-    out = gate_fwd(logits.to(_BF16), _pad_dim(compressed, D), _pad_dim(selected, D), _pad_dim(sliding, D))
+    out = _gate_fwd(logits.to(_BF16), _pad_dim(compressed, D), _pad_dim(selected, D), _pad_dim(sliding, D))
     return out if D == d else out.reshape(b, n, h, D)[..., :d].reshape(b, n, h * d)
 
 
@@ -1345,7 +1383,9 @@ def qkv_prep(qkv: Tensor, freqs: Tensor, k_positions: Tensor, v_positions: Tenso
 # ------------------------------------------------------------------ norm and column sums
 
 def colsum_supported(x: Tensor) -> bool:
-    return bool(x.is_cuda and x.dtype == _BF16 and x.shape[-1] % 8 == 0 and x.numel() > 0)
+    """One pass + a reduce of per-work-group partials (two launches) pays from about half a million elements on; below that the
+    library's one-launch sum is as fast and a step bound by its launches (a small model) is better off with one launch."""
+    return bool(x.is_cuda and x.dtype == _BF16 and x.shape[-1] % 8 == 0 and x.numel() >= (1 << 19))
 
 
 def colsum(x: Tensor, out_dtype=None) -> Tensor:
@@ -1444,6 +1484,8 @@ def _wgrad_splits(rows: int, n_in: int, n_out: int) -> int:
     per output tile the whole token axis: with a few dozen tiles of a small weight and tens of thousands of tokens most of the
     256 CUs idle (measured on 16384 tokens: 1024 x 1024 weight 109 us whole, 52 us in 8 slices + the sum; 48 x 1024 99 -> 31 us;
     a 2048 x 2048 weight over 4080 tokens has its 256 tiles already and is left whole)."""
+    if rows < 16384:          # the whole GEMM is a few microseconds: a second launch (the sum of the slices) costs more than the slices save
+        return 1
     tiles = -(-n_in // 128) * -(-n_out // 128)
     s = 8
     while s > 1 and (s * tiles > 768 or rows % s or rows // s < 1024):

@@ -66,3 +66,26 @@ def test_train_config5_matches_oracle_fixture():
     print("hip           ", got)
     for a, b in zip(got, fx["losses"]):
         assert abs(a - b) < 2e-3, (got, fx["losses"])
+
+
+def test_train_config5_with_fp32_masters_matches_oracle_fixture():
+    """The same ten steps with the model itself in bf16 and the optimizer on fp32 master weights (training.Fp32Masters)
+    instead of autocast: the same arithmetic without the per-layer casts, the same bound."""
+    from native_sparse_attention_pytorch_amd.transformer import Transformer
+    from native_sparse_attention_pytorch_amd.training import Fp32Masters
+    fx = json.load(open(os.path.join(HERE, "golden", "train_cfg5_oracle_losses.json")))
+    ids = torch.randint(0, 256, (fx["batch"], fx["seq"] + 1), generator=torch.Generator().manual_seed(fx["seed"] + 1)).to(DEV)
+    torch.manual_seed(fx["seed"])
+    model = Transformer(**fx["config"]).to(DEV)
+    mw = Fp32Masters(model)
+    opt = torch.optim.Adam(mw.masters, lr=fx["lr"])
+    got = []
+    for _ in range(fx["steps"]):
+        loss = model(ids, return_loss=True)
+        loss.backward()
+        mw.step(opt)
+        got.append(loss.item())
+    print("oracle fixture", fx["losses"])
+    print("hip, masters  ", got)
+    for a, b in zip(got, fx["losses"]):
+        assert abs(a - b) < 2e-3, (got, fx["losses"])
