@@ -63,6 +63,17 @@ def selection(b, h, n, B, S, seed, device):
     return idx.masked_fill(~mask, 0).contiguous(), mask.contiguous()
 
 
+def ceiling_bytes(cfg):
+    """HBM bytes per step that the block-major walk cannot avoid: per live (query, kv head, slot) pair G*d bf16 of Q (forward)
+    and of Q and dO (backward), one G*d bf16 partial written and read again in each direction; plus every tensor once."""
+    b, n, hq, hk, d, B, S = cfg["batch"], cfg["seq"], cfg["heads"], cfg["kv_heads"], cfg["dim_head"], cfg["block"], cfg["num_sel"]
+    W = math.ceil(n / B)
+    pairs = b * hk * sum(B * (min(w, S) + 1) for w in range(W))
+    row = (hq // hk) * d * 2
+    once = (4 * b * hq * n * d + 6 * b * hk * n * d) * 2            # q, out, dO, dq; k, v, dk, dv (k, v read twice)
+    return pairs * row * 7 + once
+
+
 def attended_pairs(b, hq, n, B, s_total):
     W = math.ceil(n / B)
     return b * hq * sum(B * (min(w, s_total - 1) * B + (B + 1) / 2) for w in range(W))
@@ -211,6 +222,11 @@ def main():
     roofline = dict(bound="mfma", kernel=dom, achieved=round(achieved, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
                     frac=round(achieved / MFMA_PEAK_TFLOPS, 4), traffic=traffic,
                     step_frac=round(value / MFMA_PEAK_TFLOPS, 4),
+                    # what this selection law allows at any kernel quality: a (query, block) pair's partial results must cross
+                    # HBM (2 KB written + 2 KB read per pair, forward and backward together) and its Q / dO rows be gathered
+                    # (3 KB); at the rate the memory system gives that access pattern (measured by the rowtraffic leg: ~5.3 TB/s
+                    # mixed gather / scatter, ~6 TB/s streams) the step cannot be shorter than those bytes take
+                    ceiling_frac=round(total_flop / (ceiling_bytes(cfg) / 5.5e12) / 1e12 / MFMA_PEAK_TFLOPS, 4),
                     # the kernels are HBM-bound in practice: measured bytes / measured time against 8 TB/s
                     hbm_GBs={nm: round(traffic_all[nm] / (kern[nm] * 1e-3) / 1e9, 1) for nm in traffic_all},
                     hbm_frac_step=round(sum(traffic_all.values()) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if traffic_all else None,
@@ -462,7 +478,9 @@ def main():
         probe = {}
         for name, sr, rd, wr in (("gather_hbm", rows_big, 2, 0), ("scatter_hbm", rows_big, 0, 2), ("gather1_scatter1_hbm", rows_big, 1, 1),
                                  ("gather2_scatter1_hbm", rows_big, 2, 1), ("gather1_scatter2_hbm", rows_big, 1, 2),
-                                 ("gather_l2_scatter_hbm", 2048, 1, 1)):
+                                 ("gather_l2_scatter_hbm", 2048, 1, 1),
+                                 # a gather set that fits the 256 MB memory-side cache (the Q and dO rows of one kv head at 32k: 134 MB)
+                                 ("gather2_128MB_scatter1_hbm", (128 << 20) // 1024, 2, 1), ("gather_128MB", (128 << 20) // 1024, 2, 0)):
             best = None
             for rep in range(4):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
