@@ -10,6 +10,13 @@
 #define NSA_PHASE_BYTES (1L << 22)
 #endif
 
+#ifndef NSA_DKV_UNITS_WANTED
+#define NSA_DKV_UNITS_WANTED 4096
+#endif
+#ifndef NSA_DKV_CHUNK_FIXED
+#define NSA_DKV_CHUNK_FIXED 0      // a power of two to override the choice (experiments)
+#endif
+
 namespace nsa {
 
 struct SelPlan {
@@ -71,7 +78,15 @@ static inline int make_plan(const nsa_select_desc* d, SelPlan& P) {
   while (ph * 2 * row_bytes <= (long)NSA_PHASE_BYTES && ph < (1L << 20)) ph *= 2;
   P.chunk[0] = 256;  P.phase[0] = (int)ph;
   P.chunk[1] = 256;  P.phase[1] = (int)(ph > 256 ? ph / 2 : ph);
-  P.chunk[2] = 1024; P.phase[2] = ((P.n + 255) / 256) * 256;
+  // dK/dV walk: a unit keeps its accumulators for `chunk` pairs and leaves a 2 x 32KT x D fp32 partial behind, so long units
+  // are cheaper per pair - but the chip holds 512 to 1024 work-groups of this kernel at a time, and a launch with fewer
+  // units than a few rounds of that runs as long as its longest units whatever the rest does (seq 8k, 4 kv heads: 512 units
+  // of 1024 pairs occupy half of the SIMDs for the whole launch).  Shorter units when the launch would have under ~4096.
+  {
+    const long want = bh * pairs / NSA_DKV_UNITS_WANTED;
+    P.chunk[2] = NSA_DKV_CHUNK_FIXED ? NSA_DKV_CHUNK_FIXED : (want >= 1024 ? 1024 : want >= 512 ? 512 : 256);
+  }
+  P.phase[2] = ((P.n + 255) / 256) * 256;
   for (int t = 0; t < 3; ++t) {
     P.np[t] = (P.n + P.phase[t] - 1) / P.phase[t];
     const long cells = (long)P.np[t] * P.W;
