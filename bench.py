@@ -63,15 +63,16 @@ def selection(b, h, n, B, S, seed, device):
     return idx.masked_fill(~mask, 0).contiguous(), mask.contiguous()
 
 
-def ceiling_bytes(cfg):
+def ceiling_bytes(cfg, rows_per_pair=7):
     """HBM bytes per step that the block-major walk cannot avoid: per live (query, kv head, slot) pair G*d bf16 of Q (forward)
-    and of Q and dO (backward), one G*d bf16 partial written and read again in each direction; plus every tensor once."""
+    and of Q and dO (backward), one G*d bf16 partial written and read again in each direction (7 rows); plus every tensor
+    once.  rows_per_pair=4 counts the partial exchange alone (as if every gather hit a cache)."""
     b, n, hq, hk, d, B, S = cfg["batch"], cfg["seq"], cfg["heads"], cfg["kv_heads"], cfg["dim_head"], cfg["block"], cfg["num_sel"]
     W = math.ceil(n / B)
     pairs = b * hk * sum(B * (min(w, S) + 1) for w in range(W))
     row = (hq // hk) * d * 2
     once = (4 * b * hq * n * d + 6 * b * hk * n * d) * 2            # q, out, dO, dq; k, v, dk, dv (k, v read twice)
-    return pairs * row * 7 + once
+    return pairs * row * rows_per_pair + once
 
 
 def attended_pairs(b, hq, n, B, s_total):
@@ -227,6 +228,8 @@ def main():
                     # (3 KB); at the rate the memory system gives that access pattern (measured by the rowtraffic leg: ~5.3 TB/s
                     # mixed gather / scatter, ~6 TB/s streams) the step cannot be shorter than those bytes take
                     ceiling_frac=round(total_flop / (ceiling_bytes(cfg) / 5.5e12) / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                    # the same with the exchange of partials alone (4 KB per pair at the 6 TB/s of plain streams)
+                    ceiling_exchange_only_frac=round(total_flop / (ceiling_bytes(cfg, 4) / 6.0e12) / 1e12 / MFMA_PEAK_TFLOPS, 4),
                     # the kernels are HBM-bound in practice: measured bytes / measured time against 8 TB/s
                     hbm_GBs={nm: round(traffic_all[nm] / (kern[nm] * 1e-3) / 1e9, 1) for nm in traffic_all},
                     hbm_frac_step=round(sum(traffic_all.values()) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if traffic_all else None,
@@ -273,8 +276,10 @@ def main():
         ck = (torch.randn(b, hk, nc + 1, d, generator=g2, device=dev) * d ** -0.5).to(torch.bfloat16).requires_grad_()
         cv = (torch.randn(b, hk, nc + 1, d, generator=g2, device=dev) * d ** -0.5).to(torch.bfloat16).requires_grad_()
         qc = q.clone().requires_grad_()
-        tms = []
-        for it in range(3):
+        # six rounds queued without a host synchronisation in between (HIP events bracket each call; with a
+        # synchronisation per round the first call of a round also times the host's allocations), the first two discarded
+        evs_c = []
+        for it in range(6):
             qc.grad = ck.grad = cv.grad = None      # a step's gradients start from None (no accumulation pass in the timing)
             e0, e1, e2, e3, e4 = (torch.cuda.Event(enable_timing=True) for _ in range(5))
             e0.record()
@@ -289,10 +294,11 @@ def main():
                 e3.record()
                 ops.importance_topk(imp, S + 1, prefix=prefix)
                 e4.record()
-            torch.cuda.synchronize()
-            tms.append((e0.elapsed_time(e1), e1.elapsed_time(e2), e2.elapsed_time(e3), e3.elapsed_time(e4)))
+            evs_c.append((e0, e1, e2, e3, e4))
+        torch.cuda.synchronize()
+        tms = [tuple(e[i].elapsed_time(e[i + 1]) for i in range(4)) for e in evs_c]
         p_cmp = b * hq * sum(i // 16 + 1 for i in range(n))
-        best = min(tms[1:], key=lambda t: t[0] + t[1])
+        best = min(tms[2:], key=lambda t: t[0] + t[1])
         cf, cb = 4 * d * p_cmp / (best[0] * 1e-3) / 1e12, 10 * d * p_cmp / (best[1] * 1e-3) / 1e12
         res["compressed_branch"] = dict(fwd_with_selection_ms=round(best[0], 4), bwd_ms=round(best[1], 4),
                                         attended_pairs=p_cmp, fwd_bwd_tflops=round(14 * d * p_cmp / ((best[0] + best[1]) * 1e-3) / 1e12, 2),

@@ -1,8 +1,10 @@
 /* C ABI of libnsa_hip.so - the gfx950 (MI355X) kernels for the Native Sparse Attention hot path.
  *
  * Every function is enqueue-only on the given hipStream_t (passed as void*), never allocates or
- * frees device memory, never synchronises and keeps no global state.  The caller owns every
- * buffer, including workspaces, whose sizes come from the *_workspace_bytes functions.
+ * frees device memory and never synchronises.  The caller owns every buffer, including
+ * workspaces, whose sizes come from the *_workspace_bytes functions.  The library keeps no state
+ * between calls, with one exception: nsa_decode_attend_noalloc caches, per device, the address of
+ * its fixed scratch array (looked up on the first call on that device, under a mutex).
  * Return value: 0 = ok, negative = argument error (NSA_E_*), positive = hipError_t of a launch.
  *
  * Citations are into the reference tree (lucidrains/native-sparse-attention-pytorch v0.2.3):
