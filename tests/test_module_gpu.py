@@ -156,8 +156,9 @@ def test_module_matches_oracle(ci, n):
             # of a sum over all keys that otherwise cancels (its norm is ~1/20 of the sibling weight's).  Any flash-style
             # backward in bf16 leaves two errors in it that do not cancel: delta = sum(out * d_out) from the rounded
             # forward output (TRI.py:696-756 does the same) and the bf16 dS operand of dK = dS^T Q; emulated on the CPU
-            # each alone is 0.025-0.03 of this gradient.  The causal configurations are held to the bound above.
-            bound = 1e-1
+            # each alone is 0.025-0.03 of this gradient.  Measured over the non-causal configurations of this test: 0.025,
+            # 0.034, 0.039 and 0.067.  The causal configurations are held to the bound above.
+            bound = 8e-2
             print(f"non-causal {name}: rel err {e:.4f} against the fp32 oracle (bf16 torch path: {e16:.4f}), bound {bound}", flush=True)
         assert e < bound, f"grad of {name}: rel err {e:.4f} (bf16 torch path: {e16:.4f})"
 
