@@ -128,6 +128,37 @@ class _Skip(Exception):
     """Raised inside an optional leg that --headline-only turns off."""
 
 
+def graphed_train_leg():
+    """BASELINE configs[4] training step with forward + backward replayed from one HIP graph (training.GraphedStep) on a bf16
+    model, Adam on fp32 master weights outside the graph.  Runs in a process of its own (see main): prints one JSON object."""
+    import torch
+    from native_sparse_attention_pytorch_amd.transformer import Transformer
+    from native_sparse_attention_pytorch_amd.training import Fp32Masters, GraphedStep
+    dev = "cuda"
+    torch.manual_seed(0)
+    model = Transformer(num_tokens=256, dim=512, depth=6, dim_head=64, heads=8, kv_heads=4,
+                        sparse_attn_kwargs=dict(sliding_window_size=64, compress_block_size=16, compress_block_sliding_stride=8,
+                                                selection_block_size=16, num_selected_blocks=4)).to(dev)
+    ids = torch.randint(0, 256, (8, 1025), device=dev)
+    mw = Fp32Masters(model)
+    opt = torch.optim.Adam(mw.masters, lr=1e-4)
+    gstep = GraphedStep(model, ids)
+
+    def step():
+        loss = gstep(ids)
+        mw.step(opt)
+        return loss
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        last = step()
+    torch.cuda.synchronize()
+    tt = (time.perf_counter() - t0) / 10
+    print(json.dumps(dict(ms_per_step=round(tt * 1e3, 3), tokens_per_s=round(8 * 1024 / tt, 1), loss_after=round(last.item(), 4))), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -136,7 +167,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="only the headline workload (for profiler runs): no compressed-branch, module or decode legs")
     ap.add_argument("--skip", default="", help="comma-separated legs to leave out: select_config2, rowtraffic, compressed, module, decode, train, generate")
+    ap.add_argument("--child-leg", default="", help=argparse.SUPPRESS)
     args = ap.parse_args()
+    if args.child_leg == "graphtrain":
+        graphed_train_leg()
+        return
     skip = set(filter(None, args.skip.split(","))) | ({"select_config2", "rowtraffic", "compressed", "module", "decode", "train", "generate"} if args.headline_only else set())
 
     def leg(name):
@@ -148,6 +183,20 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
         sys.exit(2)
+    # The graph-replayed training step runs first, in a child process started before this process touches the GPU: a
+    # recording that goes wrong ends its process, and that must not take the headline with it.  Not under a profiler
+    # (its preloaded library has the GPU initialised already, and a process in that state must not start another program).
+    graphed_train = None
+    profiled = any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ) or "rocprof" in os.environ.get("LD_PRELOAD", "")
+    if "train" not in skip and not profiled:
+        print("bench.py: graph-replayed train leg (child process)", file=sys.stderr, flush=True)
+        try:
+            import subprocess
+            cp = subprocess.run([sys.executable, os.path.abspath(__file__), "--child-leg", "graphtrain"], capture_output=True, text=True, timeout=600)
+            lines = [ln for ln in cp.stdout.strip().splitlines() if ln.startswith("{")]
+            graphed_train = json.loads(lines[-1]) if cp.returncode == 0 and lines else dict(error=f"child exited with {cp.returncode}")
+        except Exception as ex:
+            graphed_train = dict(error=repr(ex))
     if not torch.cuda.is_available():
         print("bench.py needs an MI355X (no CPU fallback for the product path)", file=sys.stderr)
         sys.exit(2)
@@ -441,6 +490,8 @@ def main():
         torch.cuda.synchronize()
         tt = (time.perf_counter() - t0) / 10
         res["train_config5"]["fp32_masters"] = dict(ms_per_step=round(tt * 1e3, 3), tokens_per_s=round(8 * 1024 / tt, 1), loss_after=round(last.item(), 4))
+        if graphed_train is not None:
+            res["train_config5"]["graphed_fp32_masters"] = graphed_train
         del model, opt, mw
     except _Skip:
         pass

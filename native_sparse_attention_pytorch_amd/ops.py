@@ -1382,10 +1382,17 @@ def qkv_prep(qkv: Tensor, freqs: Tensor, k_positions: Tensor, v_positions: Tenso
 
 # ------------------------------------------------------------------ norm and column sums
 
+def capturing() -> bool:
+    """A HIP graph is being recorded on the current stream."""
+    return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+
+
 def colsum_supported(x: Tensor) -> bool:
     """One pass + a reduce of per-work-group partials (two launches) pays from about half a million elements on; below that the
-    library's one-launch sum is as fast and a step bound by its launches (a small model) is better off with one launch."""
-    return bool(x.is_cuda and x.dtype == _BF16 and x.shape[-1] % 8 == 0 and x.numel() >= (1 << 19))
+    library's one-launch sum is as fast and a step bound by its launches (a small model) is better off with one launch.
+    While a graph is being recorded every size takes the kernel: the library's sum over many work-groups records a memset
+    node, and on replays after the first its results were wrong here (bias gradients of 1e37 in a replayed training step)."""
+    return bool(x.is_cuda and x.dtype == _BF16 and x.shape[-1] % 8 == 0 and x.numel() > 0 and (x.numel() >= (1 << 19) or capturing()))
 
 
 def colsum(x: Tensor, out_dtype=None) -> Tensor:

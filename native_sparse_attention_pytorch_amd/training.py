@@ -7,6 +7,9 @@ Here the model itself is bf16 (no casts inside the step) and the optimizer works
 one multi-tensor copy takes the bf16 gradients to the masters, one takes the updated masters back.  The arithmetic is
 the same as under autocast - bf16 operands rounded from fp32 masters, fp32 accumulation, fp32 update - and the loss
 curve agrees with the fp32 oracle as closely.
+
+`GraphedStep` goes one further for fixed shapes: the forward and backward of the bf16 model are recorded once into a HIP
+graph and replayed per step (one launch instead of ~700); the optimizer stays outside the graph.
 """
 from __future__ import annotations
 
@@ -38,3 +41,63 @@ class Fp32Masters:
         torch._foreach_copy_(self.params, self.masters)
         for p in self.params:
             p.grad = None
+
+
+class GraphedStep:
+    """Forward + backward of `model(ids, return_loss=True)` as one replayed HIP graph, for a bf16 model (e.g. under
+    `Fp32Masters`) and inputs of one fixed shape.
+
+        step = GraphedStep(model, example_ids)
+        loss = step(ids)            # gradients are in p.grad of the model's parameters afterwards
+        masters.step(optimizer)     # or optimizer.step() on the model's own parameters
+
+    The graph holds no memset node of a library reduction (their replays gave wrong bias gradients on this platform):
+    while it is recorded every bias gradient is a column sum by this library's kernel (ops.colsum_supported) and the
+    feed-forward projections go through ops.linear (Transformer._feed_forward).  The gradient tensors are the graph's own:
+    every call re-attaches them to the parameters (an optimizer helper may have set `p.grad = None`) and every replay
+    overwrites them, so gradients do not accumulate across calls.  `loss` is a tensor that the next call overwrites.
+    Create it before the model's first normally launched training step (a `Transformer` that has been stepped is refused:
+    recording one ended the process here); replays and launched steps may be mixed freely afterwards."""
+
+    def __init__(self, model: nn.Module, example_ids: torch.Tensor, warmup: int = 3):
+        if not example_ids.is_cuda:
+            raise RuntimeError("GraphedStep needs device tensors")
+        if getattr(model, "_launched_grad_steps", False):
+            # recording after normally launched training steps of the same model ended the process (segmentation fault inside
+            # the recording) on this platform, with backward() and with autograd.grad() alike; a model that has not been
+            # stepped yet records and replays correctly, also next to other models trained in the same process
+            raise RuntimeError("GraphedStep must be created before the model's first normally launched training step "
+                               "(build the model, then GraphedStep, then train through it)")
+        self.model = model
+        self.params = [p for p in model.parameters()]
+        self.ids = example_ids.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        # torch.autograd.grad, not backward(): the gradients come back as the recording's own tensors instead of passing
+        # through the parameters' gradient accumulator nodes (which belong to the stream that created them)
+        wanted = [p for p in self.params if p.requires_grad]
+        model._recording_warmup = True
+        try:
+            with torch.cuda.stream(side):                # allocator and library warm-up outside the recording
+                for _ in range(max(1, warmup)):
+                    torch.autograd.grad(model(self.ids, return_loss=True), wanted, allow_unused=True)
+        finally:
+            model._recording_warmup = False
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            loss = model(self.ids, return_loss=True)
+            grads = torch.autograd.grad(loss, wanted, allow_unused=True)
+            self.loss = loss.detach()
+        by_param = dict(zip(map(id, wanted), grads))
+        self.grads = [by_param.get(id(p)) for p in self.params]
+
+    def __call__(self, ids: torch.Tensor) -> torch.Tensor:
+        if ids.shape != self.ids.shape or ids.dtype != self.ids.dtype:
+            raise RuntimeError(f"GraphedStep was recorded for ids of shape {tuple(self.ids.shape)}, got {tuple(ids.shape)}")
+        for p, g in zip(self.params, self.grads):
+            p.grad = g
+        self.ids.copy_(ids)
+        self.graph.replay()
+        return self.loss

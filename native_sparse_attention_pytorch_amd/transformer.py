@@ -43,9 +43,27 @@ class Transformer(nn.Module):
         self.norm = nn.RMSNorm(dim)
         self.to_logits = nn.Linear(dim, num_tokens, bias=False)
 
+    @staticmethod
+    def _feed_forward(ff, tokens):
+        """The feed-forward block (transformer.py:142-152 of the reference: norm, linear, GELU, linear).  While a HIP graph is
+        being recorded (training.GraphedStep) the two projections go through ops.linear, whose bias gradients are column sums
+        by this library's kernel: the library's own sum records a memset node that replays wrongly on this platform."""
+        from . import ops
+        if not (ops.capturing() and torch.is_grad_enabled() and tokens.dtype == torch.bfloat16 and isinstance(ff, nn.Sequential) and len(ff) == 4):
+            return ff(tokens)
+        norm, up, act, down = ff
+        plain = SparseAttention._plain
+        if not (plain(ff, nn.Sequential) and plain(norm, nn.RMSNorm) and plain(up, nn.Linear) and plain(act, nn.GELU) and plain(down, nn.Linear)):
+            return ff(tokens)
+        return ops.linear(act(ops.linear(norm(tokens), up.weight, up.bias)), down.weight, down.bias)
+
     def forward(self, ids, return_loss=False, disable_flex=False, disable_triton_kernel=False, cache=None, return_cache=False):
         if return_loss:
             ids, labels = ids[:, :-1], ids[:, 1:]
+        if torch.is_grad_enabled() and ids.is_cuda and not getattr(self, "_recording_warmup", False):
+            from . import ops
+            if not ops.capturing():
+                self._launched_grad_steps = True      # training.GraphedStep must be recorded before the first of these
         # with caches only the newest token is embedded and every layer takes one decode step
         tokens = self.token_emb(ids if cache is None else ids[:, -1:])
         layer_caches = iter(cache or [])
@@ -57,7 +75,7 @@ class Transformer(nn.Module):
                 attn_out, layer_cache = attn(tokens), None
             caches.append(layer_cache)
             tokens = attn_out + tokens
-            tokens = ff(tokens) + tokens
+            tokens = self._feed_forward(ff, tokens) + tokens
         logits = self.to_logits(self.norm(tokens))
         if not return_loss:
             return (logits, caches) if return_cache else logits

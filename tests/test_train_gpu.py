@@ -89,3 +89,79 @@ def test_train_config5_with_fp32_masters_matches_oracle_fixture():
     print("hip, masters  ", got)
     for a, b in zip(got, fx["losses"]):
         assert abs(a - b) < 2e-3, (got, fx["losses"])
+
+
+def _small_model():
+    from native_sparse_attention_pytorch_amd.transformer import Transformer
+    torch.manual_seed(5)
+    return Transformer(num_tokens=256, dim=256, depth=3, dim_head=64, heads=4, kv_heads=2,
+                       sparse_attn_kwargs=dict(sliding_window_size=32, compress_block_size=16, compress_block_sliding_stride=8,
+                                               selection_block_size=16, num_selected_blocks=4)).to(DEV)
+
+
+def test_graphed_step_equals_the_launched_step_on_every_replay():
+    """training.GraphedStep: forward + backward replayed from one HIP graph.  Every replay - different tokens each time, the
+    same step launched normally and a synchronisation in between - must give the launched step's loss and gradients.  (A graph
+    that contains the library's multi-block sums gives the first replay right and later ones wrong on this platform: bias
+    gradients of 1e37.  While recording, those sums are this library's kernels instead.)"""
+    from native_sparse_attention_pytorch_amd.training import Fp32Masters, GraphedStep
+    model = _small_model()
+    Fp32Masters(model)                                    # bf16 model
+    params = list(model.parameters())
+    names = [n for n, _ in model.named_parameters()]
+    data = [torch.randint(0, 256, (4, 513), device=DEV, generator=torch.Generator(device=DEV).manual_seed(i)) for i in range(7)]
+    step = GraphedStep(model, data[0])
+    assert sum(g is not None for g in step.grads) >= len(params) - 8
+    for rep, ids in enumerate(data):
+        for p in params:
+            p.grad = None
+        want_loss = model(ids, return_loss=True)
+        want_loss.backward()
+        want = [None if p.grad is None else p.grad.clone() for p in params]
+        torch.cuda.synchronize()
+        loss = step(ids)
+        torch.cuda.synchronize()
+        assert abs(loss.item() - want_loss.item()) < 1e-5, (rep, loss.item(), want_loss.item())
+        for n, p, w in zip(names, params, want):
+            assert (p.grad is None) == (w is None), n
+            if w is not None:
+                assert torch.isfinite(p.grad).all(), f"replay {rep}: non-finite gradient of {n}"
+                err = (p.grad.float() - w.float()).abs().max().item()
+                # identical kernels on identical inputs; only the bias sums take another kernel while recording (fp32 sums of
+                # bf16 values in another order: within one bf16 rounding of the result)
+                tol = 1e-2 * max(w.float().abs().max().item(), 1e-6) if n.endswith("bias") else 0.0
+                assert err <= tol, f"replay {rep}: gradient of {n} differs by {err} (largest entry {w.float().abs().max().item()})"
+
+
+def test_train_config5_graphed_with_fp32_masters_matches_oracle_fixture():
+    """Ten Adam steps with forward + backward replayed from a graph and the optimizer on fp32 masters outside it: the loss
+    sequence of the oracle fixture, to the bound of the launched step."""
+    from native_sparse_attention_pytorch_amd.transformer import Transformer
+    from native_sparse_attention_pytorch_amd.training import Fp32Masters, GraphedStep
+    fx = json.load(open(os.path.join(HERE, "golden", "train_cfg5_oracle_losses.json")))
+    ids = torch.randint(0, 256, (fx["batch"], fx["seq"] + 1), generator=torch.Generator().manual_seed(fx["seed"] + 1)).to(DEV)
+    torch.manual_seed(fx["seed"])
+    model = Transformer(**fx["config"]).to(DEV)
+    mw = Fp32Masters(model)
+    opt = torch.optim.Adam(mw.masters, lr=fx["lr"])
+    step = GraphedStep(model, ids)
+    got = []
+    for _ in range(fx["steps"]):
+        got.append(step(ids).item())
+        mw.step(opt)
+    print("oracle fixture", fx["losses"])
+    print("graphed       ", got)
+    for a, b in zip(got, fx["losses"]):
+        assert abs(a - b) < 2e-3, (got, fx["losses"])
+
+
+def test_graphed_step_refuses_a_model_that_was_already_stepped():
+    """Recording after normally launched training steps of the same model is not supported (it ended the process on this
+    platform); the helper says so instead of starting the recording."""
+    from native_sparse_attention_pytorch_amd.training import Fp32Masters, GraphedStep
+    model = _small_model()
+    Fp32Masters(model)
+    ids = torch.randint(0, 256, (2, 257), device=DEV)
+    model(ids, return_loss=True).backward()
+    with pytest.raises(RuntimeError, match="before the model's first"):
+        GraphedStep(model, ids)
