@@ -118,3 +118,25 @@ def test_fused_selection_refuses_what_it_does_not_serve():
     assert not ops.compress_topk_supported(q, ck2, 1, 4, 16, 17, True)        # more than 16 selections
     assert not ops.compress_topk_supported(q, ck2, 1, 4, 16, 4, False)        # per-head selection
     assert ops.compress_topk_supported(q, ck2, 1, 4, 16, 16, True)
+
+
+def test_fused_selection_backward_equals_the_two_kernel_path():
+    """The output of the fused forward is differentiable like compress_attend's (the selection carries no gradient): same
+    saved output and log-sum-exp, same backward kernels, so the gradients of q and the compressed keys / values are equal bit
+    for bit."""
+    from native_sparse_attention_pytorch_amd import ops
+    b, hq, hk, n, d, st, B, mem, k = 2, 8, 2, 1100, 64, 8, 32, 1, 8
+    g = torch.Generator().manual_seed(21)
+    nc = n // st
+    mk = lambda *s, sc=1.0: (torch.randn(*s, generator=g) * sc).to(torch.bfloat16).to(DEV)
+    q, ck, cv, do = mk(b, hq, n, d, sc=d ** -0.25), mk(b, hk, mem + nc, d, sc=d ** -0.25), mk(b, hk, mem + nc, d), mk(b, hq, n, d)
+    grads = []
+    for fused in (True, False):
+        q1, ck1, cv1 = (t.clone().requires_grad_() for t in (q, ck, cv))
+        out = ops.compress_attend_topk(q1, ck1, cv1, mem, st, True, B, k)[0] if fused else ops.compress_attend(q1, ck1, cv1, mem, st, True, sel_block=B, share=True)[0]
+        out.backward(do)
+        grads.append((q1.grad, ck1.grad, cv1.grad))
+    torch.cuda.synchronize()
+    for name, a, b_ in zip(("dq", "dck", "dcv"), *grads):
+        assert a is not None and torch.isfinite(a).all(), name
+        assert torch.equal(a, b_), f"{name}: {(a.float() - b_.float()).abs().max().item()}"
