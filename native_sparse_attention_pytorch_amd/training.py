@@ -62,6 +62,10 @@ class GraphedStep:
     def __init__(self, model: nn.Module, example_ids: torch.Tensor, warmup: int = 3):
         if not example_ids.is_cuda:
             raise RuntimeError("GraphedStep needs device tensors")
+        if torch.is_autocast_enabled() or any(p.requires_grad and p.is_floating_point() and p.dtype != torch.bfloat16 for p in model.parameters()):
+            # under autocast / with fp32 parameters the projections run through the library's own autograd, whose bias
+            # gradients are the sums that replay wrongly
+            raise RuntimeError("GraphedStep records a bf16 model outside autocast (cast it with Fp32Masters or .bfloat16())")
         if getattr(model, "_launched_grad_steps", False):
             # recording after normally launched training steps of the same model ended the process (segmentation fault inside
             # the recording) on this platform, with backward() and with autograd.grad() alike; a model that has not been

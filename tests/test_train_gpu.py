@@ -165,3 +165,10 @@ def test_graphed_step_refuses_a_model_that_was_already_stepped():
     model(ids, return_loss=True).backward()
     with pytest.raises(RuntimeError, match="before the model's first"):
         GraphedStep(model, ids)
+
+
+def test_graphed_step_refuses_fp32_parameters():
+    from native_sparse_attention_pytorch_amd.training import GraphedStep
+    model = _small_model()                                # fp32 parameters: would train under autocast
+    with pytest.raises(RuntimeError, match="bf16 model"):
+        GraphedStep(model, torch.randint(0, 256, (2, 257), device=DEV))
