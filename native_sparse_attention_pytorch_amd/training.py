@@ -44,8 +44,8 @@ class Fp32Masters:
 
 
 class GraphedStep:
-    """Forward + backward of `model(ids, return_loss=True)` as one replayed HIP graph, for a bf16 model (e.g. under
-    `Fp32Masters`) and inputs of one fixed shape.
+    """Forward + backward of `model(ids, return_loss=True)` (or of `loss_fn(model, ids)`) as one replayed HIP graph, for a
+    bf16 model (e.g. under `Fp32Masters`) and inputs of one fixed shape.
 
         step = GraphedStep(model, example_ids)
         loss = step(ids)            # gradients are in p.grad of the model's parameters afterwards
@@ -59,7 +59,9 @@ class GraphedStep:
     Create it before the model's first normally launched training step (a `Transformer` that has been stepped is refused:
     recording one ended the process here); replays and launched steps may be mixed freely afterwards."""
 
-    def __init__(self, model: nn.Module, example_ids: torch.Tensor, warmup: int = 3):
+    def __init__(self, model: nn.Module, example_ids: torch.Tensor, warmup: int = 3, loss_fn=None):
+        # loss_fn(model, ids) -> scalar loss; default: the Transformer's own `model(ids, return_loss=True)`
+        self.loss_fn = loss_fn if loss_fn is not None else (lambda m, ids: m(ids, return_loss=True))
         if not example_ids.is_cuda:
             raise RuntimeError("GraphedStep needs device tensors")
         if torch.is_autocast_enabled() or any(p.requires_grad and p.is_floating_point() and p.dtype != torch.bfloat16 for p in model.parameters()):
@@ -84,14 +86,14 @@ class GraphedStep:
         try:
             with torch.cuda.stream(side):                # allocator and library warm-up outside the recording
                 for _ in range(max(1, warmup)):
-                    torch.autograd.grad(model(self.ids, return_loss=True), wanted, allow_unused=True)
+                    torch.autograd.grad(self.loss_fn(model, self.ids), wanted, allow_unused=True)
         finally:
             model._recording_warmup = False
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
-            loss = model(self.ids, return_loss=True)
+            loss = self.loss_fn(model, self.ids)
             grads = torch.autograd.grad(loss, wanted, allow_unused=True)
             self.loss = loss.detach()
         by_param = dict(zip(map(id, wanted), grads))

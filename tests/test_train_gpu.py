@@ -172,3 +172,34 @@ def test_graphed_step_refuses_fp32_parameters():
     model = _small_model()                                # fp32 parameters: would train under autocast
     with pytest.raises(RuntimeError, match="bf16 model"):
         GraphedStep(model, torch.randint(0, 256, (2, 257), device=DEV))
+
+
+def test_graphed_step_of_a_bare_attention_module():
+    """GraphedStep with a loss function of its own: one SparseAttention layer, float inputs instead of token ids."""
+    from native_sparse_attention_pytorch_amd import SparseAttention
+    from native_sparse_attention_pytorch_amd.training import GraphedStep
+    torch.manual_seed(9)
+    attn = SparseAttention(dim=256, dim_head=64, heads=4, kv_heads=2, sliding_window_size=32, compress_block_size=16,
+                           compress_block_sliding_stride=8, selection_block_size=16, num_selected_blocks=4).to(DEV).bfloat16()
+    w = torch.randn(2, 384, 256, device=DEV, dtype=torch.bfloat16)
+    loss_fn = lambda m, x: (m(x).float() * w.float()).mean()
+    xs = [torch.randn(2, 384, 256, device=DEV, dtype=torch.bfloat16, generator=torch.Generator(device=DEV).manual_seed(i)) for i in range(4)]
+    step = GraphedStep(attn, xs[0], loss_fn=loss_fn)
+    params = list(attn.parameters())
+    names = [n for n, _ in attn.named_parameters()]
+    for rep, x in enumerate(xs):
+        for p in params:
+            p.grad = None
+        want_loss = loss_fn(attn, x)
+        want_loss.backward()
+        want = [None if p.grad is None else p.grad.clone() for p in params]
+        torch.cuda.synchronize()
+        loss = step(x)
+        torch.cuda.synchronize()
+        assert abs(loss.item() - want_loss.item()) <= 1e-6 * max(1.0, abs(want_loss.item())), (rep, loss.item(), want_loss.item())
+        for n, p, wg in zip(names, params, want):
+            assert (p.grad is None) == (wg is None), n
+            if wg is not None:
+                err = (p.grad.float() - wg.float()).abs().max().item()
+                tol = 1e-2 * max(wg.float().abs().max().item(), 1e-6) if n.endswith("bias") else 0.0
+                assert torch.isfinite(p.grad).all() and err <= tol, f"replay {rep}: gradient of {n} differs by {err}"
