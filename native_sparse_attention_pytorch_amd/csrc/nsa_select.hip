@@ -587,6 +587,15 @@ __device__ __forceinline__ unsigned long long live_slots(const SelPlan& P, const
 // at most half a wave (d = 64 with G <= 4) and the slots fit 32 mask bits, two queries share a wave instead of idling half of it.
 __host__ __device__ __forceinline__ bool merge_two_per_wave(const SelPlan& P, int cpr) { return P.g * cpr <= 32 && P.SP <= 32; }
 
+// slots whose loads a merge round issues together (measured at seq 32k, d 128, 16 slots: forward merge 0.819 / 0.825 / 0.790 /
+// 0.815 ms for 1 / 2 / 4 / 8, dQ merge 0.757 / 0.783 / 0.794 / 0.801 ms: the merges stream at what the memory gives
+// non-temporal reads, about 6 TB/s, and more rows in flight per wave only help the one that also has exponentials to hide)
+#ifndef NSA_MERGE_BATCH
+#define NSA_MERGE_BATCH 4
+#endif
+#ifndef NSA_MERGE_BATCH_BWD
+#define NSA_MERGE_BATCH_BWD 1
+#endif
 // merge the per-slot partials of one query: out = sum_s exp(lse_s - LSE) * o_s
 template <int D>
 __global__ __launch_bounds__(256) void sel_fwd_combine_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, const char* __restrict__ fws,
@@ -609,17 +618,35 @@ __global__ __launch_bounds__(256) void sel_fwd_combine_kernel(const SelPlan P, c
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    for (unsigned long long m = live; m; m &= m - 1) {
-      const int s = __builtin_ctzll(m);
-      const size_t row = row0 + (size_t)s * P.g;
-      const float ls = __builtin_nontemporal_load(lsepart + row);
-      const bf16x8 o = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(opart + row * D + dd));
-      const float mn = fmaxf(mx, ls);
-      const float a = __expf(mx - mn), w = __expf(ls - mn);      // first slot: mx = -inf -> a = 0
-      sum = sum * a + w;
+    // NSA_MERGE_BATCH slots per round, their loads issued together: one row in flight per wave leaves the memory system
+    // waiting for the waves (a round is then one memory latency long).  A round's spare entries repeat its last live slot
+    // with weight zero.
+    for (unsigned long long m = live; m;) {
+      size_t row[NSA_MERGE_BATCH];
+      bool ok[NSA_MERGE_BATCH];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = acc[e] * a + w * (float)o[e];
-      mx = mn;
+      for (int j = 0; j < NSA_MERGE_BATCH; ++j) {
+        ok[j] = m != 0;
+        if (ok[j]) { row[j] = row0 + (size_t)__builtin_ctzll(m) * P.g; m &= m - 1; }
+        else row[j] = row[j > 0 ? j - 1 : 0];
+      }
+      float ls[NSA_MERGE_BATCH];
+      bf16x8 o[NSA_MERGE_BATCH];
+#pragma unroll
+      for (int j = 0; j < NSA_MERGE_BATCH; ++j) {
+        ls[j] = __builtin_nontemporal_load(lsepart + row[j]);
+        o[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(opart + row[j] * D + dd));
+      }
+#pragma unroll
+      for (int j = 0; j < NSA_MERGE_BATCH; ++j) {
+        const float lj = ok[j] ? ls[j] : -INFINITY;
+        const float mn = fmaxf(mx, lj);
+        const float a = __expf(mx - mn), w = __expf(lj - mn);      // first slot: mx = -inf -> a = 0; spare entry: w = 0
+        sum = sum * a + w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = acc[e] * a + w * (float)o[j][e];
+        mx = mn;
+      }
     }
     const float L = live ? mx + __logf(sum) : -INFINITY;
     const float inv = live ? 1.0f / sum : 0.f;
@@ -818,11 +845,23 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    for (unsigned long long m = live; m; m &= m - 1) {
-      const int s = __builtin_ctzll(m);
-      const bf16x8 o = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(dqpart + (row0 + (size_t)s * P.g) * D + dd));
+    // (NSA_MERGE_BATCH_BWD rows in flight per round, see the forward merge)
+    for (unsigned long long m = live; m;) {
+      size_t row[NSA_MERGE_BATCH_BWD];
+      bool ok[NSA_MERGE_BATCH_BWD];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += (float)o[e];
+      for (int j = 0; j < NSA_MERGE_BATCH_BWD; ++j) {
+        ok[j] = m != 0;
+        if (ok[j]) { row[j] = row0 + (size_t)__builtin_ctzll(m) * P.g; m &= m - 1; }
+        else row[j] = row[j > 0 ? j - 1 : 0];
+      }
+      bf16x8 o[NSA_MERGE_BATCH_BWD];
+#pragma unroll
+      for (int j = 0; j < NSA_MERGE_BATCH_BWD; ++j) o[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(dqpart + row[j] * D + dd));
+#pragma unroll
+      for (int j = 0; j < NSA_MERGE_BATCH_BWD; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += ok[j] ? (float)o[j][e] : 0.f;
     }
     bf16x8 r;
 #pragma unroll
