@@ -890,8 +890,15 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 #ifndef NSA_BWD_STAGES_D64
 #define NSA_BWD_STAGES_D64 1
 #endif
+// waves per SIMD the d = 64 walk is compiled for: two (256 registers) ...
 #ifndef NSA_BWD_D64_WAVES
 #define NSA_BWD_D64_WAVES 2
+#endif
+// ... but only with two waves per work-group (64-key blocks).  Blocks of up to 32 keys are walked by one wave that gathers
+// both tiles and holds every dQ feature tile: in 256 registers it spills, and the reloads inside the loop wait behind the
+// gathers in flight (seq 16k, 32-key blocks: backward 0.515 ms with two waves per SIMD, 0.405 with one and no spills).
+#ifndef NSA_BWD_D64_WAVES_MIN_KT
+#define NSA_BWD_D64_WAVES_MIN_KT 2
 #endif
 #ifndef NSA_BWD_AHEAD_D64
 #define NSA_BWD_AHEAD_D64 3
@@ -903,7 +910,7 @@ __global__ __launch_bounds__(256) void sel_bwd_dq_combine_kernel(const SelPlan P
 #define NSA_BWD_STAGES 2      // measured on MI355X (seq 32k, d 128): 1, 2 and 3 stages all 2.68-2.70 ms once the LDS operand reads run ahead
 #endif
 template <int D, int KT, bool FUSE_DQ>
-__global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64 ? NSA_BWD_D64_WAVES : 1))) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
+__global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64 && KT >= NSA_BWD_D64_WAVES_MIN_KT ? NSA_BWD_D64_WAVES : 1))) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                               const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
                                                               const float* __restrict__ lse, const float* __restrict__ delta,
                                                               const char* __restrict__ iws, char* __restrict__ bws) {
@@ -932,8 +939,9 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
 
   // the first list entries, then the block's K / V rows: all requested before anything waits
   const int ppt = 32 >> P.lg;
-  // a single wave gathers both tiles: no registers for a second stage; at d = 64 the kernel runs two waves per SIMD in 256
-  // registers, where a second stage only adds spills (measured at b4 n4096: 375 us with one stage, 460 us with two)
+  // a single wave gathers both tiles: one stage (a second measured no faster where the registers allow it, d = 64 at one wave
+  // per SIMD); two waves at d = 64 run two to a SIMD in 256 registers, where a second stage only adds spills (measured at
+  // b4 n4096: 375 us with one stage, 460 us with two)
   constexpr int NS = KT == 1 ? 1 : (D == 64 ? NSA_BWD_STAGES_D64 : NSA_BWD_STAGES);
   RawEntry e0[NS];
 #pragma unroll
