@@ -1490,8 +1490,10 @@ def _wgrad_splits(rows: int, n_in: int, n_out: int) -> int:
     """How many slices of the token axis the weight gradient 'o i' = dy^T x is cut into.  The library's GEMM gives one work-group
     per output tile the whole token axis: with a few dozen tiles of a small weight and tens of thousands of tokens most of the
     256 CUs idle (measured on 16384 tokens: 1024 x 1024 weight 109 us whole, 52 us in 8 slices + the sum; 48 x 1024 99 -> 31 us;
-    a 2048 x 2048 weight over 4080 tokens has its 256 tiles already and is left whole)."""
-    if rows < 16384:          # the whole GEMM is a few microseconds: a second launch (the sum of the slices) costs more than the slices save
+    on 8192 tokens every weight from 24 x 512 to 2048 x 512 takes 47-57 us whole - the time follows the token count, not the
+    weight - and 30-35 us in 4 or 8 slices, launches included; a 2048 x 2048 weight over 4080 tokens has its 256 tiles already and
+    is left whole, and at 4096 tokens the whole GEMM's 27-31 us are what the two launches of the sliced one cost)."""
+    if rows < 8192:
         return 1
     tiles = -(-n_in // 128) * -(-n_out // 128)
     s = 8

