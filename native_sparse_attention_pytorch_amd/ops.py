@@ -1486,17 +1486,19 @@ def rms_norm(x: Tensor, weight: Tensor, eps: float | None = None) -> Tensor:
 
 # ------------------------------------------------------------------ projections
 
-def _wgrad_splits(rows: int, n_in: int, n_out: int) -> int:
+def _wgrad_splits(rows: int, n_in: int, n_out: int, replayed: bool = False) -> int:
     """How many slices of the token axis the weight gradient 'o i' = dy^T x is cut into.  The library's GEMM gives one work-group
     per output tile the whole token axis: with a few dozen tiles of a small weight and tens of thousands of tokens most of the
     256 CUs idle (measured on 16384 tokens: 1024 x 1024 weight 109 us whole, 52 us in 8 slices + the sum; 48 x 1024 99 -> 31 us;
     on 8192 tokens every weight from 24 x 512 to 2048 x 512 takes 47-57 us whole - the time follows the token count, not the
     weight - and 30-35 us in 4 or 8 slices, launches included; a 2048 x 2048 weight over 4080 tokens has its 256 tiles already and
-    is left whole, and at 4096 tokens the whole GEMM's 27-31 us are what the two launches of the sliced one cost)."""
-    if rows < 8192:
+    is left whole, and at 4096 tokens the whole GEMM's 27-31 us are what the two launches of the sliced one cost).
+    `replayed`: the launches are being recorded into a graph, where they cost nothing at replay; then 4096 tokens are cut as
+    well (GPU time alone: 64 x 1024 weight 27 -> 10 us in 4 slices, 1024 x 1024 30 -> 23 us) and 16 slices are allowed."""
+    if rows < (4096 if replayed else 8192):
         return 1
     tiles = -(-n_in // 128) * -(-n_out // 128)
-    s = 8
+    s = 16 if replayed else 8
     while s > 1 and (s * tiles > 768 or rows % s or rows // s < 1024):
         s //= 2
     return s if s >= 4 else 1
@@ -1538,7 +1540,7 @@ def linear(x: Tensor, weight: Tensor, bias: Tensor | None = None) -> Tensor:
 def _wgrad(dy2: Tensor, x2: Tensor, dtype) -> Tensor:
     """Weight gradient 'o i' = dy2^T x2 of a projection, over slices of the token axis where that fills the chip."""
     rows, n_in, n_out = x2.shape[0], x2.shape[1], dy2.shape[1]
-    s = _wgrad_splits(rows, n_in, n_out) if x2.is_cuda and x2.dtype in (_BF16, torch.float16) and dy2.dtype == x2.dtype else 1
+    s = _wgrad_splits(rows, n_in, n_out, capturing()) if x2.is_cuda and x2.dtype in (_BF16, torch.float16) and dy2.dtype == x2.dtype else 1
     if s > 1 and dy2.is_contiguous() and x2.is_contiguous():
         try:
             part = torch.bmm(dy2.view(s, rows // s, n_out).transpose(1, 2), x2.view(s, rows // s, n_in), out_dtype=torch.float32)

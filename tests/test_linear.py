@@ -17,6 +17,9 @@ def test_slices_by_shape():
     assert ops._wgrad_splits(32768, 1024, 1024) == 8
     assert ops._wgrad_splits(8192, 512, 512) == 8          # a config-5 step: 8 x 1024 tokens
     assert ops._wgrad_splits(8192, 512, 2048) == 8
+    assert ops._wgrad_splits(4096, 1024, 64, replayed=True) == 4      # recorded into a graph: launches are free at replay
+    assert ops._wgrad_splits(16384, 512, 512, replayed=True) == 16
+    assert ops._wgrad_splits(2048, 1024, 64, replayed=True) == 1
     assert ops._wgrad_splits(16383, 1024, 1024) == 1       # no even cut
     assert ops._wgrad_splits(2048, 64, 64) == 1
 
