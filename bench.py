@@ -141,7 +141,7 @@ def graphed_train_leg():
                                                 selection_block_size=16, num_selected_blocks=4)).to(dev)
     ids = torch.randint(0, 256, (8, 1025), device=dev)
     mw = Fp32Masters(model)
-    opt = torch.optim.Adam(mw.masters, lr=1e-4)
+    opt = torch.optim.Adam(mw.masters, lr=1e-4, fused=True)       # (one kernel per parameter list instead of one per operation)
     gstep = GraphedStep(model, ids)
 
     def step():
@@ -474,7 +474,7 @@ def main():
                             sparse_attn_kwargs=dict(sliding_window_size=64, compress_block_size=16, compress_block_sliding_stride=8,
                                                     selection_block_size=16, num_selected_blocks=4)).to(dev)
         mw = Fp32Masters(model)
-        opt = torch.optim.Adam(mw.masters, lr=1e-4)
+        opt = torch.optim.Adam(mw.masters, lr=1e-4, fused=True)       # (one kernel per parameter list instead of one per operation)
 
         def master_step():
             loss = model(ids, return_loss=True)
