@@ -33,25 +33,37 @@ __device__ __forceinline__ int read_idx(const void* idx, int is64, size_t pos) {
   return reinterpret_cast<const int*>(idx)[pos];
 }
 
-// cnt[bh][chunk][j] = number of live slots of the chunk's queries that name block j
+// cnt[bh][chunk][j] = number of live slots of the chunk's queries that name block j.  Consecutive lanes take consecutive
+// entries of the chunk's [query][slot] run (coalesced), sixteen rounds' loads in flight before the first is used: with up
+// to 16 slots per query the whole chunk is one memory round trip.
 __global__ __launch_bounds__(256) void sel_count_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, char* iws) {
   extern __shared__ int hist[];
   const int c = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
-  for (int j = tid; j < P.W; j += 256) hist[j] = 0;
-  __syncthreads();
-  const int i = c * kCountChunk + tid;
-  if (i < P.n) {
-    const size_t base = ((size_t)bh * P.n + i) * P.S;
-    for (int s = 0; s < P.S; ++s) {
-      if (fmask[base + s]) {
-        const int j = read_idx(idx, P.idx64, base + s);
-        if (j >= 0 && j < P.W) atomicAdd(&hist[j], 1);     // integer LDS counter: order-independent
-      }
+  const int q0 = c * kCountChunk;
+  const int total = min(kCountChunk, P.n - q0) * P.S;
+  const size_t base = ((size_t)bh * P.n + q0) * P.S;
+  constexpr int RK = 16;
+  int live[RK], j[RK];
+  auto load = [&](int e0) {
+#pragma unroll
+    for (int r = 0; r < RK; ++r) {
+      const int e = e0 + r * 256 + tid, ec = max(0, min(e, total - 1));
+      live[r] = e < total ? fmask[base + ec] : 0;
+      j[r] = e < total ? read_idx(idx, P.idx64, base + ec) : -1;
     }
+  };
+  if (total > 0) load(0);
+  for (int jj = tid; jj < P.W; jj += 256) hist[jj] = 0;
+  __syncthreads();
+  for (int e0 = 0; e0 < total; e0 += RK * 256) {
+    if (e0 > 0) load(e0);
+#pragma unroll
+    for (int r = 0; r < RK; ++r)
+      if (live[r] && j[r] >= 0 && j[r] < P.W) atomicAdd(&hist[j[r]], 1);     // integer LDS counter: order-independent
   }
   __syncthreads();
   int* cnt = reinterpret_cast<int*>(iws + P.off_cnt) + ((size_t)bh * P.nch + c) * P.W;
-  for (int j = tid; j < P.W; j += 256) cnt[j] = hist[j];
+  for (int jj = tid; jj < P.W; jj += 256) cnt[jj] = hist[jj];
 }
 
 // exclusive scan over the counting chunks of every block (in place in cnt) and over blocks
@@ -117,43 +129,64 @@ __device__ __forceinline__ CellInfo cell_info(const SelPlan& P, const char* iws,
 }
 
 // unit_off[t][bh][cell] = exclusive prefix sum of ceil(pairs(cell) / chunk[t]), cells phase-major
-__global__ __launch_bounds__(256) void sel_units_kernel(const SelPlan P, char* iws) {
-  __shared__ int part[256];
+__global__ __launch_bounds__(1024) void sel_units_kernel(const SelPlan P, char* iws) {
+  __shared__ int wave_tot[16];
   __shared__ int total_s;
-  const int bh = blockIdx.x, t = blockIdx.y, tid = threadIdx.x;
+  const int bh = blockIdx.x, t = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int cells = P.np[t] * P.W;
   int* uo = reinterpret_cast<int*>(iws + P.off_unit[t]) + (size_t)bh * (cells + 1);
-  const int per = (cells + 255) / 256;
+  const int per = (cells + 1023) / 1024;
   const int lo = min(cells, tid * per), hi = min(cells, lo + per);
-  // (phase, block) of a cell are carried along instead of divided out: this kernel has few waves and
-  // is bound by its integer arithmetic; chunk[] is a power of two
+  // (phase, block) of a cell are carried along instead of divided out; chunk[] is a power of two.  The kernel is a handful
+  // of waves and a chain of dependent loads: the cell records of a thread's first cells are kept for the second pass
+  // instead of fetched again.
   const int csh = 31 - __clz(P.chunk[t]);
+  constexpr int KEEP = 8;
+  CellInfo kept[KEEP];
   int sum = 0;
   {
     int pp = lo / P.W, j = lo % P.W;
-    for (int c = lo; c < hi; ++c) {
+#pragma unroll
+    for (int u = 0; u < KEEP; ++u) {
+      kept[u] = CellInfo{0, 0, 0};
+      if (lo + u < hi) {
+        kept[u] = cell_info(P, iws, bh, t, pp, j);
+        sum += (kept[u].own + kept[u].count + P.chunk[t] - 1) >> csh;
+        if (++j == P.W) { j = 0; ++pp; }
+      }
+    }
+    for (int c = lo + KEEP; c < hi; ++c) {
       const CellInfo ci = cell_info(P, iws, bh, t, pp, j);
       sum += (ci.own + ci.count + P.chunk[t] - 1) >> csh;
       if (++j == P.W) { j = 0; ++pp; }
     }
   }
-  part[tid] = sum;
+  // exclusive scan of the threads' sums over the work-group: inside a wave by shuffles, then the 16 wave totals
+  int incl = sum;
+  for (int dlt = 1; dlt < 64; dlt <<= 1) {
+    const int y = __shfl_up(incl, dlt, 64);
+    if (lane >= dlt) incl += y;
+  }
+  if (lane == 63) wave_tot[wave] = incl;
   __syncthreads();
-  if (tid == 0) {
-    int acc = 0;
-    for (int k = 0; k < 256; ++k) { const int v = part[k]; part[k] = acc; acc += v; }
-    uo[cells] = acc;
-    total_s = acc;
+  if (wave == 0) {
+    const int tw = lane < 16 ? wave_tot[lane] : 0;
+    int xs = tw;
+    for (int dlt = 1; dlt < 16; dlt <<= 1) {
+      const int y = __shfl_up(xs, dlt, 64);
+      if (lane >= dlt) xs += y;
+    }
+    if (lane < 16) wave_tot[lane] = xs - tw;
+    if (lane == 15) { total_s = xs; uo[cells] = xs; }
   }
   __syncthreads();
   // besides the prefix sums, one record per unit: a walk's work-group then finds its unit with one
   // load instead of a binary search over the prefix sums (a dozen dependent loads at one wave per SIMD)
   int4* rec = reinterpret_cast<int4*>(iws + P.off_urec[t]) + (size_t)bh * P.ub[t] * 2;
-  int acc = part[tid];
+  int acc = incl - sum + wave_tot[wave];
   {
     int pp = lo / P.W, j = lo % P.W;
-    for (int c = lo; c < hi; ++c) {
-      const CellInfo ci = cell_info(P, iws, bh, t, pp, j);
+    auto emit = [&](int c, const CellInfo& ci) {
       uo[c] = acc;
       const int L = ci.own + ci.count, nu = (L + P.chunk[t] - 1) >> csh;
       for (int k = 0; k < nu; ++k) {
@@ -162,51 +195,83 @@ __global__ __launch_bounds__(256) void sel_units_kernel(const SelPlan P, char* i
       }
       acc += nu;
       if (++j == P.W) { j = 0; ++pp; }
-    }
+    };
+#pragma unroll
+    for (int u = 0; u < KEEP; ++u)
+      if (lo + u < hi) emit(lo + u, kept[u]);
+    for (int c = lo + KEEP; c < hi; ++c) emit(c, cell_info(P, iws, bh, t, pp, j));
   }
-  for (int u = total_s + tid; u < P.ub[t]; u += 256) {       // padding units: empty range
+  for (int u = total_s + tid; u < P.ub[t]; u += 1024) {       // padding units: empty range
     rec[2 * u] = int4{0, 0, 0, 0};
     rec[2 * u + 1] = int4{0, 0, 0, 0};
   }
 }
 
-// list[bh][blk_off[j] + ...] = query * SP + slot, ordered by (block, counting chunk, query, slot)
-__global__ __launch_bounds__(64) void sel_fill_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, char* iws) {
-  extern __shared__ int base[];
-  const int c = blockIdx.x, bh = blockIdx.y, lane = threadIdx.x;
+// NW waves per work-group, each with a quarter (NW = 4) of the chunk's queries: a wave's entries are ranked 64 at a time, one
+// dependent round per 64 entries, so the rounds of a chunk run four abreast.  The waves' starting positions inside a block's
+// run of the chunk come from a count of each wave's entries first (integer LDS counters again); the lists are the same as
+// one wave walking the whole chunk would write.  NW = 1 where 5 W counters do not fit the 64 KB of LDS a launch may ask for.
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void sel_fill_kernel(const SelPlan P, const void* idx, const uint8_t* fmask, char* iws) {
+  extern __shared__ int base_all[];              // [NW][W]: where wave w's next entry of block j goes
+  const int c = blockIdx.x, bh = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int* cnt = reinterpret_cast<const int*>(iws + P.off_cnt) + ((size_t)bh * P.nch + c) * P.W;
   const int* blk = reinterpret_cast<const int*>(iws + P.off_blk) + (size_t)bh * (P.W + 1);
   int* list = reinterpret_cast<int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
-  for (int j = lane; j < P.W; j += 64) base[j] = blk[j] + cnt[j];
-  __syncthreads();
-  const int q0 = c * kCountChunk;
-  const int nq = min(kCountChunk, P.n - q0);
+  int* base = base_all + w * P.W;
+  const int q0c = c * kCountChunk;
+  const int nqc = min(kCountChunk, P.n - q0c);
+  constexpr int QW = kCountChunk / NW;           // queries per wave
+  const int q0 = q0c + w * QW;
+  const int nq = max(0, min(QW, q0c + nqc - q0));
   const int total = nq * P.S;
-  if (total <= 0) return;
-  // the slot mask and block index of an entry are fetched two rounds ahead of their use (branch-free, from a clamped
-  // position): a round is otherwise one dependent global load long
-  struct Fetched { int live, j; };
-  auto fetch = [&](int e0) {
-    const int e = min(e0 + lane, total - 1);
-    const size_t pos = ((size_t)bh * P.n + q0) * P.S + e;
-    Fetched f;
-    f.live = fmask[pos];
-    f.j = read_idx(idx, P.idx64, pos);
-    return f;
-  };
-  Fetched f0 = fetch(0), f1 = fetch(64);
-  const int nbits = 32 - __builtin_clz((unsigned)max(P.W - 1, 1));      // bits of a block index
-  for (int e0 = 0; e0 < total; e0 += 64) {
-    const Fetched cur = f0;
-    f0 = f1;
-    f1 = fetch(e0 + 128);
-    const int e = e0 + lane;
-    int j = -1, entry = 0;
-    if (e < total && cur.live) {
-      j = cur.j;
-      if (j >= P.W) j = -1;
-      entry = (q0 + e / P.S) * P.SP + e % P.S;
+  const size_t pos0 = ((size_t)bh * P.n + q0) * P.S;
+  // The wave's first RK rounds of entries (all of them with up to 16 slots per query and four waves) are fetched at once and
+  // stay in registers: one memory round trip for the count and the ranking together, instead of one per round.
+  constexpr int RK = 16;
+  int live[RK], jv[RK];
+#pragma unroll
+  for (int r = 0; r < RK; ++r) {
+    const int e = r * 64 + lane, ec = max(0, min(e, total - 1));
+    live[r] = e < total ? fmask[pos0 + ec] : 0;
+    jv[r] = e < total ? read_idx(idx, P.idx64, pos0 + ec) : -1;
+    if (jv[r] >= P.W) jv[r] = -1;
+  }
+  if (NW > 1) {
+    for (int j = threadIdx.x; j < NW * P.W; j += 64 * NW) base_all[j] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < RK; ++r)
+      if (live[r] && jv[r] >= 0) atomicAdd(&base[jv[r]], 1);
+    for (int e0 = RK * 64; e0 < total; e0 += 64) {
+      const int e = e0 + lane;
+      if (e < total && fmask[pos0 + e]) {
+        const int j = read_idx(idx, P.idx64, pos0 + e);
+        if (j >= 0 && j < P.W) atomicAdd(&base[j], 1);
+      }
     }
+    __syncthreads();
+    // counts -> starting positions: the block's run, the chunk's offset in it, the waves before this one
+    for (int j = threadIdx.x; j < P.W; j += 64 * NW) {
+      int run = blk[j] + cnt[j];
+#pragma unroll
+      for (int w2 = 0; w2 < NW; ++w2) { const int v = base_all[w2 * P.W + j]; base_all[w2 * P.W + j] = run; run += v; }
+    }
+    __syncthreads();
+  } else {
+    for (int j = lane; j < P.W; j += 64) base[j] = blk[j] + cnt[j];
+    __syncthreads();
+  }
+  if (total <= 0) return;
+  // (from here on a wave is on its own - the waves of a partial chunk have different numbers of rounds - and touches only its
+  // own row of counters.  A wave's LDS operations execute in the order they were issued, so all that has to be kept is the
+  // compiler's order of them; a fence would also wait for the list stores in flight, one memory round trip per round.)
+  auto wave_sync = [] { asm volatile("" ::: "memory"); };
+  const int nbits = 32 - __builtin_clz((unsigned)max(P.W - 1, 1));      // bits of a block index
+  // one round: the 64 entries e0 + lane; j = the lane's block (-1: no entry, dead slot or block out of range)
+  auto round = [&](int e0, int j) {
+    const int e = e0 + lane;
+    const int entry = (q0 + e / P.S) * P.SP + e % P.S;
     // lanes of this pass that name the same block: intersect, bit by bit of the block index, the ballots of the lanes
     // that agree with this lane (about 10 ballots instead of 64 lane reads); dead lanes are masked out
     unsigned long long same_m = __ballot(j >= 0);
@@ -218,9 +283,33 @@ __global__ __launch_bounds__(64) void sel_fill_kernel(const SelPlan P, const voi
     const int rank = __popcll(same_m & ((1ull << lane) - 1ull));
     const int same = __popcll(same_m);
     if (j >= 0) list[base[j] + rank] = entry;
-    __syncthreads();
+    wave_sync();
     if (j >= 0 && rank == same - 1) base[j] += same;
-    __syncthreads();
+    wave_sync();
+  };
+#pragma unroll
+  for (int r = 0; r < RK; ++r)
+    if (r * 64 < total) round(r * 64, live[r] ? jv[r] : -1);
+  // what does not fit the registers (more than 16 slots per query, or one wave for the whole chunk): fetched two rounds
+  // ahead of their use (branch-free, from a clamped position) - a round is otherwise one dependent global load long
+  if (total > RK * 64) {
+    struct Fetched { int live, j; };
+    auto fetch = [&](int e0) {
+      const int e = min(e0 + lane, total - 1);
+      Fetched f;
+      f.live = fmask[pos0 + e];
+      f.j = read_idx(idx, P.idx64, pos0 + e);
+      return f;
+    };
+    Fetched f0 = fetch(RK * 64), f1 = fetch(RK * 64 + 64);
+    for (int e0 = RK * 64; e0 < total; e0 += 64) {
+      const Fetched cur = f0;
+      f0 = f1;
+      f1 = fetch(e0 + 128);
+      int j = -1;
+      if (e0 + lane < total && cur.live) j = cur.j >= P.W ? -1 : cur.j;
+      round(e0, j);
+    }
   }
 }
 
@@ -1237,9 +1326,12 @@ extern "C" int nsa_select_build_index(const nsa_select_desc* d, const void* idx,
   NSA_LAUNCH_CHECK();
   hipLaunchKernelGGL(sel_scan_kernel, dim3(P.bh), dim3(256), lds, st, P, iws);
   NSA_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sel_units_kernel, dim3(P.bh, 3), dim3(256), 0, st, P, iws);
+  hipLaunchKernelGGL(sel_units_kernel, dim3(P.bh, 3), dim3(1024), 0, st, P, iws);
   NSA_LAUNCH_CHECK();
-  hipLaunchKernelGGL(sel_fill_kernel, dim3(P.nch, P.bh), dim3(64), lds, st, P, idx, fmask, iws);
+  if (4 * lds <= 65536)
+    hipLaunchKernelGGL(sel_fill_kernel<4>, dim3(P.nch, P.bh), dim3(256), 4 * lds, st, P, idx, fmask, iws);
+  else
+    hipLaunchKernelGGL(sel_fill_kernel<1>, dim3(P.nch, P.bh), dim3(64), lds, st, P, idx, fmask, iws);
   NSA_LAUNCH_CHECK();
   return 0;
 }
