@@ -332,6 +332,12 @@ __device__ __forceinline__ bool locate_unit(const SelPlan& P, const char* iws, i
   return ui.v0 < ui.v1;
 }
 
+// the dK/dV walk's table has one phase: unit_off[bh][j] .. unit_off[bh][j + 1] are block j's units
+__device__ __forceinline__ bool block_has_one_unit(const SelPlan& P, const char* iws, int bh, int j) {
+  const int* unit_off = reinterpret_cast<const int*>(iws + P.off_unit[2]) + (size_t)bh * (P.W + 1);
+  return unit_off[j + 1] - unit_off[j] == 1;
+}
+
 // Work-group id -> (batch*kv head, unit) such that all units of one head run, in table order,
 // on as few XCDs as possible (consecutive work-group ids go round-robin over the 8 XCDs), so
 // that the Q rows of a query phase are fetched into one L2 only.
@@ -1002,7 +1008,8 @@ template <int D, int KT, bool FUSE_DQ>
 __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64 && KT >= NSA_BWD_D64_WAVES_MIN_KT ? NSA_BWD_D64_WAVES : 1))) void sel_bwd_dkv_kernel(const SelPlan P, const __bf16* __restrict__ q, const __bf16* __restrict__ k,
                                                               const __bf16* __restrict__ v, const __bf16* __restrict__ dout,
                                                               const float* __restrict__ lse, const float* __restrict__ delta,
-                                                              const char* __restrict__ iws, char* __restrict__ bws) {
+                                                              const char* __restrict__ iws, char* __restrict__ bws,
+                                                              __bf16* __restrict__ dk, __bf16* __restrict__ dv) {
   constexpr int KS = D / 16, DT = D / 32, RS = D + 8;
   constexpr int RST = 32 + 16;                 // row stride of the [key][row] dS tile (transpose loads only: 8 banks mod 32 per row)
   constexpr int RSK = D + 16;                  // row stride of the K block copy (transpose loads only)
@@ -1024,6 +1031,7 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
   UnitInfo ui;
   if (!locate_unit(P, iws, 2, bh, u, ui)) return;
   const int* list = reinterpret_cast<const int*>(iws + P.off_list) + (size_t)bh * P.list_cap;
+  const bool single_unit = dk != nullptr && block_has_one_unit(P, iws, bh, ui.j);
   const bool load_q = kt == 0;                 // with two waves: wave 0 gathers Q rows, wave 1 dO rows; one wave does both
 
   // the first list entries, then the block's K / V rows: all requested before anything waits
@@ -1238,6 +1246,24 @@ __global__ __launch_bounds__(64 * KT) __attribute__((amdgpu_waves_per_eu(D == 64
   for (int s2 = 0; s2 < NS - 1; ++s2)
     if (vt + s2 * ppt < ui.v1) step(vt + s2 * ppt, stg[s2]);
 
+  // A block all of whose pairs fit this one unit (most blocks: the later a block lies the fewer queries can select it) has
+  // nothing to be summed with: its dK / dV leave as bf16 straight away - what the reduce kernel would make of a single
+  // partial, bit for bit - instead of 2 x 32 KT x D floats written here and read back there.
+  if (single_unit) {
+    const int keys = min(P.B, P.n - ui.j * P.B);
+    if (kl < keys) {
+      __bf16* ok_ = dk + (((size_t)bh * P.n) + (size_t)ui.j * P.B + kl) * D + 4 * h;
+      __bf16* ov_ = dv + (((size_t)bh * P.n) + (size_t)ui.j * P.B + kl) * D + 4 * h;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          store4_bf16(ok_ + 32 * dt + 8 * a, dKa[dt][4 * a] * P.scale, dKa[dt][4 * a + 1] * P.scale, dKa[dt][4 * a + 2] * P.scale, dKa[dt][4 * a + 3] * P.scale);
+          store4_bf16(ov_ + 32 * dt + 8 * a, dVa[dt][4 * a], dVa[dt][4 * a + 1], dVa[dt][4 * a + 2], dVa[dt][4 * a + 3]);
+        }
+    }
+    return;
+  }
   // partial [unit][2][32*KT keys][D] fp32; dKa/dVa hold [feature 32dt + 8a + 4h + bb][key kl]
   float* part = reinterpret_cast<float*>(bws + P.off_dkvpart) + ((size_t)bh * P.ub_kv + u) * (2 * 32 * KT * D);
   float* pk = part + (size_t)kl * D + 4 * h;
@@ -1261,6 +1287,7 @@ __global__ __launch_bounds__(256) void sel_bwd_dkv_reduce_kernel(const SelPlan P
   const int j = blockIdx.x, bh = blockIdx.y;
   const int* unit_off = reinterpret_cast<const int*>(iws + P.off_unit[2]) + (size_t)bh * (P.W + 1);
   const int u0 = unit_off[j], u1 = unit_off[j + 1];
+  if (u1 - u0 == 1) return;                       // written by the walk itself
   const float* part = reinterpret_cast<const float*>(bws + P.off_dkvpart) + (size_t)bh * P.ub_kv * (2 * 32 * KT * D);
   const int keys = min(P.B, P.n - j * P.B);
   // a unit's partial is 2 x ROWS x D floats in the order (dk | dv, key, feature): the work group reads
@@ -1394,10 +1421,10 @@ static int launch_bwd(const SelPlan& P, const void* q, const void* k, const void
   mark(ev, nev, 2, st);
   if (fused) {
     hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT, true>), dim3(P.ub_kv, P.bh), dim3(64 * KT), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
-                       (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
+                       (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws, (__bf16*)dk, (__bf16*)dv);
   } else {
     hipLaunchKernelGGL((sel_bwd_dkv_kernel<D, KT, false>), dim3(P.ub_kv, P.bh), dim3(64 * KT), 0, st, P, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v,
-                       (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws);
+                       (const __bf16*)dout, lse, delta, (const char*)iws, (char*)bws, (__bf16*)dk, (__bf16*)dv);
   }
   NSA_LAUNCH_CHECK();
   mark(ev, nev, 3, st);
