@@ -58,6 +58,12 @@ CASES = [
 ]
 
 
+def test_select_more_than_4096_blocks():
+    """4125 blocks per sequence: beyond 4096 the index build's list fill runs one wave per chunk of queries instead of four
+    (its per-wave position table no longer fits the shared memory a launch may ask for); same checks as the cases below."""
+    test_select_fwd_bwd_matches_oracle(1, 2, 1, 33000, 64, 8, 2)
+
+
 @pytest.mark.parametrize("b,hq,hk,n,d,B,S", CASES)
 def test_select_fwd_bwd_matches_oracle(b, hq, hk, n, d, B, S):
     from native_sparse_attention_pytorch_amd import native_sparse_attend
